@@ -1,0 +1,305 @@
+"""Writes the golden fixtures under tests/golden/ from the REAL reference.
+
+Run once, in the build container only (the reference checkout does not travel):
+
+    python tests/golden/make_fixtures.py [/root/reference]
+
+It imports `distributed_shampoo` from the reference checkout, runs it on CPU in
+fp32 on tiny seeded cases and stores inputs/outputs as .npz (data only, no
+pickles).  It is used only for what nothing else pins: the multi-step
+composition of `DistributedShampoo.step()`, the coupled-Newton trajectory
+(iteration counts, behaviour on rank-deficient input) and the QR-refresh column
+ordering.  Every case is described by plain hyper-parameters so that
+tests/test_oracle_golden.py can rebuild it for the oracle without the reference.
+"""
+
+from __future__ import annotations
+
+import json
+import os
+import sys
+from fractions import Fraction
+from unittest import mock
+
+import numpy as np
+import torch
+
+REF = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
+sys.path.insert(0, REF)
+
+from distributed_shampoo import (  # noqa: E402
+    AdaGradPreconditionerConfig,
+    AdamPreconditionerConfig,
+    CoupledNewtonConfig,
+    DefaultSOAPConfig,
+    DistributedShampoo,
+    EigenConfig,
+    EigenvalueCorrectedShampooPreconditionerConfig,
+    QREigendecompositionConfig,
+    RootInvShampooPreconditionerConfig,
+    WeightDecayType,
+)
+from distributed_shampoo.preconditioner.matrix_functions import (  # noqa: E402
+    matrix_eigendecomposition,
+    matrix_inverse_root,
+)
+from distributed_shampoo.shampoo_types import ClassicMomentumConfig  # noqa: E402
+
+OUT = os.path.dirname(os.path.abspath(__file__))
+
+
+def case_params(shapes, seed):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randn(*s, generator=g) for s in shapes]
+
+
+def case_grads(shapes, seed, step, scale):
+    g = torch.Generator().manual_seed(seed * 1000 + step)
+    return [scale * torch.randn(*s, generator=g) for s in shapes]
+
+
+# Plain-data descriptions; tests rebuild the oracle from the same dicts.
+CASES = {
+    "ragged_newton": dict(
+        shapes=[[48, 40], [40]], seed=1, grad_scale=1.0, steps=12,
+        lr=1e-2, betas=[0.9, 0.999], epsilon=1e-12, weight_decay=1e-2, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=32, precondition_frequency=2, start_preconditioning_step=6,
+        preconditioner="newton", override_1d=True, grafting="adam", grafting_beta2=0.999, grafting_epsilon=1e-8,
+    ),
+    "ragged_newton_1d": dict(  # 1-D blocks preconditioned, large epsilon keeps rank-1 factors well posed
+        shapes=[[20, 12], [12]], seed=2, grad_scale=1.0, steps=6,
+        lr=1e-2, betas=[0.9, 0.99], epsilon=1e-2, weight_decay=0.0, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=8, precondition_frequency=1, start_preconditioning_step=2,
+        preconditioner="newton", override_1d=False, grafting="adam", grafting_beta2=0.99, grafting_epsilon=1e-8,
+    ),
+    "momentum_l2_beta3": dict(
+        shapes=[[24, 36]], seed=3, grad_scale=0.1, steps=8,
+        lr=5e-3, betas=[0.8, 0.95], beta3=0.7, epsilon=1e-10, weight_decay=1e-3, weight_decay_type="L2",
+        max_preconditioner_dim=16, precondition_frequency=1, start_preconditioning_step=4,
+        preconditioner="newton", override_1d=True, grafting="adagrad", grafting_epsilon=1e-8,
+        momentum=0.5, dampening=0.1, use_nesterov=True,
+    ),
+    "eigh_rootinv": dict(
+        shapes=[[24, 20], [20]], seed=4, grad_scale=1.0, steps=6,
+        lr=1e-2, betas=[0.9, 1.0], epsilon=1e-12, weight_decay=0.0, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=16, precondition_frequency=3, start_preconditioning_step=3,
+        preconditioner="eigh", override_1d=False, grafting="adam", grafting_beta2=0.999, grafting_epsilon=1e-8,
+    ),
+    "soap_qr": dict(
+        shapes=[[24, 20], [20]], seed=5, grad_scale=1.0, steps=9,
+        lr=1e-2, betas=[0.9, 0.999], epsilon=1e-12, weight_decay=0.0, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=16, precondition_frequency=3, start_preconditioning_step=3,
+        preconditioner="soap_qr", override_1d=False, grafting=None,
+    ),
+    "cfg1_override": dict(  # BASELINE config 1 with 1-D blocks left to grafting
+        shapes=[[512, 512], [512]], seed=0, grad_scale=1.0, steps=10, zero_init=True, torch_seed_grads=True,
+        lr=1e-3, betas=[0.9, 0.999], epsilon=1e-12, weight_decay=0.0, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=512, precondition_frequency=1, start_preconditioning_step=1,
+        preconditioner="newton", override_1d=True, grafting="adam", grafting_beta2=0.999, grafting_epsilon=1e-8,
+    ),
+}
+
+
+def build_reference(c, params):
+    if c["preconditioner"] == "newton":
+        pc = RootInvShampooPreconditionerConfig(
+            amortized_computation_config=CoupledNewtonConfig(),
+            inverse_exponent_override={1: {0: 0.0}} if c["override_1d"] else {},
+        )
+    elif c["preconditioner"] == "eigh":
+        pc = RootInvShampooPreconditionerConfig(
+            amortized_computation_config=EigenConfig(),
+            inverse_exponent_override={1: {0: 0.0}} if c["override_1d"] else {},
+        )
+    elif c["preconditioner"] == "soap_qr":
+        pc = EigenvalueCorrectedShampooPreconditionerConfig(
+            amortized_computation_config=QREigendecompositionConfig()
+        )
+        assert pc == DefaultSOAPConfig
+    else:
+        raise ValueError(c["preconditioner"])
+    graft = {
+        None: None,
+        "adam": AdamPreconditionerConfig(beta2=c.get("grafting_beta2", 0.999), epsilon=c.get("grafting_epsilon", 1e-10)),
+        "adagrad": AdaGradPreconditionerConfig(epsilon=c.get("grafting_epsilon", 1e-10)),
+    }[c["grafting"]]
+    mom = (
+        ClassicMomentumConfig(momentum=c["momentum"], dampening=c["dampening"], use_nesterov=c["use_nesterov"])
+        if c.get("momentum", 0.0) != 0.0
+        else None
+    )
+    return DistributedShampoo(
+        params, lr=c["lr"], betas=tuple(c["betas"]), beta3=c.get("beta3", -1.0), epsilon=c["epsilon"],
+        weight_decay=c["weight_decay"], weight_decay_type=WeightDecayType[c["weight_decay_type"]],
+        max_preconditioner_dim=c["max_preconditioner_dim"], precondition_frequency=c["precondition_frequency"],
+        start_preconditioning_step=c["start_preconditioning_step"], preconditioner_config=pc, grafting_config=graft,
+        iterate_averaging_config=mom,
+    )
+
+
+def run_case(name, c):
+    shapes = [tuple(s) for s in c["shapes"]]
+    if c.get("zero_init"):
+        init = [torch.zeros(*s) for s in shapes]
+    else:
+        init = case_params(shapes, c["seed"])
+    params = [torch.nn.Parameter(t.clone()) for t in init]
+    opt = build_reference(c, params)
+    out = {}
+    dist_calls = []
+    real_dist = torch.dist
+
+    def counting_dist(*a, **k):
+        dist_calls[-1] += 1
+        return real_dist(*a, **k)
+
+    real_mir = matrix_inverse_root
+
+    def counting_mir(*a, **k):
+        dist_calls.append(0)
+        return real_mir(*a, **k)
+
+    iters_per_step = []
+    if c.get("torch_seed_grads"):
+        torch.manual_seed(c["seed"])
+    with mock.patch.object(torch, "dist", counting_dist), mock.patch(
+        "distributed_shampoo.preconditioner.shampoo_preconditioner_list.matrix_inverse_root", counting_mir
+    ):
+        for s in range(1, c["steps"] + 1):
+            if c.get("torch_seed_grads"):
+                grads = [torch.randn_like(p) for p in params]
+            else:
+                grads = case_grads(shapes, c["seed"], s, c["grad_scale"])
+            for p, g in zip(params, grads):
+                p.grad = g
+            dist_calls.clear()
+            opt.step()
+            # torch.dist is called once before the loop and once per iteration
+            iters_per_step.append([n - 1 for n in dist_calls])
+            for i, p in enumerate(params):
+                out[f"norm_s{s}_p{i}"] = np.float64(p.detach().double().norm().item())
+    big = max(p.numel() for p in params) > 100_000
+    for i, p in enumerate(params):
+        flat = p.detach().reshape(-1)
+        out[f"final_p{i}"] = (flat[::37] if big else flat).numpy().copy()
+    # optimizer state (only for the small cases)
+    if not big:
+        for pi, p in enumerate(params):
+            st = opt.state[p]
+            for key, val in st.items():
+                if not isinstance(val, dict):
+                    continue
+                for sk, sv in val.items():
+                    if isinstance(sv, torch.Tensor):
+                        out[f"state_p{pi}_{key}_{sk}"] = sv.numpy().copy()
+                    elif sk == "shampoo":
+                        for fname in ("factor_matrices", "inv_factor_matrices", "factor_matrices_eigenvectors"):
+                            for k, t in enumerate(getattr(sv, fname, ())):
+                                out[f"state_p{pi}_{key}_{fname}_{k}"] = t.numpy().copy()
+                        if hasattr(sv, "corrected_eigenvalues"):
+                            out[f"state_p{pi}_{key}_corrected_eigenvalues"] = sv.corrected_eigenvalues.numpy().copy()
+    maxlen = max((len(x) for x in iters_per_step), default=0)
+    it = np.full((len(iters_per_step), max(maxlen, 1)), -1, dtype=np.int64)
+    for r, row in enumerate(iters_per_step):
+        it[r, : len(row)] = row
+    out["newton_iterations"] = it
+    np.savez_compressed(os.path.join(OUT, f"{name}.npz"), **out)
+    print(name, "ok; iterations per amortized step:", [r for r in iters_per_step if r][:3])
+
+
+def cfg1_as_stated():
+    """BASELINE config 1 verbatim: what does the reference do?"""
+    torch.manual_seed(0)
+    w = torch.nn.Parameter(torch.zeros(512, 512))
+    b = torch.nn.Parameter(torch.zeros(512))
+    opt = DistributedShampoo(
+        [w, b], lr=1e-3, betas=(0.9, 0.999), epsilon=1e-12, max_preconditioner_dim=512,
+        precondition_frequency=1, start_preconditioning_step=1,
+        preconditioner_config=RootInvShampooPreconditionerConfig(amortized_computation_config=CoupledNewtonConfig()),
+        grafting_config=AdamPreconditionerConfig(beta2=0.999, epsilon=1e-8),
+    )
+    rec = {"raised": False}
+    for s in range(1, 11):
+        w.grad = torch.randn_like(w)
+        b.grad = torch.randn_like(b)
+        try:
+            opt.step()
+        except Exception as e:  # noqa: BLE001
+            rec = {"raised": True, "step": s, "type": type(e).__name__, "mro": [k.__name__ for k in type(e).__mro__],
+                   "message_prefix": str(e)[:80]}
+            break
+    with open(os.path.join(OUT, "cfg1_as_stated.json"), "w") as f:
+        json.dump(rec, f, indent=1)
+    print("cfg1_as_stated", rec)
+
+
+def newton_trajectories():
+    """matrix_inverse_root (coupled Newton) on stored inputs: X, iteration count, finiteness."""
+    g = torch.Generator().manual_seed(7)
+    mats = {}
+    a = torch.randn(64, 256, generator=g)
+    mats["wellcond64_r4"] = (a @ a.T / 256, 4, 1e-12)
+    a = torch.randn(48, 100, generator=g)
+    mats["wellcond48_r2"] = (a @ a.T / 100, 2, 1e-12)
+    a = torch.randn(128, 128, generator=g)
+    mats["square128_r4"] = (a @ a.T, 4, 1e-12)
+    a = torch.randn(96, 1, generator=g)
+    mats["rank1_96_r2_bigeps"] = (a @ a.T, 2, 1e-1)
+    a = torch.randn(32, 1, generator=g)
+    mats["rank1_32_r2"] = (a @ a.T, 2, 1e-12)
+    a = torch.randn(40, 24, generator=g)
+    mats["rank24_40_r4"] = (a @ a.T, 4, 1e-12)
+    mats["scaled_identity_r4"] = (3.0 * torch.eye(20), 4, 0.0)
+    out = {}
+    for name, (A, root, eps) in mats.items():
+        calls = [0]
+        real = torch.dist
+
+        def cd(*aa, **kk):
+            calls[0] += 1
+            return real(*aa, **kk)
+
+        with mock.patch.object(torch, "dist", cd):
+            X = matrix_inverse_root(A, Fraction(root), CoupledNewtonConfig(), eps)
+        out[f"{name}_A"] = A.numpy()
+        out[f"{name}_X"] = X.numpy()
+        out[f"{name}_meta"] = np.array([root, calls[0] - 1, int(torch.isfinite(X).all())], dtype=np.int64)
+        out[f"{name}_eps"] = np.float64(eps)
+        print("newton", name, "iters", calls[0] - 1, "finite", bool(torch.isfinite(X).all()))
+    np.savez_compressed(os.path.join(OUT, "newton_trajectories.npz"), **out)
+
+
+def eig_cases():
+    """eigh root inverse and one QR refresh on stored inputs."""
+    g = torch.Generator().manual_seed(11)
+    out = {}
+    a = torch.randn(40, 64, generator=g)
+    A = a @ a.T / 64
+    out["eigh_A"] = A.numpy()
+    out["eigh_X_r4"] = matrix_inverse_root(A, Fraction(4), EigenConfig(), 1e-12).numpy()
+    a = torch.randn(30, 10, generator=g)
+    A2 = a @ a.T
+    out["eigh_def_A"] = A2.numpy()
+    out["eigh_def_X_r2_eps1e-3"] = matrix_inverse_root(A2, Fraction(2), EigenConfig(), 1e-3).numpy()
+    # QR refresh from identity and from a previous basis, incl. sort permutation
+    Q0 = torch.eye(40)
+    l1, Q1 = matrix_eigendecomposition(A, 1e-12, QREigendecompositionConfig(), Q0)
+    a = torch.randn(40, 64, generator=g)
+    A3 = 0.9 * A + 0.1 * (a @ a.T / 64)
+    l2, Q2 = matrix_eigendecomposition(A3, 1e-12, QREigendecompositionConfig(), Q1)
+    l3, Q3 = matrix_eigendecomposition(A3, 1e-12, QREigendecompositionConfig(max_iterations=5, tolerance=0.05), Q2)
+    for k, v in dict(qr_A=A, qr_A3=A3, qr_l1=l1, qr_Q1=Q1, qr_l2=l2, qr_Q2=Q2, qr_l3=l3, qr_Q3=Q3).items():
+        out[k] = v.numpy()
+    np.savez_compressed(os.path.join(OUT, "eig_cases.npz"), **out)
+    print("eig cases ok")
+
+
+if __name__ == "__main__":
+    torch.set_num_threads(8)
+    with open(os.path.join(OUT, "cases.json"), "w") as f:
+        json.dump(CASES, f, indent=1)
+    newton_trajectories()
+    eig_cases()
+    cfg1_as_stated()
+    for n, c in CASES.items():
+        run_case(n, c)
