@@ -1,0 +1,167 @@
+/*
+ * C ABI of the MI355X-native Distributed Shampoo step (libshampoo_amd.so).
+ *
+ * The reference (facebookresearch/optimizers) is pure Python over torch ops and has no FFI
+ * of its own; the seam this library plugs into is the `PreconditionerList` interface
+ * (distributed_shampoo/preconditioner/preconditioner_list.py:49-102) together with the
+ * default `Distributor` (distributed_shampoo/distributor/shampoo_distributor.py:302-430)
+ * and the elementwise part of `DistributedShampoo._compute_search_directions`
+ * (distributed_shampoo/distributed_shampoo.py:1384-1501).  Each entry point names the
+ * reference routine it replaces.
+ *
+ * Conventions: every pointer inside a descriptor is a DEVICE pointer borrowed from the
+ * caller (who keeps it alive until the stream work has finished); `stream` is a
+ * hipStream_t passed as void*; every call returns SA_OK or an error code and leaves a
+ * message for sa_last_error().  No exceptions cross the boundary.  All arithmetic is fp32.
+ * One plan describes the blocks of one parameter group on one GPU; calls on one plan must
+ * not overlap.
+ */
+#ifndef SHAMPOO_AMD_H
+#define SHAMPOO_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SA_OK 0
+#define SA_ERR_INVALID 1     /* bad argument */
+#define SA_ERR_HIP 2         /* a HIP runtime call failed */
+#define SA_ERR_WORKSPACE 3   /* workspace missing or too small */
+#define SA_ERR_UNSUPPORTED 4 /* valid in the reference, not built here */
+#define SA_ERR_STATE 5       /* call order violated (e.g. gradients not bound) */
+
+/* Per-factor status written by sa_compute_root_inverses_newton. */
+#define SA_FACTOR_OK 0
+#define SA_FACTOR_INPUT_NONFINITE 1  /* bias-corrected factor holds nan/inf (shampoo_preconditioner_list.py:374) */
+#define SA_FACTOR_RESULT_NONFINITE 2 /* inverse root holds nan/inf        (shampoo_preconditioner_list.py:405) */
+#define SA_FACTOR_NOT_CONVERGED 3    /* max_iterations reached; result kept (matrix_functions.py:678-681) */
+#define SA_FACTOR_SKIPPED 4          /* follows a non-finite factor; not computed, state untouched */
+
+/* Grafting flavours (distributed_shampoo.py:673-714). */
+#define SA_GRAFT_NONE 0
+#define SA_GRAFT_SGD 1
+#define SA_GRAFT_ADAGRAD 2 /* AdaGrad / RMSprop / Adam: second moment + optional bias correction */
+
+typedef struct sa_plan sa_plan;
+
+/*
+ * One block of a (merged) parameter: an fp32 rows x cols strided view, produced by
+ * merge_small_dims + multi_dim_split (utils/shampoo_utils.py:38-174).  A 1-D block of
+ * length d is rows = d, cols = 1, ld = 1.  State buffers are contiguous (rows*cols).
+ * Mirrors what BlockInfo + the per-block optimizer state hold
+ * (distributor/shampoo_block_info.py:18-65; state keys shampoo_types.py:35-41).
+ */
+typedef struct sa_block_desc {
+  int32_t rows, cols;
+  int64_t ld;             /* row stride, in elements, of the block inside its parameter and gradient */
+  float* param;           /* block of the parameter (updated in place) */
+  float* filtered_grad;   /* EMA of the gradient, or NULL when beta1 == 0 */
+  float* adagrad;         /* grafting second moment, or NULL */
+  float* momentum_buffer; /* classic momentum buffer, or NULL */
+  float* factor[2];       /* packed upper-triangular Kronecker factor of dim 0 / dim 1; NULL = dim not preconditioned */
+  float* inv_factor[2];   /* packed upper-triangular inverse root of that factor */
+  int32_t root[2];        /* integer inverse root (4 for matrices, 2 for vectors by default) */
+} sa_block_desc;
+
+/* Scalars of one step, already evaluated by the host exactly as the reference evaluates
+ * them (fp32 bias corrections: distributed_shampoo.py:1190-1195,
+ * adagrad_preconditioner_list.py:139-141). */
+typedef struct sa_step_scalars {
+  float lr;
+  float beta1;             /* 0 disables the filtered gradient */
+  float beta3;             /* == beta1 unless set */
+  float bias_correction1;  /* divisor of the filtered gradient, 1.0f when off */
+  int32_t graft_type;      /* SA_GRAFT_* */
+  float graft_beta2;
+  float graft_weight;      /* weighting factor of g*g */
+  float graft_bias_correction2; /* divisor of the second moment, 1.0f when off */
+  float graft_epsilon;
+  float weight_decay_alpha; /* added to the direction as alpha*W (decoupled / corrected / independent); 0 = none */
+  float momentum;           /* 0 = classic momentum off */
+  float dampening;
+  int32_t use_nesterov;
+} sa_step_scalars;
+
+const char* sa_last_error(void);
+int32_t sa_abi_version(void);
+
+/* Builds the ragged batched descriptor table for a parameter group (replaces the per-step
+ * Python list building of shampoo_distributor.py:237-299 and the per-block loops of
+ * shampoo_preconditioner_list.py:1509-1539, 1672-1695). */
+int32_t sa_plan_create(const sa_block_desc* blocks, int32_t n_blocks, sa_plan** plan_out);
+void sa_plan_destroy(sa_plan* plan);
+
+/* Scratch + dense-inverse cache the caller must provide (device memory, 256-byte aligned). */
+int64_t sa_plan_workspace_bytes(const sa_plan* plan);
+int32_t sa_plan_bind_workspace(sa_plan* plan, void* workspace, int64_t bytes);
+
+/* Number of factor matrices, in block order then dim order (the order of every per-factor array). */
+int32_t sa_plan_num_factors(const sa_plan* plan);
+
+/* Marks the dense inverse cache stale (after the caller wrote inv_factor itself, e.g. load_state_dict). */
+int32_t sa_plan_invalidate_inverse_cache(sa_plan* plan);
+
+/* Gradients of this step, one device pointer per block (same rows/cols/ld as the block); NULL
+ * masks a block out of every following call (shampoo_distributor.py:269-277). */
+int32_t sa_plan_bind_gradients(sa_plan* plan, float* const* grads, void* stream);
+
+/* G += weight_decay * W, in place on the gradient (distributed_shampoo.py:1127-1139). */
+int32_t sa_add_l2_regularization(sa_plan* plan, float weight_decay, void* stream);
+
+/* L <- beta2 L + w G G^T, R <- beta2 R + w G^T G on packed storage
+ * (shampoo_preconditioner_list.py:1490-1539). */
+int32_t sa_update_factor_matrices(sa_plan* plan, float beta2, float weighting_factor, void* stream);
+
+/* Batched coupled inverse Newton iteration on every factor, A = unpack(factor / bias_correction2)
+ * (matrix_functions.py:368-437 via shampoo_preconditioner_list.py:314-443, 631-680).
+ * iterations_out / status_out: host arrays of sa_plan_num_factors() entries.  Inverse roots of
+ * factors that precede the first non-finite one are stored into inv_factor (upper triangle);
+ * the call synchronises the stream before it returns. */
+int32_t sa_compute_root_inverses_newton(sa_plan* plan, float bias_correction2, float epsilon,
+                                        int32_t max_iterations, float tolerance,
+                                        int32_t* iterations_out, int32_t* status_out, void* stream);
+
+/* Grafting second moment, filtered gradient and the grafted direction's squared norm per block
+ * (adagrad_preconditioner_list.py:122-162, distributed_shampoo.py:1162-1199, 1110-1114). */
+int32_t sa_update_grafting_and_filtered_grad(sa_plan* plan, const sa_step_scalars* s, void* stream);
+
+/* P = L^-1/r0 * Ghat * R^-1/r1 into the workspace plus its squared norm per block
+ * (shampoo_preconditioner_list.py:1541-1578, 1672-1695, 1780-1790). */
+int32_t sa_precondition(sa_plan* plan, const sa_step_scalars* s, void* stream);
+
+/* Grafting rescale, weight decay, momentum, learning rate and W += P
+ * (distributed_shampoo.py:1115-1122, 1202-1293, 1484; shampoo_distributor.py:335-365). */
+int32_t sa_apply_update(sa_plan* plan, const sa_step_scalars* s, void* stream);
+
+/* Whole step before preconditioning starts: the grafted direction is the update
+ * (distributed_shampoo.py:1093-1098 followed by :1202-1293, 1484). */
+int32_t sa_grafting_only_step(sa_plan* plan, const sa_step_scalars* s, void* stream);
+
+/* Test / measurement aids. */
+
+/* Per-block squared norms of the last step: graft_sq[i], precond_sq[i] (host arrays of n_blocks). */
+int32_t sa_plan_read_norms(sa_plan* plan, float* graft_sq, float* precond_sq, void* stream);
+
+/* Copies the preconditioned (unscaled) direction of block i into out (device, contiguous rows*cols). */
+int32_t sa_plan_read_preconditioned(sa_plan* plan, int32_t block, float* out, void* stream);
+
+/* C = op(A) op(B) with the grouped MFMA kernel, one problem, `batch` copies strided by the given
+ * element strides.  a_layout: 0 = A[m*lda+k], 1 = A[k*lda+m]; b_layout: 0 = B[k*ldb+n], 1 = B[n*ldb+k]. */
+int32_t sa_gemm_f32(const float* A, const float* B, float* C, int32_t M, int32_t N, int32_t K,
+                    int64_t lda, int64_t ldb, int64_t ldc, int32_t a_layout, int32_t b_layout,
+                    int32_t batch, int64_t stride_a, int64_t stride_b, int64_t stride_c, void* stream);
+
+/* Averaged duration (milliseconds, HIP events on `stream`) of the kernels of the named phase during
+ * the most recent call that ran it: "newton_gemm", "syrk", "precondition_gemm", "grafting", "apply".
+ * Timing is off unless sa_set_profiling(1) was called; returns a negative value if unavailable. */
+int32_t sa_set_profiling(int32_t enabled);
+double sa_phase_ms(const char* phase);
+double sa_phase_flops(const char* phase); /* algorithmic flops (or bytes for HBM-bound phases) of that call */
+int32_t sa_phase_launches(const char* phase); /* kernel launches the phase issued in that call */
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SHAMPOO_AMD_H */

@@ -1,0 +1,527 @@
+// HBM-bound kernels of the Shampoo step: grafting second moment + filtered gradient,
+// norm reductions, the final parameter update, and the symmetric pack / unpack / Newton
+// initialisation passes over factor matrices.
+//
+// Elementwise work is cut into chunks of 4096 consecutive block elements (256 threads x
+// 4 x float4); a chunk table maps a workgroup to (block, first element), so one launch
+// covers every ragged block of a parameter group and fills all 256 CUs.  Reductions are
+// wavefront shuffles -> one LDS slot per wavefront -> one partial per chunk, summed in a
+// fixed order by a second tiny kernel, so results do not depend on scheduling.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/shampoo_amd.h"
+#include "gemm.h"
+
+namespace sa {
+
+constexpr int EW_THREADS = 256;
+constexpr int EW_CHUNK = 4096;
+
+struct BlockDev {
+  float* param;
+  float* grad;
+  float* filtered_grad;
+  float* adagrad;
+  float* momentum;
+  float* ghat_tmp;        // lerp(m, g, 1-beta3) when beta3 != beta1, else nullptr
+  const float* ghat_src;  // where the (undivided) filtered gradient is read from after the prologue
+  const float* p_src;     // direction the update kernel consumes
+  long long ld;           // row stride of param / grad
+  long long ghat_ld;
+  long long p_ld;
+  int rows, cols;
+  int chunk_begin, chunk_end;  // range in the per-chunk partial arrays
+  int ptile_begin, ptile_end;  // range in the per-tile partial array (preconditioned blocks)
+  int vec;                // every pointer of this block is 16-byte aligned and rows hold multiples of 4
+  int p_vec;              // same for p_src
+  int p_is_ghat;          // block has no preconditioned dim: direction = filtered gradient
+};
+
+struct ChunkRef { int block; int start; };
+
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+__device__ __forceinline__ float lerp_like_torch(float a, float b, float w) {
+  // ATen lerp: a + w*(b-a) for w < 0.5, else b - (b-a)*(1-w)
+  const float diff = b - a;
+  return (w < 0.5f) ? a + w * diff : b - diff * (1.0f - w);
+}
+
+struct PreOut { float graft; float ghat; };
+
+// One element of: v <- b2 v + w g^2 ; m <- lerp(m, g, 1-b1) ; ghat = m / bc1 ;
+// graft = ghat / (sqrt(v / bc2) + eps)
+__device__ __forceinline__ PreOut pre_element(float g, float& m, float& v, float& gh_tmp,
+                                              const sa_step_scalars& s, bool has_m, bool has_v,
+                                              bool beta3_differs) {
+  PreOut o;
+  if (has_v) {
+    float vv = v;
+    if (s.graft_beta2 != 1.0f) vv = vv * s.graft_beta2;
+    vv = vv + (s.graft_weight * g) * g;
+    v = vv;
+  }
+  float num;
+  if (has_m) {
+    float mm = m;
+    if (beta3_differs) {
+      gh_tmp = lerp_like_torch(mm, g, 1.0f - s.beta3);
+      num = gh_tmp;
+    }
+    mm = lerp_like_torch(mm, g, 1.0f - s.beta1);
+    m = mm;
+    if (!beta3_differs) num = mm;
+  } else {
+    num = g;
+  }
+  o.ghat = num / s.bias_correction1;
+  if (s.graft_type == SA_GRAFT_ADAGRAD) {
+    const float den = sqrtf(v / s.graft_bias_correction2) + s.graft_epsilon;
+    o.graft = o.ghat / den;
+  } else {
+    o.graft = o.ghat;
+  }
+  return o;
+}
+
+__device__ __forceinline__ float apply_element(float p, float& w, float& mom, const sa_step_scalars& s,
+                                               float scale, bool has_mom) {
+  p = p * scale;
+  if (s.weight_decay_alpha != 0.0f) p = p + s.weight_decay_alpha * w;
+  if (has_mom) {
+    float mb = mom * s.momentum;
+    mb = mb + (1.0f - s.dampening) * p;
+    mom = mb;
+    p = s.use_nesterov ? (p * (1.0f - s.dampening)) + s.momentum * mb : mb;
+  }
+  p = p * (-s.lr);
+  w = w + p;
+  return p;
+}
+
+// MODE 0: prologue of a preconditioned step (updates v, m; partial norms).
+// MODE 1: whole grafting-only step (also applies the update to W).
+template <int MODE>
+__global__ __launch_bounds__(EW_THREADS) void grafting_kernel(const BlockDev* __restrict__ blocks,
+                                                             const ChunkRef* __restrict__ chunks,
+                                                             sa_step_scalars s,
+                                                             float* __restrict__ graft_partial,
+                                                             float* __restrict__ ghat_partial) {
+  __shared__ float red[4];
+  const ChunkRef cr = chunks[blockIdx.x];
+  const BlockDev& B = blocks[cr.block];
+  const int n_el = B.rows * B.cols;
+  const bool has_m = B.filtered_grad != nullptr, has_v = B.adagrad != nullptr;
+  const bool has_mom = B.momentum != nullptr && s.momentum != 0.0f;
+  const bool b3 = B.ghat_tmp != nullptr;
+  const bool contig = (B.ld == B.cols);
+  float gsum = 0.f, hsum = 0.f;
+#pragma unroll
+  for (int it = 0; it < EW_CHUNK / (EW_THREADS * 4); ++it) {
+    const int e = cr.start + (it * EW_THREADS + threadIdx.x) * 4;
+    if (e >= n_el) continue;
+    const long long gi = contig ? (long long)e : (long long)(e / B.cols) * B.ld + (e % B.cols);
+    const bool vec = (e + 3 < n_el) && (B.vec != 0);
+    if (vec) {
+      float4 g = *reinterpret_cast<const float4*>(B.grad + gi);
+      float4 m = has_m ? *reinterpret_cast<const float4*>(B.filtered_grad + e) : make_float4(0, 0, 0, 0);
+      float4 v = has_v ? *reinterpret_cast<const float4*>(B.adagrad + e) : make_float4(0, 0, 0, 0);
+      float4 t = make_float4(0, 0, 0, 0);
+      PreOut o0 = pre_element(g.x, m.x, v.x, t.x, s, has_m, has_v, b3);
+      PreOut o1 = pre_element(g.y, m.y, v.y, t.y, s, has_m, has_v, b3);
+      PreOut o2 = pre_element(g.z, m.z, v.z, t.z, s, has_m, has_v, b3);
+      PreOut o3 = pre_element(g.w, m.w, v.w, t.w, s, has_m, has_v, b3);
+      if (has_m) *reinterpret_cast<float4*>(B.filtered_grad + e) = m;
+      if (has_v) *reinterpret_cast<float4*>(B.adagrad + e) = v;
+      if (b3) *reinterpret_cast<float4*>(B.ghat_tmp + e) = t;
+      if (MODE == 0) {
+        gsum += (o0.graft * o0.graft + o1.graft * o1.graft) + (o2.graft * o2.graft + o3.graft * o3.graft);
+        hsum += (o0.ghat * o0.ghat + o1.ghat * o1.ghat) + (o2.ghat * o2.ghat + o3.ghat * o3.ghat);
+      } else {
+        float4 w = *reinterpret_cast<const float4*>(B.param + gi);
+        float4 mo = has_mom ? *reinterpret_cast<const float4*>(B.momentum + e) : make_float4(0, 0, 0, 0);
+        apply_element(o0.graft, w.x, mo.x, s, 1.0f, has_mom);
+        apply_element(o1.graft, w.y, mo.y, s, 1.0f, has_mom);
+        apply_element(o2.graft, w.z, mo.z, s, 1.0f, has_mom);
+        apply_element(o3.graft, w.w, mo.w, s, 1.0f, has_mom);
+        *reinterpret_cast<float4*>(B.param + gi) = w;
+        if (has_mom) *reinterpret_cast<float4*>(B.momentum + e) = mo;
+      }
+    } else {
+      for (int k = 0; k < 4 && e + k < n_el; ++k) {
+        const int ee = e + k;
+        const long long gk = contig ? (long long)ee : (long long)(ee / B.cols) * B.ld + (ee % B.cols);
+        float g = B.grad[gk];
+        float m = has_m ? B.filtered_grad[ee] : 0.f;
+        float v = has_v ? B.adagrad[ee] : 0.f;
+        float t = 0.f;
+        PreOut o = pre_element(g, m, v, t, s, has_m, has_v, b3);
+        if (has_m) B.filtered_grad[ee] = m;
+        if (has_v) B.adagrad[ee] = v;
+        if (b3) B.ghat_tmp[ee] = t;
+        if (MODE == 0) {
+          gsum += o.graft * o.graft;
+          hsum += o.ghat * o.ghat;
+        } else {
+          float w = B.param[gk];
+          float mo = has_mom ? B.momentum[ee] : 0.f;
+          apply_element(o.graft, w, mo, s, 1.0f, has_mom);
+          B.param[gk] = w;
+          if (has_mom) B.momentum[ee] = mo;
+        }
+      }
+    }
+  }
+  if (MODE == 0) {
+    const float gs = block_sum(gsum, red);
+    __syncthreads();
+    const float hs = block_sum(hsum, red);
+    if (threadIdx.x == 0) {
+      graft_partial[blockIdx.x] = gs;
+      ghat_partial[blockIdx.x] = hs;
+    }
+  }
+}
+
+// norms[b] = sum of graft partials, norms[n + b] = sum of the direction's partials; one workgroup per block.
+__global__ __launch_bounds__(EW_THREADS) void reduce_norms_kernel(const BlockDev* __restrict__ blocks,
+                                                                 const int* __restrict__ active_blocks,
+                                                                 int n_blocks,
+                                                                 const float* __restrict__ graft_partial,
+                                                                 const float* __restrict__ ghat_partial,
+                                                                 const float* __restrict__ ptile_partial,
+                                                                 float* __restrict__ norms) {
+  __shared__ float red[4];
+  const int b = active_blocks[blockIdx.x];
+  const BlockDev& B = blocks[b];
+  float a = 0.f;
+  for (int i = B.chunk_begin + threadIdx.x; i < B.chunk_end; i += EW_THREADS) a += graft_partial[i];
+  const float g = block_sum(a, red);
+  __syncthreads();
+  float c = 0.f;
+  if (B.p_is_ghat) {
+    for (int i = B.chunk_begin + threadIdx.x; i < B.chunk_end; i += EW_THREADS) c += ghat_partial[i];
+  } else {
+    for (int i = B.ptile_begin + threadIdx.x; i < B.ptile_end; i += EW_THREADS) c += ptile_partial[i];
+  }
+  const float p = block_sum(c, red);
+  if (threadIdx.x == 0) {
+    norms[b] = g;
+    norms[n_blocks + b] = p;
+  }
+}
+
+// W <- W - lr * (momentum(P * ||graft|| / (||P|| + 1e-16) + alpha W))
+__global__ __launch_bounds__(EW_THREADS) void apply_kernel(const BlockDev* __restrict__ blocks,
+                                                          const ChunkRef* __restrict__ chunks,
+                                                          sa_step_scalars s, int n_blocks,
+                                                          const float* __restrict__ norms) {
+  const ChunkRef cr = chunks[blockIdx.x];
+  const BlockDev& B = blocks[cr.block];
+  const int n_el = B.rows * B.cols;
+  const bool has_mom = B.momentum != nullptr && s.momentum != 0.0f;
+  const bool contig = (B.ld == B.cols);
+  const bool p_contig = (B.p_ld == B.cols);
+  const float p_div = B.p_is_ghat ? s.bias_correction1 : 1.0f;
+  float scale = 1.0f;
+  if (s.graft_type != SA_GRAFT_NONE) {
+    const float gn = sqrtf(norms[cr.block]);
+    const float pn = sqrtf(norms[n_blocks + cr.block]) + 1e-16f;
+    scale = gn / pn;
+  }
+#pragma unroll
+  for (int it = 0; it < EW_CHUNK / (EW_THREADS * 4); ++it) {
+    const int e = cr.start + (it * EW_THREADS + threadIdx.x) * 4;
+    if (e >= n_el) continue;
+    const long long wi = contig ? (long long)e : (long long)(e / B.cols) * B.ld + (e % B.cols);
+    const long long pi = p_contig ? (long long)e : (long long)(e / B.cols) * B.p_ld + (e % B.cols);
+    const bool vec = (e + 3 < n_el) && (B.vec != 0) && (B.p_vec != 0);
+    if (vec) {
+      float4 p = *reinterpret_cast<const float4*>(B.p_src + pi);
+      float4 w = *reinterpret_cast<const float4*>(B.param + wi);
+      float4 mo = has_mom ? *reinterpret_cast<const float4*>(B.momentum + e) : make_float4(0, 0, 0, 0);
+      apply_element(p.x / p_div, w.x, mo.x, s, scale, has_mom);
+      apply_element(p.y / p_div, w.y, mo.y, s, scale, has_mom);
+      apply_element(p.z / p_div, w.z, mo.z, s, scale, has_mom);
+      apply_element(p.w / p_div, w.w, mo.w, s, scale, has_mom);
+      *reinterpret_cast<float4*>(B.param + wi) = w;
+      if (has_mom) *reinterpret_cast<float4*>(B.momentum + e) = mo;
+    } else {
+      for (int k = 0; k < 4 && e + k < n_el; ++k) {
+        const int ee = e + k;
+        const long long wk = contig ? (long long)ee : (long long)(ee / B.cols) * B.ld + (ee % B.cols);
+        const long long pk = p_contig ? (long long)ee : (long long)(ee / B.cols) * B.p_ld + (ee % B.cols);
+        float w = B.param[wk];
+        float mo = has_mom ? B.momentum[ee] : 0.f;
+        apply_element(B.p_src[pk] / p_div, w, mo, s, scale, has_mom);
+        B.param[wk] = w;
+        if (has_mom) B.momentum[ee] = mo;
+      }
+    }
+  }
+}
+
+// G += wd * W in place on the gradient.
+__global__ __launch_bounds__(EW_THREADS) void l2_kernel(const BlockDev* __restrict__ blocks,
+                                                       const ChunkRef* __restrict__ chunks, float wd) {
+  const ChunkRef cr = chunks[blockIdx.x];
+  const BlockDev& B = blocks[cr.block];
+  const int n_el = B.rows * B.cols;
+  const bool contig = (B.ld == B.cols);
+  for (int it = 0; it < EW_CHUNK / EW_THREADS; ++it) {
+    const int e = cr.start + it * EW_THREADS + threadIdx.x;
+    if (e >= n_el) break;
+    const long long gi = contig ? (long long)e : (long long)(e / B.cols) * B.ld + (e % B.cols);
+    B.grad[gi] = B.grad[gi] + wd * B.param[gi];
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Symmetric factor passes.  A factor of dimension d is stored packed (row-major upper
+// triangle, (r,c), c >= r at r*d - r*(r-1)/2 + c - r) in optimizer state and dense, mirrored
+// and zero padded to dpad x dpad (dpad a multiple of 128) in the workspace.  All three
+// passes walk pairs of 64x64 tiles (bi <= bj): the upper tile is read coalesced and its
+// transpose is produced through LDS.
+// ---------------------------------------------------------------------------------------
+
+constexpr int ST = 64;  // symmetric pass tile
+
+struct SymFactor {
+  const float* packed_in;  // packed source (factor for Newton init, inverse for unpack)
+  float* packed_out;       // packed destination (commit)
+  const float* dense_in;   // dense source (commit)
+  float* dense_out[3];     // dense destinations
+  unsigned int* err_bits;
+  const float* norm_partial;  // Newton init: per-chunk partial sums of squares
+  int n_norm_partial;
+  int d, dpad;
+  int tile_begin;          // first tile-pair id
+  int tiles;               // dpad / ST
+  int root;
+  int enabled;
+};
+
+__device__ __forceinline__ long long packed_off(int r, int c, int d) {
+  return (long long)r * d - ((long long)r * (r - 1)) / 2 + (c - r);
+}
+
+__device__ __forceinline__ void sym_locate(const SymFactor* __restrict__ f, int n, int id, int& fi, int& bi, int& bj) {
+  int lo = 0, hi = n - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (f[mid].tile_begin <= id) lo = mid; else hi = mid - 1;
+  }
+  fi = lo;
+  int t = id - f[lo].tile_begin;
+  bi = 0;
+  int rowlen = f[lo].tiles;
+  while (t >= rowlen) { t -= rowlen; ++bi; --rowlen; }
+  bj = bi + t;
+}
+
+enum SymMode { SYM_UNPACK = 0, SYM_NEWTON_INIT = 1, SYM_COMMIT = 2 };
+
+// SYM_UNPACK:      dense_out[0] = mirror(packed_in)
+// SYM_NEWTON_INIT: a = packed_in / bc2 (+ eps on the diagonal); z = (root+1)/(2 ||A||_F);
+//                  dense_out[0] = M = z a, dense_out[1] = M_p = M*mp_scale + mp_diag I,
+//                  dense_out[2] = X = z^(1/root) I, err = max |M - I|
+// SYM_COMMIT:      packed_out = upper(dense_in) (if packed_out), dense_out[0] = mirror(upper(dense_in))
+template <int MODE>
+__global__ __launch_bounds__(256) void sym_pass_kernel(const SymFactor* __restrict__ factors, int n_factors,
+                                                      float bc2, float eps, float mp_scale, float mp_diag) {
+  __shared__ float tile[ST][ST + 1];
+  __shared__ float zsh;
+  int fi, bi, bj;
+  sym_locate(factors, n_factors, blockIdx.x, fi, bi, bj);
+  const SymFactor& F = factors[fi];
+  if (!F.enabled) return;
+  const int d = F.d, dpad = F.dpad;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 x 4
+
+  float z = 1.0f, x0 = 0.f;
+  if (MODE == SYM_NEWTON_INIT) {
+    if (threadIdx.x == 0) {
+      float ssum = 0.f;
+      for (int i = 0; i < F.n_norm_partial; ++i) ssum += F.norm_partial[i];
+      zsh = (float)(F.root + 1) / (2.0f * sqrtf(ssum));
+    }
+    __syncthreads();
+    z = zsh;
+    x0 = powf(z, 1.0f / (float)F.root);
+  }
+
+  // load the upper tile (rows of block bi, cols of block bj); symmetric value for the diagonal tile
+  for (int rr = ty; rr < ST; rr += 4) {
+    const int r = bi * ST + rr, c = bj * ST + tx;
+    float v = 0.f;
+    if (r < d && c < d) {
+      if (MODE == SYM_COMMIT) {
+        const int rs = min(r, c), cs = max(r, c);
+        v = F.dense_in[(long long)rs * dpad + cs];
+      } else {
+        const int rs = min(r, c), cs = max(r, c);
+        v = F.packed_in[packed_off(rs, cs, d)];
+        if (MODE == SYM_NEWTON_INIT) {
+          v = v / bc2;
+          if (r == c && eps != 0.0f) v = v + eps;
+        }
+      }
+    }
+    tile[rr][tx] = v;
+  }
+  __syncthreads();
+
+  float errmax = 0.f;
+  bool errnan = false;
+  // upper placement (bi, bj) and, for off-diagonal tiles, the mirrored placement (bj, bi)
+  for (int pass = 0; pass < ((bi == bj) ? 1 : 2); ++pass) {
+    for (int rr = ty; rr < ST; rr += 4) {
+      const int r = (pass == 0 ? bi : bj) * ST + rr;
+      const int c = (pass == 0 ? bj : bi) * ST + tx;
+      const float v = (pass == 0) ? tile[rr][tx] : tile[tx][rr];
+      const long long o = (long long)r * dpad + c;
+      if (MODE == SYM_UNPACK) {
+        F.dense_out[0][o] = v;
+      } else if (MODE == SYM_COMMIT) {
+        F.dense_out[0][o] = v;
+        if (pass == 0 && F.packed_out != nullptr && r < d && c < d && c >= r) F.packed_out[packed_off(r, c, d)] = v;
+      } else {
+        const float m = z * v;
+        float mp = __fmul_rn(m, mp_scale);
+        const bool diag = (r == c && r < d);
+        if (diag) mp = __fadd_rn(mp, mp_diag);
+        F.dense_out[0][o] = m;
+        F.dense_out[1][o] = mp;
+        F.dense_out[2][o] = diag ? x0 : 0.f;
+        if (r < d && c < d) {
+          const float dv = fabsf(m - (r == c ? 1.0f : 0.0f));
+          if (dv != dv) errnan = true;
+          errmax = fmaxf(errmax, dv);
+        }
+      }
+    }
+  }
+  if (MODE == SYM_NEWTON_INIT) {
+    if (errnan) errmax = __builtin_nanf("");
+    errmax = wave_max_nan(errmax);
+    if ((threadIdx.x & 63) == 0) atomicMax(F.err_bits, __float_as_uint(errmax));
+  }
+}
+
+// Per-factor, per-chunk sums of squares of the bias-corrected, ridged matrix (off-diagonal
+// entries of the packed triangle count twice) and a non-finite flag.
+struct NormJob {
+  const float* src;     // packed factor, or dense matrix when dense != 0
+  float* partial;       // n_chunks partial sums
+  int* nonfinite;       // set to 1 when a non-finite value is seen
+  int d, dpad, dense;
+  int chunk_begin;      // first workgroup id of this job
+  int n_chunks;
+  int enabled;
+};
+
+constexpr int NORM_CHUNK = 16384;
+
+template <bool CHECK_ONLY>
+__global__ __launch_bounds__(256) void factor_norm_kernel(const NormJob* __restrict__ jobs, int n_jobs,
+                                                         float bc2, float eps) {
+  __shared__ float red[4];
+  int lo = 0, hi = n_jobs - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (jobs[mid].chunk_begin <= (int)blockIdx.x) lo = mid; else hi = mid - 1;
+  }
+  const NormJob& J = jobs[lo];
+  if (!J.enabled) return;
+  const int chunk = blockIdx.x - J.chunk_begin;
+  const int d = J.d;
+  float acc = 0.f;
+  bool bad = false;
+  if (J.dense) {
+    // dense d x d inside a dpad-strided buffer; chunked by rows
+    const long long total = (long long)d * d;
+    const long long e0 = (long long)chunk * NORM_CHUNK;
+    for (long long e = e0 + threadIdx.x; e < min(e0 + NORM_CHUNK, total); e += 256) {
+      const int r = (int)(e / d), c = (int)(e % d);
+      const float v = J.src[(long long)r * J.dpad + c];
+      if (!(fabsf(v) <= 3.4028234663852886e38f)) bad = true;
+    }
+  } else {
+    const long long total = (long long)d * (d + 1) / 2;
+    const long long e0 = (long long)chunk * NORM_CHUNK;
+    const long long e1 = min(e0 + NORM_CHUNK, total);
+    // row of the first element of this chunk: largest r with r*d - r(r-1)/2 <= e0
+    // (solved once per thread by a short search from a closed-form guess)
+    for (long long e = e0 + threadIdx.x; e < e1; e += 256) {
+      // invert the packed offset
+      const double dd = (double)d + 0.5;
+      int r = (int)(dd - sqrt(dd * dd - 2.0 * (double)e));
+      if (r < 0) r = 0;
+      if (r > d - 1) r = d - 1;
+      while (r > 0 && packed_off(r, r, d) > e) --r;
+      while (r + 1 < d && packed_off(r + 1, r + 1, d) <= e) ++r;
+      const bool diag = (packed_off(r, r, d) == e);
+      float v = J.src[e] / bc2;
+      if (!(fabsf(v) <= 3.4028234663852886e38f)) bad = true;
+      if (diag && eps != 0.0f) v = v + eps;
+      acc += diag ? v * v : 2.0f * (v * v);
+    }
+  }
+  if (bad) *J.nonfinite = 1;
+  if (!CHECK_ONLY) {
+    const float s = block_sum(acc, red);
+    if (threadIdx.x == 0) J.partial[chunk] = s;
+  }
+}
+
+// Convergence bookkeeping of the batched Newton loop: one thread per factor.
+struct NewtonCtl {
+  unsigned int* err_bits;
+  int* active;
+  int* iterations;
+  int* final_parity;
+  float* final_err;
+};
+
+__global__ void newton_control_kernel(NewtonCtl c, const int* __restrict__ ids, int n, float tol, int max_iter,
+                                      int cur_parity, int* __restrict__ n_active) {
+  __shared__ int cnt;
+  if (threadIdx.x == 0) cnt = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const int f = ids[i];
+    if (!c.active[f]) continue;
+    const float err = __uint_as_float(c.err_bits[f]);
+    // same test as `while error > tolerance and iteration < max_iterations`: NaN ends the loop
+    const bool go = (err > tol) && (c.iterations[f] < max_iter);
+    if (go) {
+      c.iterations[f] += 1;
+      atomicAdd(&cnt, 1);
+    } else {
+      c.active[f] = 0;
+      c.final_parity[f] = cur_parity;
+      c.final_err[f] = err;
+    }
+    c.err_bits[f] = 0u;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) *n_active = cnt;
+}
+
+__global__ void copy_strided_kernel(const float* __restrict__ src, long long lds_, float* __restrict__ dst,
+                                    int rows, int cols) {
+  const long long n = (long long)rows * cols;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (long long)gridDim.x * blockDim.x)
+    dst[e] = src[(e / cols) * lds_ + (e % cols)];
+}
+
+}  // namespace sa

@@ -1,0 +1,318 @@
+// Grouped fp32 MFMA GEMM for gfx950 (CDNA4), the one contraction engine behind the
+// Kronecker-factor update, the coupled-Newton iteration and the preconditioning pair.
+//
+// One launch walks a table of independent problems C = op(A) * op(B).  A workgroup of
+// 256 threads (4 wavefronts of 64, arranged 2x2) owns a 128x128 tile of C; each wavefront
+// owns 64x64 of it as 2x2 v_mfma_f32_32x32x2_f32 accumulators.  K is consumed in slabs of
+// 16 staged through LDS, double buffered: the global loads of slab s+1 are issued before
+// the MFMAs of slab s.  Both operands live in LDS k-major ([k][m] / [k][n], row stride 132
+// floats), so every MFMA fragment is one conflict-free ds_read_b32 per lane.
+//
+// The workgroup id -> tile mapping is XCD aware: hardware deals consecutive workgroup ids
+// round-robin over the 8 XCDs, so id w is remapped to (w % 8) * ceil(T/8) + w / 8, which
+// gives every XCD one contiguous run of tiles; inside a problem tiles are enumerated in
+// 8-row super-rows so that a run of 64 tiles is an 8x8 patch sharing A and B panels in
+// that XCD's L2.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace sa {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 128;
+constexpr int BN = 128;
+constexpr int BK = 16;
+constexpr int LDS_STRIDE = 132;  // 128 + 4: keeps rows 16-byte aligned, skews banks
+constexpr int GEMM_THREADS = 256;
+constexpr int NUM_XCD = 8;
+constexpr int GROUP_ROWS = 8;
+
+// Operand storage.  A_MK: A(m,k) = A[m*lda + k]   A_KM: A(m,k) = A[k*lda + m]
+//                   B_KN: B(k,n) = B[k*ldb + n]   B_NK: B(k,n) = B[n*ldb + k]
+enum ALayout { A_MK = 0, A_KM = 1 };
+enum BLayout { B_KN = 0, B_NK = 1 };
+
+// Epilogues.
+enum Epilogue {
+  EPI_STORE = 0,        // C = acc
+  EPI_STORE_SQNORM = 1, // C = acc, partial[tile] = sum(acc^2) over the tile
+  EPI_SYRK_EMA = 2,     // packed upper triangle: C = beta*C + alpha*acc   (tiles tn >= tm only)
+  EPI_NEWTON_M = 3,     // C = acc (new M), C2 = acc*mp_scale + mp_diag*I, err = max|acc - I| over d x d
+};
+
+struct GemmProblem {
+  const float* A;
+  const float* B;
+  float* C;
+  float* C2;               // EPI_NEWTON_M: M_p output.  EPI_STORE_SQNORM: per-tile partial sums
+  unsigned int* err_bits;  // EPI_NEWTON_M: atomicMax target (bit pattern of a non-negative float)
+  const int* active;       // optional: skip the problem when *active == 0
+  long long lda, ldb, ldc;
+  int M, N, K;
+  int tiles_m, tiles_n;
+  int tile_begin;          // first logical tile id of this problem
+  int d;                   // EPI_NEWTON_M: true (unpadded) dimension
+  int a_vec, b_vec;        // operand may be read with 16-byte loads (pointer and ld aligned)
+};
+
+// Scalars shared by every problem of one launch.
+struct GemmScalars {
+  float a_div, b_div;      // operand is divided by this on load (1.0f = as stored)
+  float alpha, beta;       // EPI_SYRK_EMA: C = beta*C + alpha*acc
+  float mp_scale, mp_diag; // EPI_NEWTON_M: M_p = M*mp_scale + mp_diag*I
+};
+
+__device__ __forceinline__ float4 load4_guarded(const float* p, bool vec, int valid) {
+  // valid = number of in-range elements starting at p (clamped to [0,4]).
+  float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (valid >= 4 && vec) {
+    v = *reinterpret_cast<const float4*>(p);
+  } else {
+    if (valid > 0) v.x = p[0];
+    if (valid > 1) v.y = p[1];
+    if (valid > 2) v.z = p[2];
+    if (valid > 3) v.w = p[3];
+  }
+  return v;
+}
+
+// Fetch this thread's share of one 128 x 16 operand slab into registers.
+// K_CONTIG: the operand is k-contiguous in memory (A_MK or B_NK): thread reads 4 k's of one row.
+// otherwise the operand is row/col-contiguous for fixed k (A_KM or B_KN): 4 m's (or n's) of one k.
+template <bool K_CONTIG, bool EDGE>
+__device__ __forceinline__ void slab_load(const float* __restrict__ base, long long ld, int row0,
+                                          int rows, int k0, int K, bool vec, float4 (&r)[2]) {
+  const int t = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int idx = t + i * GEMM_THREADS;
+    if (K_CONTIG) {
+      const int row = idx >> 2, k = k0 + ((idx & 3) << 2);
+      const float* p = base + (long long)(row0 + row) * ld + k;
+      if (EDGE) {
+        const int valid = (row0 + row < rows) ? (K - k) : 0;
+        r[i] = load4_guarded(p, vec, valid);
+      } else {
+        r[i] = *reinterpret_cast<const float4*>(p);
+      }
+    } else {
+      const int k = k0 + (idx >> 5), row = (idx & 31) << 2;
+      const float* p = base + (long long)k * ld + row0 + row;
+      if (EDGE) {
+        const int valid = (k < K) ? (rows - (row0 + row)) : 0;
+        r[i] = load4_guarded(p, vec, valid);
+      } else {
+        r[i] = *reinterpret_cast<const float4*>(p);
+      }
+    }
+  }
+}
+
+template <bool K_CONTIG>
+__device__ __forceinline__ void slab_store(float* __restrict__ lds, const float4 (&r)[2]) {
+  const int t = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int idx = t + i * GEMM_THREADS;
+    if (K_CONTIG) {
+      const int row = idx >> 2, k = (idx & 3) << 2;
+      lds[(k + 0) * LDS_STRIDE + row] = r[i].x;
+      lds[(k + 1) * LDS_STRIDE + row] = r[i].y;
+      lds[(k + 2) * LDS_STRIDE + row] = r[i].z;
+      lds[(k + 3) * LDS_STRIDE + row] = r[i].w;
+    } else {
+      const int k = idx >> 5, row = (idx & 31) << 2;
+      *reinterpret_cast<float4*>(&lds[k * LDS_STRIDE + row]) = r[i];
+    }
+  }
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max_nan(float v) {
+  // max that propagates NaN (a NaN anywhere must end the Newton loop like torch.dist does)
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    float w = __shfl_xor(v, o, 64);
+    v = (v != v || w != w) ? __builtin_nanf("") : fmaxf(v, w);
+  }
+  return v;
+}
+
+template <int AL, int BL, int EPI, bool EDGE>
+__global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(
+    const GemmProblem* __restrict__ problems, int n_problems, int total_tiles, GemmScalars sc) {
+  __shared__ __attribute__((aligned(16))) float As[2][BK * LDS_STRIDE];
+  __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDS_STRIDE];
+  __shared__ float red[4];
+
+  // XCD-aware remap of the hardware workgroup id to a logical tile id.
+  const int per_xcd = (total_tiles + NUM_XCD - 1) / NUM_XCD;
+  const int logical = (blockIdx.x % NUM_XCD) * per_xcd + blockIdx.x / NUM_XCD;
+  if (logical >= total_tiles) return;
+
+  // Which problem owns this tile (tile_begin is ascending).
+  int lo = 0, hi = n_problems - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (problems[mid].tile_begin <= logical) lo = mid; else hi = mid - 1;
+  }
+  const GemmProblem& P = problems[lo];
+  if (P.active != nullptr && *P.active == 0) return;
+
+  int tm, tn;
+  {
+    int t = logical - P.tile_begin;
+    if (EPI == EPI_SYRK_EMA) {
+      // upper-triangular tile enumeration, row by row
+      tm = 0;
+      int rowlen = P.tiles_n;
+      while (t >= rowlen) { t -= rowlen; ++tm; --rowlen; }
+      tn = tm + t;
+    } else {
+      const int per_group = GROUP_ROWS * P.tiles_n;
+      const int g = t / per_group, r = t - g * per_group;
+      const int first = g * GROUP_ROWS;
+      const int gsz = min(P.tiles_m - first, GROUP_ROWS);
+      tm = first + r % gsz;
+      tn = r / gsz;
+    }
+  }
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int M = P.M, N = P.N, K = P.K;
+  const float* __restrict__ A = P.A;
+  const float* __restrict__ B = P.B;
+  const long long lda = P.lda, ldb = P.ldb;
+  const bool avec = P.a_vec != 0, bvec = P.b_vec != 0;
+  const float a_div = sc.a_div, b_div = sc.b_div;
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int l32 = lane & 31, h = lane >> 5;
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  float4 ra[2], rb[2];
+  const int slabs = (K + BK - 1) / BK;
+
+  slab_load<AL == A_MK, EDGE>(A, lda, m0, M, 0, K, avec, ra);
+  slab_load<BL == B_NK, EDGE>(B, ldb, n0, N, 0, K, bvec, rb);
+  if (a_div != 1.0f) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) { ra[i].x /= a_div; ra[i].y /= a_div; ra[i].z /= a_div; ra[i].w /= a_div; }
+  }
+  if (b_div != 1.0f) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) { rb[i].x /= b_div; rb[i].y /= b_div; rb[i].z /= b_div; rb[i].w /= b_div; }
+  }
+  slab_store<AL == A_MK>(As[0], ra);
+  slab_store<BL == B_NK>(Bs[0], rb);
+  __syncthreads();
+
+  for (int s = 0; s < slabs; ++s) {
+    const int cur = s & 1;
+    const bool more = (s + 1 < slabs);
+    if (more) {
+      slab_load<AL == A_MK, EDGE>(A, lda, m0, M, (s + 1) * BK, K, avec, ra);
+      slab_load<BL == B_NK, EDGE>(B, ldb, n0, N, (s + 1) * BK, K, bvec, rb);
+    }
+    const float* as = As[cur] + wm * 64 + l32;
+    const float* bs = Bs[cur] + wn * 64 + l32;
+#pragma unroll
+    for (int ks = 0; ks < BK / 2; ++ks) {
+      const int krow = (ks * 2 + h) * LDS_STRIDE;
+      const float a0 = as[krow], a1 = as[krow + 32];
+      const float b0 = bs[krow], b1 = bs[krow + 32];
+      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+      acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+      acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+      acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+    }
+    if (more) {
+      if (a_div != 1.0f) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) { ra[i].x /= a_div; ra[i].y /= a_div; ra[i].z /= a_div; ra[i].w /= a_div; }
+      }
+      if (b_div != 1.0f) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) { rb[i].x /= b_div; rb[i].y /= b_div; rb[i].z /= b_div; rb[i].w /= b_div; }
+      }
+      slab_store<AL == A_MK>(As[cur ^ 1], ra);
+      slab_store<BL == B_NK>(Bs[cur ^ 1], rb);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue -------------------------------------------------------------------
+  // accumulator element e of tile (i,j): row = 32*i + 8*(e/4) + 4*h + e%4, col = 32*j + l32
+  float local = 0.f;      // sum of squares or running max
+  bool local_nan = false;
+  float* __restrict__ C = P.C;
+  const long long ldc = P.ldc;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int col = n0 + wn * 64 + j * 32 + l32;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
+        const float v = acc[i][j][e];
+        if (EPI == EPI_STORE) {
+          if (!EDGE || (row < M && col < N)) C[(long long)row * ldc + col] = v;
+        } else if (EPI == EPI_STORE_SQNORM) {
+          if (!EDGE || (row < M && col < N)) {
+            C[(long long)row * ldc + col] = v;
+            local += v * v;
+          }
+        } else if (EPI == EPI_SYRK_EMA) {
+          // packed row-major upper triangle of an N x N matrix: (r,c), c >= r, lives at
+          // r*N - r*(r-1)/2 + (c - r)
+          if (row < M && col < N && col >= row) {
+            const long long off = (long long)row * N - ((long long)row * (row - 1)) / 2 + (col - row);
+            const float old = C[off];
+            C[off] = __fadd_rn(__fmul_rn(old, sc.beta), __fmul_rn(v, sc.alpha));
+          }
+        } else if (EPI == EPI_NEWTON_M) {
+          // operands are zero padded to the tile grid, so every (row, col) is in bounds
+          C[(long long)row * ldc + col] = v;
+          float mp = __fmul_rn(v, sc.mp_scale);
+          if (row == col && row < P.d) mp = __fadd_rn(mp, sc.mp_diag);
+          P.C2[(long long)row * ldc + col] = mp;
+          if (row < P.d && col < P.d) {
+            const float dv = fabsf(v - (row == col ? 1.0f : 0.0f));
+            if (dv != dv) local_nan = true;
+            local = fmaxf(local, dv);
+          }
+        }
+      }
+    }
+  }
+  if (EPI == EPI_STORE_SQNORM) {
+    local = wave_sum(local);
+    if (lane == 0) red[wave] = local;
+    __syncthreads();
+    if (threadIdx.x == 0) P.C2[tm * P.tiles_n + tn] = (red[0] + red[1]) + (red[2] + red[3]);
+  } else if (EPI == EPI_NEWTON_M) {
+    if (local_nan) local = __builtin_nanf("");
+    local = wave_max_nan(local);
+    if (lane == 0) {
+      // non-negative floats order like their bit patterns; a NaN pattern (0x7fc00000) is above +inf
+      atomicMax(P.err_bits, __float_as_uint(local != local ? __builtin_nanf("") : local));
+    }
+  }
+}
+
+}  // namespace sa

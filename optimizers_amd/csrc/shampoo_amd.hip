@@ -1,0 +1,1038 @@
+// libshampoo_amd.so: C ABI (include/shampoo_amd.h) over the gfx950 kernels in gemm.h and
+// elementwise.h.  Host side of the library: the ragged batched descriptor tables of a
+// parameter group ("plan"), the batched coupled-Newton driver, and per-phase HIP-event timing.
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "../../include/shampoo_amd.h"
+#include "elementwise.h"
+#include "gemm.h"
+
+using namespace sa;
+
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int code, const std::string& msg) {
+  g_err = msg;
+  return code;
+}
+
+#define HIPCHECK(expr)                                                                     \
+  do {                                                                                     \
+    hipError_t e__ = (expr);                                                               \
+    if (e__ != hipSuccess)                                                                 \
+      return fail(SA_ERR_HIP, std::string(#expr) + " failed: " + hipGetErrorString(e__)); \
+  } while (0)
+
+#define SACHECK(expr)             \
+  do {                            \
+    int r__ = (expr);             \
+    if (r__ != SA_OK) return r__; \
+  } while (0)
+
+inline long long round_up(long long x, long long a) { return (x + a - 1) / a * a; }
+
+// A host-built table mirrored on the device.  The host copy is pinned so the upload is a
+// true asynchronous copy; an event guards the pinned copy against being rewritten while a
+// previous upload may still be reading it.
+template <class T>
+struct Table {
+  T* host = nullptr;
+  T* dev = nullptr;
+  size_t cap = 0;
+  size_t n = 0;
+  hipEvent_t ev = nullptr;
+  bool pending = false;
+
+  int reserve(size_t m) {
+    if (m <= cap) return SA_OK;
+    SACHECK(wait());
+    size_t ncap = std::max<size_t>(m, cap * 2 + 16);
+    T* nh = nullptr;
+    T* nd = nullptr;
+    HIPCHECK(hipHostMalloc(reinterpret_cast<void**>(&nh), ncap * sizeof(T), hipHostMallocDefault));
+    HIPCHECK(hipMalloc(reinterpret_cast<void**>(&nd), ncap * sizeof(T)));
+    if (host) {
+      std::memcpy(nh, host, n * sizeof(T));
+      HIPCHECK(hipHostFree(host));
+    }
+    if (dev) HIPCHECK(hipFree(dev));
+    host = nh;
+    dev = nd;
+    cap = ncap;
+    return SA_OK;
+  }
+  int wait() {
+    if (pending) {
+      HIPCHECK(hipEventSynchronize(ev));
+      pending = false;
+    }
+    return SA_OK;
+  }
+  // start a rewrite of `m` entries
+  int begin(size_t m) {
+    SACHECK(wait());
+    SACHECK(reserve(m));
+    n = m;
+    return SA_OK;
+  }
+  int upload(hipStream_t s) {
+    if (n == 0) return SA_OK;
+    if (!ev) HIPCHECK(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+    HIPCHECK(hipMemcpyAsync(dev, host, n * sizeof(T), hipMemcpyHostToDevice, s));
+    HIPCHECK(hipEventRecord(ev, s));
+    pending = true;
+    return SA_OK;
+  }
+  void destroy() {
+    if (pending) (void)hipEventSynchronize(ev);
+    if (host) (void)hipHostFree(host);
+    if (dev) (void)hipFree(dev);
+    if (ev) (void)hipEventDestroy(ev);
+    host = nullptr; dev = nullptr; ev = nullptr; cap = n = 0; pending = false;
+  }
+};
+
+struct GemmTable {
+  Table<GemmProblem> t;
+  int total_tiles = 0;
+  bool aligned = true;  // every problem may use the unguarded loader
+  std::vector<GemmProblem> build;
+
+  void clear() { build.clear(); total_tiles = 0; aligned = true; }
+  void add(GemmProblem p, bool triangular) {
+    p.tiles_m = (p.M + BM - 1) / BM;
+    p.tiles_n = (p.N + BN - 1) / BN;
+    p.tile_begin = total_tiles;
+    total_tiles += triangular ? p.tiles_n * (p.tiles_n + 1) / 2 : p.tiles_m * p.tiles_n;
+    if (p.M % BM || p.N % BN || p.K % BK || !p.a_vec || !p.b_vec) aligned = false;
+    build.push_back(p);
+  }
+  int commit(hipStream_t s) {
+    SACHECK(t.begin(build.size()));
+    if (!build.empty()) std::memcpy(t.host, build.data(), build.size() * sizeof(GemmProblem));
+    return t.upload(s);
+  }
+};
+
+inline int vec_ok(const void* p, long long ld) { return ((reinterpret_cast<uintptr_t>(p) & 15) == 0 && (ld % 4) == 0) ? 1 : 0; }
+
+template <int AL, int BL, int EPI, bool EDGE>
+int launch_gemm(const GemmTable& g, GemmScalars sc, hipStream_t s) {
+  if (g.total_tiles == 0) return SA_OK;
+  const int per = (g.total_tiles + NUM_XCD - 1) / NUM_XCD;
+  hipLaunchKernelGGL((grouped_gemm_kernel<AL, BL, EPI, EDGE>), dim3(per * NUM_XCD), dim3(GEMM_THREADS), 0, s,
+                     g.t.dev, (int)g.t.n, g.total_tiles, sc);
+  HIPCHECK(hipGetLastError());
+  return SA_OK;
+}
+template <int AL, int BL, int EPI>
+int launch_gemm_auto(const GemmTable& g, GemmScalars sc, hipStream_t s) {
+  return g.aligned ? launch_gemm<AL, BL, EPI, false>(g, sc, s) : launch_gemm<AL, BL, EPI, true>(g, sc, s);
+}
+
+GemmScalars unit_scalars() { return GemmScalars{1.0f, 1.0f, 1.0f, 0.0f, 0.0f, 0.0f}; }
+
+// ---- phase timing -------------------------------------------------------------------------
+struct Phase {
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> spans;
+  size_t used = 0;
+  double work = 0.0;  // flops or bytes
+  int launches = 0;
+};
+bool g_profiling = false;
+std::map<std::string, Phase> g_phases;
+
+struct Span {
+  Phase* ph = nullptr;
+  hipStream_t s = nullptr;
+  hipEvent_t stop = nullptr;
+  Span(const char* name, hipStream_t st, double work, int launches, bool reset) {
+    if (!g_profiling) return;
+    ph = &g_phases[name];
+    if (reset) { ph->used = 0; ph->work = 0.0; ph->launches = 0; }
+    if (ph->used == ph->spans.size()) {
+      hipEvent_t a, b;
+      if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) { ph = nullptr; return; }
+      ph->spans.emplace_back(a, b);
+    }
+    s = st;
+    (void)hipEventRecord(ph->spans[ph->used].first, s);
+    stop = ph->spans[ph->used].second;
+    ph->used++;
+    ph->work += work;
+    ph->launches += launches;
+  }
+  ~Span() {
+    if (ph) (void)hipEventRecord(stop, s);
+  }
+};
+
+struct Factor {
+  int block, side, d, dpad, root;
+  float* factor;
+  float* inv;
+  long long dense_off;   // offset (floats) of this factor inside every dense array
+  long long norm_off;    // offset into the norm-partial array
+  int norm_chunks;
+};
+
+}  // namespace
+
+struct sa_plan {
+  int n_blocks = 0;
+  std::vector<sa_block_desc> blocks;
+  std::vector<float*> grads;
+  bool grads_bound = false;
+  bool tables_valid = false;
+  int table_mode = -1;  // 0: ghat from grad, 1: from filtered_grad, 2: from the beta3 temporary
+  std::vector<Factor> factors;
+  std::vector<int> block_factor[2];
+  std::vector<long long> elem_off;
+  std::vector<int> chunk_begin_all, ptile_begin_all;  // per block, over ALL blocks (fixed layout)
+  long long total_elems = 0, dense_total = 0, norm_partials_total = 0;
+  int total_chunks_all = 0, total_ptiles_all = 0;
+
+  // workspace carve-up
+  char* ws = nullptr;
+  long long ws_bytes = 0, ws_needed = 0;
+  long long off_inv_dense = 0, off_norms = 0, off_graft_partial = 0, off_ghat_partial = 0, off_ptile_partial = 0,
+            off_norm_partial = 0, off_scratch = 0, scratch_floats = 0;
+  bool inv_cache_valid = false;
+
+  // device tables
+  Table<BlockDev> t_blocks;
+  Table<ChunkRef> t_chunks;
+  Table<int> t_active_blocks;
+  GemmTable syrk0, syrk1, g1_store, g1_norm, g2_norm, g2g_norm;
+  GemmTable nt_a[2], nt_pow[8], nt_m[2];  // Newton: X/M_p^2 launch per parity, power chain, M update per parity
+  Table<SymFactor> t_sym;
+  Table<NormJob> t_normjobs;
+  Table<int> t_ids;
+  int n_active_blocks = 0;
+
+  // Newton control state (device) and pinned readback
+  unsigned int* d_err = nullptr;
+  int* d_active = nullptr;
+  int* d_iters = nullptr;
+  int* d_final_parity = nullptr;
+  float* d_final_err = nullptr;
+  int* d_flags = nullptr;
+  int* d_nactive = nullptr;
+  int* h_pinned = nullptr;  // 4 * F + 16 ints
+
+  float* f(long long off) const { return reinterpret_cast<float*>(ws) + off; }
+};
+
+namespace {
+
+void compute_layout(sa_plan* p) {
+  long long o = 0;
+  auto take = [&](long long n) { long long r = o; o += round_up(std::max<long long>(n, 1), 64); return r; };
+  p->off_inv_dense = take(p->dense_total);
+  p->off_norms = take(2LL * p->n_blocks);
+  p->off_graft_partial = take(p->total_chunks_all);
+  p->off_ghat_partial = take(p->total_chunks_all);
+  p->off_ptile_partial = take(p->total_ptiles_all);
+  p->off_norm_partial = take(p->norm_partials_total);
+  p->scratch_floats = std::max(8LL * p->dense_total, 3LL * round_up(p->total_elems, 64) + 192);
+  p->off_scratch = take(p->scratch_floats);
+  p->ws_needed = o * (long long)sizeof(float);
+}
+
+// dense array k (0..7) of the Newton scratch: X0 X1 M0 M1 Mp0 Mp1 S1 S2
+inline float* newton_buf(const sa_plan* p, int k, const Factor& F) {
+  return p->f(p->off_scratch + (long long)k * p->dense_total + F.dense_off);
+}
+enum { NB_X0 = 0, NB_X1 = 1, NB_M0 = 2, NB_M1 = 3, NB_MP0 = 4, NB_MP1 = 5, NB_S1 = 6, NB_S2 = 7 };
+
+inline float* tbuf(const sa_plan* p) { return p->f(p->off_scratch); }
+inline float* pbuf(const sa_plan* p) { return p->f(p->off_scratch + round_up(p->total_elems, 64) + 64); }
+inline float* ghbuf(const sa_plan* p) { return p->f(p->off_scratch + 2 * (round_up(p->total_elems, 64) + 64)); }
+
+int need_ws(const sa_plan* p) {
+  if (!p->ws) return fail(SA_ERR_WORKSPACE, "no workspace bound (sa_plan_bind_workspace)");
+  return SA_OK;
+}
+
+bool block_active(const sa_plan* p, int b) { return p->grads[b] != nullptr; }
+
+// Rebuild every table that depends on the bound gradients / mask / filtered-gradient mode.
+int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
+  SACHECK(need_ws(p));
+  const int nb = p->n_blocks;
+  // blocks
+  SACHECK(p->t_blocks.begin(nb));
+  std::vector<int> active;
+  std::vector<ChunkRef> chunks;
+  for (int b = 0; b < nb; ++b) {
+    const sa_block_desc& d = p->blocks[b];
+    BlockDev& B = p->t_blocks.host[b];
+    std::memset(&B, 0, sizeof(B));
+    B.param = d.param;
+    B.grad = p->grads[b];
+    B.filtered_grad = d.filtered_grad;
+    B.adagrad = d.adagrad;
+    B.momentum = d.momentum_buffer;
+    B.ld = d.ld;
+    B.rows = d.rows;
+    B.cols = d.cols;
+    const long long eo = p->elem_off[b];
+    B.ghat_tmp = (mode == 2) ? ghbuf(p) + eo : nullptr;
+    if (mode == 0) { B.ghat_src = B.grad; B.ghat_ld = d.ld; }
+    else if (mode == 1) { B.ghat_src = d.filtered_grad; B.ghat_ld = d.cols; }
+    else { B.ghat_src = ghbuf(p) + eo; B.ghat_ld = d.cols; }
+    const bool precond = p->block_factor[0][b] >= 0 || p->block_factor[1][b] >= 0;
+    B.p_is_ghat = precond ? 0 : 1;
+    if (precond) { B.p_src = pbuf(p) + eo; B.p_ld = d.cols; }
+    else { B.p_src = B.ghat_src; B.p_ld = B.ghat_ld; }
+    const bool contig = (d.ld == d.cols);
+    auto al = [](const void* q) { return q == nullptr || (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    const bool shape_ok = contig || (d.cols % 4 == 0 && d.ld % 4 == 0);
+    B.vec = (shape_ok && al(B.param) && al(B.grad) && al(B.filtered_grad) && al(B.adagrad) && al(B.momentum) &&
+             al(B.ghat_tmp)) ? 1 : 0;
+    const bool p_contig = (B.p_ld == d.cols);
+    B.p_vec = ((p_contig || (d.cols % 4 == 0 && B.p_ld % 4 == 0)) && al(B.p_src)) ? 1 : 0;
+    B.chunk_begin = B.chunk_end = 0;
+    B.ptile_begin = p->ptile_begin_all[b];
+    B.ptile_end = p->ptile_begin_all[b + 1];
+    if (block_active(p, b)) {
+      active.push_back(b);
+      B.chunk_begin = (int)chunks.size();
+      const long long n_el = (long long)d.rows * d.cols;
+      for (long long e = 0; e < n_el; e += EW_CHUNK) chunks.push_back(ChunkRef{b, (int)e});
+      B.chunk_end = (int)chunks.size();
+    }
+  }
+  SACHECK(p->t_blocks.upload(s));
+  SACHECK(p->t_chunks.begin(chunks.size()));
+  if (!chunks.empty()) std::memcpy(p->t_chunks.host, chunks.data(), chunks.size() * sizeof(ChunkRef));
+  SACHECK(p->t_chunks.upload(s));
+  SACHECK(p->t_active_blocks.begin(active.size()));
+  if (!active.empty()) std::memcpy(p->t_active_blocks.host, active.data(), active.size() * sizeof(int));
+  SACHECK(p->t_active_blocks.upload(s));
+  p->n_active_blocks = (int)active.size();
+
+  // factor-update tables
+  p->syrk0.clear();
+  p->syrk1.clear();
+  for (int b : active) {
+    const sa_block_desc& d = p->blocks[b];
+    const float* G = p->grads[b];
+    if (d.factor[0]) {  // L = G G^T  (rows x rows, K = cols)
+      GemmProblem q{};
+      q.A = G; q.B = G; q.C = d.factor[0];
+      q.lda = d.ld; q.ldb = d.ld; q.ldc = 0;
+      q.M = d.rows; q.N = d.rows; q.K = d.cols;
+      q.a_vec = q.b_vec = vec_ok(G, d.ld);
+      p->syrk0.add(q, true);
+    }
+    if (d.factor[1]) {  // R = G^T G  (cols x cols, K = rows)
+      GemmProblem q{};
+      q.A = G; q.B = G; q.C = d.factor[1];
+      q.lda = d.ld; q.ldb = d.ld; q.ldc = 0;
+      q.M = d.cols; q.N = d.cols; q.K = d.rows;
+      q.a_vec = q.b_vec = vec_ok(G, d.ld);
+      p->syrk1.add(q, true);
+    }
+  }
+  SACHECK(p->syrk0.commit(s));
+  SACHECK(p->syrk1.commit(s));
+
+  // preconditioning tables
+  p->g1_store.clear(); p->g1_norm.clear(); p->g2_norm.clear(); p->g2g_norm.clear();
+  for (int b : active) {
+    const sa_block_desc& d = p->blocks[b];
+    const BlockDev& B = p->t_blocks.host[b];
+    const int f0 = p->block_factor[0][b], f1 = p->block_factor[1][b];
+    const long long eo = p->elem_off[b];
+    float* part = p->f(p->off_ptile_partial) + p->ptile_begin_all[b];
+    if (f0 >= 0) {
+      const Factor& F = p->factors[f0];
+      GemmProblem q{};
+      q.A = p->f(p->off_inv_dense) + F.dense_off; q.lda = F.dpad; q.a_vec = 1;
+      q.B = B.ghat_src; q.ldb = B.ghat_ld; q.b_vec = vec_ok(B.ghat_src, B.ghat_ld);
+      q.M = d.rows; q.N = d.cols; q.K = d.rows;
+      q.ldc = d.cols;
+      if (f1 >= 0) { q.C = tbuf(p) + eo; p->g1_store.add(q, false); }
+      else { q.C = pbuf(p) + eo; q.C2 = part; p->g1_norm.add(q, false); }
+    }
+    if (f1 >= 0) {
+      const Factor& F = p->factors[f1];
+      GemmProblem q{};
+      q.B = p->f(p->off_inv_dense) + F.dense_off; q.ldb = F.dpad; q.b_vec = 1;
+      q.M = d.rows; q.N = d.cols; q.K = d.cols;
+      q.C = pbuf(p) + eo; q.ldc = d.cols; q.C2 = part;
+      if (f0 >= 0) {
+        q.A = tbuf(p) + eo; q.lda = d.cols; q.a_vec = vec_ok(q.A, q.lda);
+        p->g2_norm.add(q, false);
+      } else {
+        q.A = B.ghat_src; q.lda = B.ghat_ld; q.a_vec = vec_ok(q.A, q.lda);
+        p->g2g_norm.add(q, false);
+      }
+    }
+  }
+  SACHECK(p->g1_store.commit(s));
+  SACHECK(p->g1_norm.commit(s));
+  SACHECK(p->g2_norm.commit(s));
+  SACHECK(p->g2g_norm.commit(s));
+  p->tables_valid = true;
+  p->table_mode = mode;
+  return SA_OK;
+}
+
+int mode_of(const sa_step_scalars* s) {
+  if (s->beta1 == 0.0f) return 0;
+  return (s->beta3 == s->beta1) ? 1 : 2;
+}
+
+int ensure_tables(sa_plan* p, const sa_step_scalars* s, hipStream_t st) {
+  if (!p->grads_bound) return fail(SA_ERR_STATE, "gradients not bound (sa_plan_bind_gradients)");
+  const int mode = s ? mode_of(s) : (p->table_mode < 0 ? 1 : p->table_mode);
+  if (!p->tables_valid || p->table_mode != mode) return rebuild_tables(p, mode, st);
+  return SA_OK;
+}
+
+int validate_scalars(const sa_plan* p, const sa_step_scalars* s) {
+  if (!s) return fail(SA_ERR_INVALID, "step scalars are NULL");
+  for (int b = 0; b < p->n_blocks; ++b) {
+    const sa_block_desc& d = p->blocks[b];
+    if (s->beta1 != 0.0f && !d.filtered_grad) return fail(SA_ERR_INVALID, "beta1 != 0 needs filtered_grad state in every block");
+    if (s->graft_type == SA_GRAFT_ADAGRAD && !d.adagrad) return fail(SA_ERR_INVALID, "adagrad-family grafting needs adagrad state in every block");
+    if (s->momentum != 0.0f && !d.momentum_buffer) return fail(SA_ERR_INVALID, "momentum != 0 needs momentum_buffer state in every block");
+  }
+  if (!(s->bias_correction1 != 0.0f) || !(s->graft_bias_correction2 != 0.0f)) return fail(SA_ERR_INVALID, "bias corrections must be non-zero divisors");
+  return SA_OK;
+}
+
+// packed -> dense mirrored cache of every inverse root
+int refresh_inverse_cache(sa_plan* p, hipStream_t s) {
+  if (p->inv_cache_valid || p->factors.empty()) { p->inv_cache_valid = true; return SA_OK; }
+  const int F = (int)p->factors.size();
+  SACHECK(p->t_sym.begin(F));
+  int tiles = 0;
+  for (int i = 0; i < F; ++i) {
+    const Factor& f = p->factors[i];
+    SymFactor& S = p->t_sym.host[i];
+    std::memset(&S, 0, sizeof(S));
+    S.packed_in = f.inv;
+    S.dense_out[0] = p->f(p->off_inv_dense) + f.dense_off;
+    S.d = f.d; S.dpad = f.dpad; S.tiles = f.dpad / ST; S.root = f.root; S.enabled = 1;
+    S.tile_begin = tiles;
+    tiles += S.tiles * (S.tiles + 1) / 2;
+  }
+  SACHECK(p->t_sym.upload(s));
+  hipLaunchKernelGGL((sym_pass_kernel<SYM_UNPACK>), dim3(tiles), dim3(256), 0, s, p->t_sym.dev, F, 1.0f, 0.0f, 0.0f, 0.0f);
+  HIPCHECK(hipGetLastError());
+  p->inv_cache_valid = true;
+  return SA_OK;
+}
+
+}  // namespace
+
+// ============================================================================================
+// C ABI
+// ============================================================================================
+
+extern "C" {
+
+const char* sa_last_error(void) { return g_err.c_str(); }
+int32_t sa_abi_version(void) { return 1; }
+
+int32_t sa_set_profiling(int32_t enabled) {
+  g_profiling = enabled != 0;
+  return SA_OK;
+}
+
+double sa_phase_ms(const char* phase) {
+  auto it = g_phases.find(phase ? phase : "");
+  if (it == g_phases.end() || it->second.used == 0) return -1.0;
+  double total = 0.0;
+  for (size_t i = 0; i < it->second.used; ++i) {
+    float ms = 0.f;
+    if (hipEventSynchronize(it->second.spans[i].second) != hipSuccess) return -1.0;
+    if (hipEventElapsedTime(&ms, it->second.spans[i].first, it->second.spans[i].second) != hipSuccess) return -1.0;
+    total += ms;
+  }
+  return total;
+}
+double sa_phase_flops(const char* phase) {
+  auto it = g_phases.find(phase ? phase : "");
+  return it == g_phases.end() ? -1.0 : it->second.work;
+}
+int32_t sa_phase_launches(const char* phase) {
+  auto it = g_phases.find(phase ? phase : "");
+  return it == g_phases.end() ? -1 : it->second.launches;
+}
+
+int32_t sa_plan_create(const sa_block_desc* blocks, int32_t n_blocks, sa_plan** plan_out) {
+  if (!blocks || n_blocks <= 0 || !plan_out) return fail(SA_ERR_INVALID, "sa_plan_create: bad arguments");
+  sa_plan* p = new sa_plan();
+  p->n_blocks = n_blocks;
+  p->blocks.assign(blocks, blocks + n_blocks);
+  p->grads.assign(n_blocks, nullptr);
+  p->block_factor[0].assign(n_blocks, -1);
+  p->block_factor[1].assign(n_blocks, -1);
+  p->elem_off.resize(n_blocks);
+  p->chunk_begin_all.resize(n_blocks + 1);
+  p->ptile_begin_all.resize(n_blocks + 1);
+  long long eo = 0, dense = 0, normp = 0;
+  int chunks = 0, ptiles = 0;
+  for (int b = 0; b < n_blocks; ++b) {
+    const sa_block_desc& d = blocks[b];
+    if (d.rows <= 0 || d.cols <= 0 || !d.param || d.ld < d.cols) {
+      delete p;
+      return fail(SA_ERR_INVALID, "sa_plan_create: block " + std::to_string(b) + " has a bad shape, stride or NULL param");
+    }
+    if ((long long)d.rows * d.cols >= (1LL << 31)) {
+      delete p;
+      return fail(SA_ERR_UNSUPPORTED, "sa_plan_create: block with 2^31 or more elements");
+    }
+    p->elem_off[b] = eo;
+    eo += round_up((long long)d.rows * d.cols, 64);
+    p->chunk_begin_all[b] = chunks;
+    chunks += (int)(((long long)d.rows * d.cols + EW_CHUNK - 1) / EW_CHUNK);
+    p->ptile_begin_all[b] = ptiles;
+    ptiles += ((d.rows + BM - 1) / BM) * ((d.cols + BN - 1) / BN);
+    for (int side = 0; side < 2; ++side) {
+      if (!d.factor[side]) continue;
+      if (!d.inv_factor[side] || d.root[side] < 1) {
+        delete p;
+        return fail(SA_ERR_INVALID, "sa_plan_create: factor without inverse storage or with root < 1");
+      }
+      Factor f{};
+      f.block = b; f.side = side;
+      f.d = side == 0 ? d.rows : d.cols;
+      f.dpad = (int)round_up(f.d, BM);
+      f.root = d.root[side];
+      f.factor = d.factor[side];
+      f.inv = d.inv_factor[side];
+      f.dense_off = dense;
+      dense += (long long)f.dpad * f.dpad;
+      f.norm_off = normp;
+      f.norm_chunks = (int)(((long long)f.d * (f.d + 1) / 2 + NORM_CHUNK - 1) / NORM_CHUNK);
+      normp += f.norm_chunks;
+      p->block_factor[side][b] = (int)p->factors.size();
+      p->factors.push_back(f);
+    }
+  }
+  p->chunk_begin_all[n_blocks] = chunks;
+  p->ptile_begin_all[n_blocks] = ptiles;
+  p->total_elems = eo;
+  p->dense_total = dense;
+  p->norm_partials_total = normp;
+  p->total_chunks_all = chunks;
+  p->total_ptiles_all = ptiles;
+  compute_layout(p);
+  const size_t F = std::max<size_t>(p->factors.size(), 1);
+  auto dm = [&](void** q, size_t bytes) { return hipMalloc(q, bytes); };
+  if (dm((void**)&p->d_err, F * 4) != hipSuccess || dm((void**)&p->d_active, F * 4) != hipSuccess ||
+      dm((void**)&p->d_iters, F * 4) != hipSuccess || dm((void**)&p->d_final_parity, F * 4) != hipSuccess ||
+      dm((void**)&p->d_final_err, F * 4) != hipSuccess || dm((void**)&p->d_flags, F * 4) != hipSuccess ||
+      dm((void**)&p->d_nactive, 64) != hipSuccess ||
+      hipHostMalloc((void**)&p->h_pinned, (4 * F + 16) * sizeof(int), hipHostMallocDefault) != hipSuccess) {
+    sa_plan_destroy(p);
+    return fail(SA_ERR_HIP, "sa_plan_create: device allocation of control arrays failed");
+  }
+  *plan_out = p;
+  return SA_OK;
+}
+
+void sa_plan_destroy(sa_plan* p) {
+  if (!p) return;
+  p->t_blocks.destroy(); p->t_chunks.destroy(); p->t_active_blocks.destroy();
+  for (GemmTable* g : {&p->syrk0, &p->syrk1, &p->g1_store, &p->g1_norm, &p->g2_norm, &p->g2g_norm, &p->nt_a[0],
+                       &p->nt_a[1], &p->nt_m[0], &p->nt_m[1]})
+    g->t.destroy();
+  for (auto& g : p->nt_pow) g.t.destroy();
+  p->t_sym.destroy(); p->t_normjobs.destroy(); p->t_ids.destroy();
+  for (void* q : {(void*)p->d_err, (void*)p->d_active, (void*)p->d_iters, (void*)p->d_final_parity,
+                  (void*)p->d_final_err, (void*)p->d_flags, (void*)p->d_nactive})
+    if (q) (void)hipFree(q);
+  if (p->h_pinned) (void)hipHostFree(p->h_pinned);
+  delete p;
+}
+
+int64_t sa_plan_workspace_bytes(const sa_plan* p) { return p ? p->ws_needed : 0; }
+
+int32_t sa_plan_bind_workspace(sa_plan* p, void* workspace, int64_t bytes) {
+  if (!p || !workspace) return fail(SA_ERR_INVALID, "sa_plan_bind_workspace: NULL argument");
+  if (bytes < p->ws_needed) return fail(SA_ERR_WORKSPACE, "workspace too small: need " + std::to_string(p->ws_needed) + " bytes");
+  if (reinterpret_cast<uintptr_t>(workspace) & 255) return fail(SA_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+  p->ws = static_cast<char*>(workspace);
+  p->ws_bytes = bytes;
+  p->inv_cache_valid = false;
+  p->tables_valid = false;
+  return SA_OK;
+}
+
+int32_t sa_plan_num_factors(const sa_plan* p) { return p ? (int32_t)p->factors.size() : 0; }
+
+int32_t sa_plan_invalidate_inverse_cache(sa_plan* p) {
+  if (!p) return fail(SA_ERR_INVALID, "NULL plan");
+  p->inv_cache_valid = false;
+  return SA_OK;
+}
+
+int32_t sa_plan_bind_gradients(sa_plan* p, float* const* grads, void* stream) {
+  if (!p || !grads) return fail(SA_ERR_INVALID, "sa_plan_bind_gradients: NULL argument");
+  (void)stream;
+  bool changed = !p->grads_bound;
+  for (int b = 0; b < p->n_blocks; ++b) {
+    if (p->grads[b] != grads[b]) { p->grads[b] = grads[b]; changed = true; }
+  }
+  p->grads_bound = true;
+  if (changed) p->tables_valid = false;
+  return SA_OK;
+}
+
+int32_t sa_add_l2_regularization(sa_plan* p, float weight_decay, void* stream) {
+  if (!p) return fail(SA_ERR_INVALID, "NULL plan");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SACHECK(ensure_tables(p, nullptr, s));
+  if (p->t_chunks.n == 0) return SA_OK;
+  hipLaunchKernelGGL(l2_kernel, dim3((unsigned)p->t_chunks.n), dim3(EW_THREADS), 0, s, p->t_blocks.dev, p->t_chunks.dev, weight_decay);
+  HIPCHECK(hipGetLastError());
+  return SA_OK;
+}
+
+int32_t sa_update_factor_matrices(sa_plan* p, float beta2, float weighting_factor, void* stream) {
+  if (!p) return fail(SA_ERR_INVALID, "NULL plan");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SACHECK(ensure_tables(p, nullptr, s));
+  GemmScalars sc = unit_scalars();
+  sc.alpha = weighting_factor;
+  sc.beta = beta2;
+  double flops = 0.0;
+  for (const GemmTable* g : {&p->syrk0, &p->syrk1})
+    for (const GemmProblem& q : g->build) flops += (double)q.N * q.N * q.K;  // symmetric half: d^2 k
+  int launches = (p->syrk0.total_tiles ? 1 : 0) + (p->syrk1.total_tiles ? 1 : 0);
+  Span span("syrk", s, flops, launches, true);
+  SACHECK((launch_gemm_auto<A_MK, B_NK, EPI_SYRK_EMA>(p->syrk0, sc, s)));
+  SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_SYRK_EMA>(p->syrk1, sc, s)));
+  return SA_OK;
+}
+
+int32_t sa_update_grafting_and_filtered_grad(sa_plan* p, const sa_step_scalars* sc, void* stream) {
+  if (!p) return fail(SA_ERR_INVALID, "NULL plan");
+  SACHECK(validate_scalars(p, sc));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SACHECK(ensure_tables(p, sc, s));
+  if (p->t_chunks.n == 0) return SA_OK;
+  double bytes = 0.0;
+  for (int b = 0; b < p->n_blocks; ++b)
+    if (block_active(p, b)) {
+      const sa_block_desc& d = p->blocks[b];
+      const double n = (double)d.rows * d.cols;
+      bytes += 4.0 * n * (1 + (d.filtered_grad && sc->beta1 != 0.0f ? 2 : 0) + (d.adagrad && sc->graft_type == SA_GRAFT_ADAGRAD ? 2 : 0));
+    }
+  Span span("grafting", s, bytes, 1, true);
+  hipLaunchKernelGGL((grafting_kernel<0>), dim3((unsigned)p->t_chunks.n), dim3(EW_THREADS), 0, s, p->t_blocks.dev,
+                     p->t_chunks.dev, *sc, p->f(p->off_graft_partial), p->f(p->off_ghat_partial));
+  HIPCHECK(hipGetLastError());
+  return SA_OK;
+}
+
+int32_t sa_grafting_only_step(sa_plan* p, const sa_step_scalars* sc, void* stream) {
+  if (!p) return fail(SA_ERR_INVALID, "NULL plan");
+  SACHECK(validate_scalars(p, sc));
+  if (sc->graft_type == SA_GRAFT_NONE) return fail(SA_ERR_INVALID, "sa_grafting_only_step needs a grafting method");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SACHECK(ensure_tables(p, sc, s));
+  if (p->t_chunks.n == 0) return SA_OK;
+  hipLaunchKernelGGL((grafting_kernel<1>), dim3((unsigned)p->t_chunks.n), dim3(EW_THREADS), 0, s, p->t_blocks.dev,
+                     p->t_chunks.dev, *sc, p->f(p->off_graft_partial), p->f(p->off_ghat_partial));
+  HIPCHECK(hipGetLastError());
+  return SA_OK;
+}
+
+int32_t sa_precondition(sa_plan* p, const sa_step_scalars* sc, void* stream) {
+  if (!p) return fail(SA_ERR_INVALID, "NULL plan");
+  SACHECK(validate_scalars(p, sc));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SACHECK(ensure_tables(p, sc, s));
+  SACHECK(refresh_inverse_cache(p, s));
+  double flops = 0.0;
+  int launches = 0;
+  for (const GemmTable* g : {&p->g1_store, &p->g1_norm, &p->g2_norm, &p->g2g_norm}) {
+    for (const GemmProblem& q : g->build) flops += 2.0 * q.M * q.N * q.K;
+    launches += g->total_tiles ? 1 : 0;
+  }
+  {
+    Span span("precondition_gemm", s, flops, launches, true);
+    GemmScalars a = unit_scalars();
+    a.b_div = sc->bias_correction1;
+    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE>(p->g1_store, a, s)));
+    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE_SQNORM>(p->g1_norm, a, s)));
+    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE_SQNORM>(p->g2_norm, unit_scalars(), s)));
+    GemmScalars c = unit_scalars();
+    c.a_div = sc->bias_correction1;
+    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE_SQNORM>(p->g2g_norm, c, s)));
+  }
+  if (p->n_active_blocks) {
+    hipLaunchKernelGGL(reduce_norms_kernel, dim3(p->n_active_blocks), dim3(EW_THREADS), 0, s, p->t_blocks.dev,
+                       p->t_active_blocks.dev, p->n_blocks, p->f(p->off_graft_partial), p->f(p->off_ghat_partial),
+                       p->f(p->off_ptile_partial), p->f(p->off_norms));
+    HIPCHECK(hipGetLastError());
+  }
+  return SA_OK;
+}
+
+int32_t sa_apply_update(sa_plan* p, const sa_step_scalars* sc, void* stream) {
+  if (!p) return fail(SA_ERR_INVALID, "NULL plan");
+  SACHECK(validate_scalars(p, sc));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SACHECK(ensure_tables(p, sc, s));
+  if (p->t_chunks.n == 0) return SA_OK;
+  double bytes = 0.0;
+  for (int b = 0; b < p->n_blocks; ++b)
+    if (block_active(p, b)) {
+      const sa_block_desc& d = p->blocks[b];
+      bytes += 4.0 * (double)d.rows * d.cols * (3 + (d.momentum_buffer && sc->momentum != 0.0f ? 2 : 0));
+    }
+  Span span("apply", s, bytes, 1, true);
+  hipLaunchKernelGGL(apply_kernel, dim3((unsigned)p->t_chunks.n), dim3(EW_THREADS), 0, s, p->t_blocks.dev,
+                     p->t_chunks.dev, *sc, p->n_blocks, p->f(p->off_norms));
+  HIPCHECK(hipGetLastError());
+  return SA_OK;
+}
+
+int32_t sa_plan_read_norms(sa_plan* p, float* graft_sq, float* precond_sq, void* stream) {
+  if (!p || !graft_sq || !precond_sq) return fail(SA_ERR_INVALID, "NULL argument");
+  SACHECK(need_ws(p));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  std::vector<float> tmp(2 * p->n_blocks);
+  HIPCHECK(hipMemcpyAsync(tmp.data(), p->f(p->off_norms), tmp.size() * sizeof(float), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipStreamSynchronize(s));
+  std::memcpy(graft_sq, tmp.data(), p->n_blocks * sizeof(float));
+  std::memcpy(precond_sq, tmp.data() + p->n_blocks, p->n_blocks * sizeof(float));
+  return SA_OK;
+}
+
+int32_t sa_plan_read_preconditioned(sa_plan* p, int32_t block, float* out, void* stream) {
+  if (!p || !out || block < 0 || block >= p->n_blocks) return fail(SA_ERR_INVALID, "bad argument");
+  SACHECK(need_ws(p));
+  if (!p->tables_valid) return fail(SA_ERR_STATE, "no step has run");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const BlockDev& B = p->t_blocks.host[block];
+  hipLaunchKernelGGL(copy_strided_kernel, dim3(256), dim3(256), 0, s, B.p_src, B.p_ld, out, B.rows, B.cols);
+  HIPCHECK(hipGetLastError());
+  return SA_OK;
+}
+
+// --------------------------------------------------------------------------------------------
+// Batched coupled inverse Newton
+// --------------------------------------------------------------------------------------------
+
+static int newton_batch(sa_plan* p, const std::vector<int>& ids, int root, float eps, float bc2, int max_iter, float tol,
+                        hipStream_t s, double* flops_acc, int* launches_acc) {
+  const int n = (int)ids.size();
+  if (n == 0) return SA_OK;
+  // torch.linalg.matrix_power(M_p, root): squarings (and one extra product for root 3)
+  int squarings = 0;
+  bool cube = false;
+  if (root == 3) { squarings = 1; cube = true; }
+  else {
+    int r = root;
+    while (r > 1) {
+      if (r & 1) return fail(SA_ERR_UNSUPPORTED, "coupled Newton is built for roots 1, 2, 3 and powers of two; got " + std::to_string(root));
+      r >>= 1;
+      ++squarings;
+    }
+  }
+  if (std::max(squarings - 1, 0) + (cube ? 1 : 0) > 4) return fail(SA_ERR_UNSUPPORTED, "root too large for the power chain");
+  const float alpha = (float)(-1.0 / root);          // M.mul(alpha)
+  const float one_minus_alpha = (float)(1.0 - (-1.0 / root));  // .add_(I, alpha = 1 - alpha)
+
+  // ---- init: M0, Mp0, X0, err --------------------------------------------------------------
+  SACHECK(p->t_ids.begin(n));
+  std::memcpy(p->t_ids.host, ids.data(), n * sizeof(int));
+  SACHECK(p->t_ids.upload(s));
+  SACHECK(p->t_sym.begin(n));
+  int sym_tiles = 0;
+  for (int i = 0; i < n; ++i) {
+    const Factor& f = p->factors[ids[i]];
+    SymFactor& S = p->t_sym.host[i];
+    std::memset(&S, 0, sizeof(S));
+    S.packed_in = f.factor;
+    S.dense_out[0] = newton_buf(p, NB_M0, f);
+    S.dense_out[1] = newton_buf(p, NB_MP0, f);
+    S.dense_out[2] = newton_buf(p, NB_X0, f);
+    S.err_bits = p->d_err + ids[i];
+    S.norm_partial = p->f(p->off_norm_partial) + f.norm_off;
+    S.n_norm_partial = f.norm_chunks;
+    S.d = f.d; S.dpad = f.dpad; S.tiles = f.dpad / ST; S.root = root; S.enabled = 1;
+    S.tile_begin = sym_tiles;
+    sym_tiles += S.tiles * (S.tiles + 1) / 2;
+  }
+  SACHECK(p->t_sym.upload(s));
+  hipLaunchKernelGGL((sym_pass_kernel<SYM_NEWTON_INIT>), dim3(sym_tiles), dim3(256), 0, s, p->t_sym.dev, n, bc2, eps,
+                     alpha, one_minus_alpha);
+  HIPCHECK(hipGetLastError());
+
+  // ---- GEMM tables -------------------------------------------------------------------------
+  for (int par = 0; par < 2; ++par) { p->nt_a[par].clear(); p->nt_m[par].clear(); }
+  for (int k = 0; k < 8; ++k) p->nt_pow[k].clear();
+  auto prob = [&](const Factor& f, const float* A, const float* B, float* C) {
+    GemmProblem q{};
+    q.A = A; q.B = B; q.C = C;
+    q.lda = q.ldb = q.ldc = f.dpad;
+    q.M = q.N = q.K = f.dpad;
+    q.d = f.d;
+    q.a_vec = q.b_vec = 1;
+    q.active = p->d_active + (&f - p->factors.data());
+    return q;
+  };
+  for (int i = 0; i < n; ++i) {
+    const Factor& f = p->factors[ids[i]];
+    // buffer that finally holds M_p^root (depends only on the chain length)
+    const float* power = nullptr;
+    for (int par = 0; par < 2; ++par) {
+      const float* X = newton_buf(p, par ? NB_X1 : NB_X0, f);
+      float* Xn = newton_buf(p, par ? NB_X0 : NB_X1, f);
+      const float* Mp = newton_buf(p, par ? NB_MP1 : NB_MP0, f);
+      float* Mpn = newton_buf(p, par ? NB_MP0 : NB_MP1, f);
+      const float* M = newton_buf(p, par ? NB_M1 : NB_M0, f);
+      float* Mn = newton_buf(p, par ? NB_M0 : NB_M1, f);
+      float* S1 = newton_buf(p, NB_S1, f);
+      float* S2 = newton_buf(p, NB_S2, f);
+      // launch A: X <- X M_p, and the first squaring if the root needs one
+      p->nt_a[par].add(prob(f, X, Mp, Xn), false);
+      if (squarings >= 1) p->nt_a[par].add(prob(f, Mp, Mp, S1), false);
+      // remaining chain reads only S1/S2/Mp of this parity; build it for parity-specific Mp when cube
+      const float* cur = (squarings >= 1) ? S1 : Mp;
+      int slot = par * 4;  // nt_pow[0..3] parity 0, [4..7] parity 1
+      float* pong[2] = {S2, S1};
+      int which = 0;
+      for (int q = 1; q < squarings; ++q) {
+        p->nt_pow[slot++].add(prob(f, cur, cur, pong[which]), false);
+        cur = pong[which];
+        which ^= 1;
+      }
+      if (cube) {
+        p->nt_pow[slot++].add(prob(f, cur, Mp, pong[which]), false);
+        cur = pong[which];
+      }
+      power = cur;
+      GemmProblem m = prob(f, power, M, Mn);
+      m.C2 = Mpn;
+      m.err_bits = p->d_err + ids[i];
+      p->nt_m[par].add(m, false);
+    }
+  }
+  for (int par = 0; par < 2; ++par) { SACHECK(p->nt_a[par].commit(s)); SACHECK(p->nt_m[par].commit(s)); }
+  for (int k = 0; k < 8; ++k) SACHECK(p->nt_pow[k].commit(s));
+
+  NewtonCtl ctl{p->d_err, p->d_active, p->d_iters, p->d_final_parity, p->d_final_err};
+  int parity = 0;
+  hipLaunchKernelGGL(newton_control_kernel, dim3(1), dim3(256), 0, s, ctl, p->t_ids.dev, n, tol, max_iter, parity, p->d_nactive);
+  HIPCHECK(hipGetLastError());
+  int* h_active = p->h_pinned;  // F ints
+  const int Fall = (int)p->factors.size();
+  HIPCHECK(hipMemcpyAsync(h_active, p->d_active, Fall * sizeof(int), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipStreamSynchronize(s));
+  GemmScalars unit = unit_scalars();
+  GemmScalars msc = unit_scalars();
+  msc.mp_scale = alpha;
+  msc.mp_diag = one_minus_alpha;
+  const int gemms_per_iter = 1 + squarings + (cube ? 1 : 0) + 1;
+  for (int it = 0; it < max_iter; ++it) {
+    double flops = 0.0;
+    int live = 0;
+    for (int i = 0; i < n; ++i)
+      if (h_active[ids[i]]) { const double d = p->factors[ids[i]].d; flops += 2.0 * d * d * d * gemms_per_iter; ++live; }
+    if (!live) break;
+    {
+      int nl = 2;
+      for (int k = 0; k < 4; ++k) nl += p->nt_pow[parity * 4 + k].total_tiles ? 1 : 0;
+      Span span("newton_gemm", s, flops, nl, false);
+      SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false>(p->nt_a[parity], unit, s)));
+      for (int k = 0; k < 4; ++k) SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false>(p->nt_pow[parity * 4 + k], unit, s)));
+      SACHECK((launch_gemm<A_MK, B_KN, EPI_NEWTON_M, false>(p->nt_m[parity], msc, s)));
+      *flops_acc += flops;
+      *launches_acc += nl;
+    }
+    parity ^= 1;
+    hipLaunchKernelGGL(newton_control_kernel, dim3(1), dim3(256), 0, s, ctl, p->t_ids.dev, n, tol, max_iter, parity, p->d_nactive);
+    HIPCHECK(hipGetLastError());
+    HIPCHECK(hipMemcpyAsync(h_active, p->d_active, Fall * sizeof(int), hipMemcpyDeviceToHost, s));
+    HIPCHECK(hipStreamSynchronize(s));
+  }
+  return SA_OK;
+}
+
+int32_t sa_compute_root_inverses_newton(sa_plan* p, float bias_correction2, float epsilon, int32_t max_iterations,
+                                        float tolerance, int32_t* iterations_out, int32_t* status_out, void* stream) {
+  if (!p || !iterations_out || !status_out) return fail(SA_ERR_INVALID, "sa_compute_root_inverses_newton: NULL argument");
+  if (!(bias_correction2 != 0.0f) || max_iterations < 0) return fail(SA_ERR_INVALID, "bad bias correction or max_iterations");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SACHECK(ensure_tables(p, nullptr, s));
+  const int F = (int)p->factors.size();
+  if (F == 0) return SA_OK;
+  if (g_profiling) { Phase& ph = g_phases["newton_gemm"]; ph.used = 0; ph.work = 0.0; ph.launches = 0; }
+
+  // factors of masked blocks are left alone (shampoo_preconditioner_list.py:1426)
+  std::vector<int> todo;
+  for (int i = 0; i < F; ++i) {
+    iterations_out[i] = 0;
+    status_out[i] = SA_FACTOR_SKIPPED;
+    if (block_active(p, p->factors[i].block)) todo.push_back(i);
+  }
+  if (todo.empty()) return SA_OK;
+  // factors that are not recomputed below must keep a valid dense copy of their stored inverse
+  SACHECK(refresh_inverse_cache(p, s));
+
+  HIPCHECK(hipMemsetAsync(p->d_flags, 0, F * sizeof(int), s));
+  HIPCHECK(hipMemsetAsync(p->d_err, 0, F * sizeof(int), s));
+  HIPCHECK(hipMemsetAsync(p->d_iters, 0, F * sizeof(int), s));
+  HIPCHECK(hipMemsetAsync(p->d_active, 0, F * sizeof(int), s));
+  HIPCHECK(hipMemsetAsync(p->d_final_parity, 0, F * sizeof(int), s));
+
+  // 1. Frobenius norms of the ridged, bias-corrected factors + finiteness of the input
+  SACHECK(p->t_normjobs.begin(todo.size()));
+  int chunks = 0;
+  for (size_t i = 0; i < todo.size(); ++i) {
+    const Factor& f = p->factors[todo[i]];
+    NormJob& J = p->t_normjobs.host[i];
+    std::memset(&J, 0, sizeof(J));
+    J.src = f.factor;
+    J.partial = p->f(p->off_norm_partial) + f.norm_off;
+    J.nonfinite = p->d_flags + todo[i];
+    J.d = f.d; J.dpad = f.dpad; J.dense = 0;
+    J.chunk_begin = chunks;
+    J.n_chunks = f.norm_chunks;
+    J.enabled = 1;
+    chunks += f.norm_chunks;
+  }
+  SACHECK(p->t_normjobs.upload(s));
+  hipLaunchKernelGGL((factor_norm_kernel<false>), dim3(chunks), dim3(256), 0, s, p->t_normjobs.dev, (int)todo.size(),
+                     bias_correction2, epsilon);
+  HIPCHECK(hipGetLastError());
+  int* h_flags = p->h_pinned + F;
+  HIPCHECK(hipMemcpyAsync(h_flags, p->d_flags, F * sizeof(int), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipStreamSynchronize(s));
+  // the reference walks factors in order and raises at the first non-finite one
+  size_t limit = todo.size();
+  for (size_t i = 0; i < todo.size(); ++i)
+    if (h_flags[todo[i]]) { status_out[todo[i]] = SA_FACTOR_INPUT_NONFINITE; limit = i; break; }
+  todo.resize(limit);
+  if (todo.empty()) return SA_OK;
+
+  // 2. iterate, one batch per distinct root
+  std::vector<int> ones(F, 0);
+  for (int i : todo) ones[i] = 1;
+  HIPCHECK(hipMemcpyAsync(p->d_active, ones.data(), F * sizeof(int), hipMemcpyHostToDevice, s));
+  HIPCHECK(hipStreamSynchronize(s));
+  std::map<int, std::vector<int>> by_root;
+  for (int i : todo) by_root[p->factors[i].root].push_back(i);
+  double flops = 0.0;
+  int launches = 0;
+  for (auto& kv : by_root)
+    SACHECK(newton_batch(p, kv.second, kv.first, epsilon, bias_correction2, max_iterations, tolerance, s, &flops, &launches));
+
+  // 3. read back iteration counts, final errors, parities
+  int* h_iters = p->h_pinned;
+  int* h_par = p->h_pinned + F;
+  float* h_err = reinterpret_cast<float*>(p->h_pinned + 2 * F);
+  int* h_bad = p->h_pinned + 3 * F;
+  HIPCHECK(hipMemcpyAsync(h_iters, p->d_iters, F * sizeof(int), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipMemcpyAsync(h_par, p->d_final_parity, F * sizeof(int), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipMemcpyAsync(h_err, p->d_final_err, F * sizeof(float), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipStreamSynchronize(s));
+
+  // 4. finiteness of every result
+  HIPCHECK(hipMemsetAsync(p->d_flags, 0, F * sizeof(int), s));
+  SACHECK(p->t_normjobs.begin(todo.size()));
+  chunks = 0;
+  for (size_t i = 0; i < todo.size(); ++i) {
+    const Factor& f = p->factors[todo[i]];
+    NormJob& J = p->t_normjobs.host[i];
+    std::memset(&J, 0, sizeof(J));
+    J.src = newton_buf(p, h_par[todo[i]] ? NB_X1 : NB_X0, f);
+    J.partial = nullptr;
+    J.nonfinite = p->d_flags + todo[i];
+    J.d = f.d; J.dpad = f.dpad; J.dense = 1;
+    J.chunk_begin = chunks;
+    J.n_chunks = (int)(((long long)f.d * f.d + NORM_CHUNK - 1) / NORM_CHUNK);
+    J.enabled = 1;
+    chunks += J.n_chunks;
+  }
+  SACHECK(p->t_normjobs.upload(s));
+  hipLaunchKernelGGL((factor_norm_kernel<true>), dim3(chunks), dim3(256), 0, s, p->t_normjobs.dev, (int)todo.size(), 1.0f, 0.0f);
+  HIPCHECK(hipGetLastError());
+  HIPCHECK(hipMemcpyAsync(h_bad, p->d_flags, F * sizeof(int), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipStreamSynchronize(s));
+
+  // 5. commit the results that precede the first non-finite one
+  size_t ok = todo.size();
+  for (size_t i = 0; i < todo.size(); ++i) {
+    const int fi = todo[i];
+    iterations_out[fi] = h_iters[fi];
+    if (h_bad[fi]) { status_out[fi] = SA_FACTOR_RESULT_NONFINITE; ok = i; break; }
+    status_out[fi] = (h_err[fi] <= tolerance) ? SA_FACTOR_OK : SA_FACTOR_NOT_CONVERGED;
+  }
+  for (size_t i = ok + 1; i < todo.size(); ++i) iterations_out[todo[i]] = h_iters[todo[i]];
+  if (ok > 0) {
+    SACHECK(p->t_sym.begin(ok));
+    int tiles = 0;
+    for (size_t i = 0; i < ok; ++i) {
+      const Factor& f = p->factors[todo[i]];
+      SymFactor& S = p->t_sym.host[i];
+      std::memset(&S, 0, sizeof(S));
+      S.dense_in = newton_buf(p, h_par[todo[i]] ? NB_X1 : NB_X0, f);
+      S.packed_out = f.inv;
+      S.dense_out[0] = p->f(p->off_inv_dense) + f.dense_off;
+      S.d = f.d; S.dpad = f.dpad; S.tiles = f.dpad / ST; S.root = f.root; S.enabled = 1;
+      S.tile_begin = tiles;
+      tiles += S.tiles * (S.tiles + 1) / 2;
+    }
+    SACHECK(p->t_sym.upload(s));
+    hipLaunchKernelGGL((sym_pass_kernel<SYM_COMMIT>), dim3(tiles), dim3(256), 0, s, p->t_sym.dev, (int)ok, 1.0f, 0.0f, 0.0f, 0.0f);
+    HIPCHECK(hipGetLastError());
+    HIPCHECK(hipStreamSynchronize(s));
+  }
+  return SA_OK;
+}
+
+// --------------------------------------------------------------------------------------------
+// Single GEMM (tests, microbenchmarks)
+// --------------------------------------------------------------------------------------------
+
+static GemmTable g_test_table;
+
+int32_t sa_gemm_f32(const float* A, const float* B, float* C, int32_t M, int32_t N, int32_t K, int64_t lda, int64_t ldb,
+                    int64_t ldc, int32_t a_layout, int32_t b_layout, int32_t batch, int64_t stride_a, int64_t stride_b,
+                    int64_t stride_c, void* stream) {
+  if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0 || batch <= 0) return fail(SA_ERR_INVALID, "sa_gemm_f32: bad arguments");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  g_test_table.clear();
+  for (int i = 0; i < batch; ++i) {
+    GemmProblem q{};
+    q.A = A + i * stride_a; q.B = B + i * stride_b; q.C = C + i * stride_c;
+    q.lda = lda; q.ldb = ldb; q.ldc = ldc;
+    q.M = M; q.N = N; q.K = K;
+    q.a_vec = vec_ok(q.A, lda);
+    q.b_vec = vec_ok(q.B, ldb);
+    g_test_table.add(q, false);
+  }
+  SACHECK(g_test_table.commit(s));
+  Span span("gemm", s, 2.0 * M * N * K * batch, 1, true);
+  GemmScalars u = unit_scalars();
+  if (a_layout == 0 && b_layout == 0) return launch_gemm_auto<A_MK, B_KN, EPI_STORE>(g_test_table, u, s);
+  if (a_layout == 0 && b_layout == 1) return launch_gemm_auto<A_MK, B_NK, EPI_STORE>(g_test_table, u, s);
+  if (a_layout == 1 && b_layout == 0) return launch_gemm_auto<A_KM, B_KN, EPI_STORE>(g_test_table, u, s);
+  if (a_layout == 1 && b_layout == 1) return launch_gemm_auto<A_KM, B_NK, EPI_STORE>(g_test_table, u, s);
+  return fail(SA_ERR_INVALID, "sa_gemm_f32: layouts must be 0 or 1");
+}
+
+}  // extern "C"

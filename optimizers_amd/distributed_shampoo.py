@@ -1,0 +1,672 @@
+"""DistributedShampoo for one MI355X: the reference's constructor and `step()` surface over
+the native gfx950 kernels.
+
+Drop-in for `distributed_shampoo.DistributedShampoo` (reference
+distributed_shampoo/distributed_shampoo.py:361-382 ctor, :1677-1711 step) on the
+single-device distributor.  The Python here is host logic only: hyper-parameter checks,
+block partition, state allocation, the step schedule and error mapping.  Every tensor
+operation of the step runs in libshampoo_amd.so (hand-written HIP); there is no torch or
+CPU fallback for it, and construction fails if the library or a GPU is missing.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import logging
+import math
+from contextlib import nullcontext
+from fractions import Fraction
+from typing import Any, Callable
+
+import torch
+
+from optimizers_amd import native
+from optimizers_amd.blocking import BlockSpec, partition_parameter
+from optimizers_amd.matrix_functions_types import (
+    CoupledNewtonConfig,
+    EigenConfig,
+    EigendecompositionConfig,
+    PseudoInverseConfig,
+)
+from optimizers_amd.shampoo_types import (
+    ADAGRAD,
+    BETA3,
+    BETAS,
+    DISTRIBUTED_CONFIG,
+    EPSILON,
+    FILTERED_GRAD,
+    GRAFTING_CONFIG,
+    ITERATE_AVERAGING_CONFIG,
+    LR,
+    MAX_PRECONDITIONER_DIM,
+    MOMENTUM_BUFFER,
+    PARAMS,
+    PEAK_LR,
+    PRECONDITION_FREQUENCY,
+    PRECONDITIONER_CONFIG,
+    SHAMPOO,
+    START_PRECONDITIONING_STEP,
+    STEP,
+    USE_BIAS_CORRECTION,
+    USE_PIN_MEMORY,
+    WEIGHT_DECAY,
+    WEIGHT_DECAY_TYPE,
+    AdaGradPreconditionerConfig,
+    AdamPreconditionerConfig,
+    BaseShampooPreconditionerConfig,
+    ClassicMomentumConfig,
+    ConcurrencyConfig,
+    DefaultConcurrencyConfig,
+    DefaultShampooConfig,
+    DefaultShampooRuntimeConfig,
+    DefaultSingleDeviceDistributedConfig,
+    DistributedConfig,
+    IterateAveragingConfig,
+    PreconditionerConfig,
+    PreconditionerValueError,
+    RMSpropPreconditionerConfig,
+    RootInvShampooPreconditionerConfig,
+    SGDPreconditionerConfig,
+    ShampooRuntimeConfig,
+    SingleDeviceDistributedConfig,
+    WeightDecayType,
+)
+
+logger: logging.Logger = logging.getLogger(__name__)
+
+_ALIGN = 64  # floats: every state tensor starts on a 256-byte boundary of its arena
+
+
+def _round_up(x: int, a: int) -> int:
+    return (x + a - 1) // a * a
+
+
+class _Arena:
+    """One flat fp32 device buffer handing out aligned views (state tensors stay ordinary torch
+    tensors, so checkpoints see the same objects the kernels update)."""
+
+    def __init__(self, sizes: list[int], device: torch.device) -> None:
+        self.offsets = []
+        total = 0
+        for n in sizes:
+            self.offsets.append(total)
+            total += _round_up(max(n, 1), _ALIGN)
+        self.buffer = torch.zeros(max(total, _ALIGN), dtype=torch.float32, device=device)
+
+    def view(self, i: int, shape: tuple[int, ...]) -> torch.Tensor:
+        n = math.prod(shape)
+        return self.buffer[self.offsets[i] : self.offsets[i] + n].view(shape)
+
+
+class _NativeGroup:
+    """Native state and schedule of one parameter group (reference: the per-group state lists
+    built in distributed_shampoo.py:563-975 plus `_group_step_body` :1562-1667)."""
+
+    def __init__(self, optimizer: "DistributedShampoo", group: dict[str, Any], group_index: int) -> None:
+        self.lib = native.load()
+        self.group_index = group_index
+        params: list[torch.Tensor] = group[PARAMS]
+        if not params:
+            raise ValueError(f"Shampoo got an empty parameter {group=}")
+        self.params = params
+        self.device = params[0].device
+        if self.device.type != "cuda":
+            raise RuntimeError(
+                "optimizers_amd.DistributedShampoo runs on an MI355X only: parameters must live on a "
+                f"HIP device, got {self.device}. There is no CPU path."
+            )
+        for p in params:
+            if p.device != self.device:
+                raise ValueError("all parameters of a group must live on the same device")
+            if p.dtype != torch.float32:
+                raise NotImplementedError(f"only fp32 parameters are supported, got {p.dtype}")
+            if not p.is_contiguous():
+                raise ValueError("parameters must be contiguous (the reference views them with merged shapes)")
+
+        pc = group[PRECONDITIONER_CONFIG]
+        self._check_supported(group, pc)
+        self.preconditioner_config = pc
+        dist: DistributedConfig = group[DISTRIBUTED_CONFIG]
+        self.block_specs: list[BlockSpec] = []
+        self.num_blocks_per_param: list[int] = []
+        for i, p in enumerate(params):
+            specs = partition_parameter(
+                i, tuple(p.shape), group[MAX_PRECONDITIONER_DIM], dist.target_parameter_dimensionality
+            )
+            self.num_blocks_per_param.append(len(specs))
+            self.block_specs.extend(specs)
+        for s in self.block_specs:
+            if s.order > 2:
+                raise NotImplementedError(
+                    f"block of order {s.order} (shape {s.shape}): the native step covers blocks of order 1 and 2"
+                )
+
+        # native blocks = blocks with at least one element
+        self.native_index = [i for i, s in enumerate(self.block_specs) if s.numel > 0]
+        nb = len(self.native_index)
+        beta1 = group[BETAS][0]
+        graft = group[GRAFTING_CONFIG]
+        self.graft_type, self.graft_beta2, self.graft_weight, self.graft_bias, self.graft_eps = self._graft_setup(graft)
+        momentum_cfg = group[ITERATE_AVERAGING_CONFIG]
+
+        # which dims carry a Kronecker factor, and with which root
+        self.selectors: list[tuple[bool, ...]] = []
+        self.roots: list[tuple[float, ...]] = []
+        for i in self.native_index:
+            order = self.block_specs[i].order
+            exps = [self._inverse_exponent(pc, d, order) for d in range(order)]
+            self.selectors.append(tuple(e != 0.0 for e in exps))
+            self.roots.append(tuple(1 / e for e in exps if e != 0.0))
+
+        numels = [self.block_specs[i].numel for i in self.native_index]
+        fdims: list[int] = []
+        for k, i in enumerate(self.native_index):
+            s = self.block_specs[i]
+            fdims.extend(s.shape[d] for d in range(s.order) if self.selectors[k][d])
+        packed = [d * (d + 1) // 2 for d in fdims]
+        self.factor_arena = _Arena(packed, self.device)
+        self.inv_arena = _Arena(packed, self.device)
+        self.filtered_arena = _Arena(numels, self.device) if beta1 != 0.0 else None
+        self.adagrad_arena = _Arena(numels, self.device) if self.graft_type == native.SA_GRAFT_ADAGRAD else None
+        self.momentum_arena = _Arena(numels, self.device) if isinstance(momentum_cfg, ClassicMomentumConfig) else None
+
+        # optimizer.state layout (reference golden: tests/distributed_shampoo_test.py:516-622)
+        descs = (native.BlockDesc * max(nb, 1))()
+        self.factor_names: list[str] = []
+        self.factor_block: list[int] = []
+        self.bad_root_blocks: dict[int, str] = {}
+        self.failed_counter: dict[int, int] = {}
+        fi = 0
+        for k, i in enumerate(self.native_index):
+            s = self.block_specs[i]
+            p = params[s.param_index]
+            block_state: dict[str, Any] = optimizer.state[p].setdefault(s.block_key, {})
+            d = descs[k]
+            if s.order == 1:
+                d.rows, d.cols, d.ld = s.shape[0], 1, 1
+            else:
+                d.rows, d.cols, d.ld = s.shape[0], s.shape[1], s.strides[0]
+            d.param = p.data_ptr() + 4 * s.offset
+            shampoo_state: dict[str, dict[int, torch.Tensor]] = {"factor_matrices": {}, "inv_factor_matrices": {}}
+            slot = 0
+            for dim in range(s.order):
+                if not self.selectors[k][dim]:
+                    continue
+                n = s.shape[dim]
+                f = self.factor_arena.view(fi, (n * (n + 1) // 2,))
+                inv = self.inv_arena.view(fi, (n * (n + 1) // 2,))
+                idx = torch.arange(n, device=self.device)
+                inv[idx * n - idx * (idx - 1) // 2] = 1.0  # packed identity
+                shampoo_state["factor_matrices"][slot] = f
+                shampoo_state["inv_factor_matrices"][slot] = inv
+                d.factor[dim] = f.data_ptr()
+                d.inv_factor[dim] = inv.data_ptr()
+                root = Fraction(self.roots[k][slot])
+                if root.denominator != 1:
+                    # the reference raises inside matrix_inverse_root at every amortized step and
+                    # tolerates it num_tolerated_failed_amortized_computations times
+                    self.bad_root_blocks[k] = (
+                        f"{root.denominator=} must be equal to 1 to use coupled inverse Newton iteration!"
+                    )
+                    d.root[dim] = 1
+                else:
+                    d.root[dim] = int(root.numerator)
+                self.factor_names.append(f"{s.param_index}.{s.block_key}.{slot}")
+                self.factor_block.append(k)
+                slot += 1
+                fi += 1
+            block_state[SHAMPOO] = shampoo_state
+            if self.adagrad_arena is not None:
+                block_state[ADAGRAD] = self.adagrad_arena.view(k, s.shape)
+                d.adagrad = block_state[ADAGRAD].data_ptr()
+            if self.filtered_arena is not None:
+                block_state[FILTERED_GRAD] = self.filtered_arena.view(k, s.shape)
+                d.filtered_grad = block_state[FILTERED_GRAD].data_ptr()
+            if self.momentum_arena is not None:
+                block_state[MOMENTUM_BUFFER] = self.momentum_arena.view(k, s.shape)
+                d.momentum_buffer = block_state[MOMENTUM_BUFFER].data_ptr()
+            logger.info(
+                f"Instantiated Shampoo Preconditioner {s.param_index}.{s.block_key} for Parameter {s.param_index} "
+                f"({tuple(p.shape)}), Block {s.block_key} ({s.shape})."
+            )
+        # empty blocks still own a (state-less) entry, as in the reference
+        for i, s in enumerate(self.block_specs):
+            optimizer.state[params[s.param_index]].setdefault(s.block_key, {})
+
+        self.descs = descs
+        self.n_native = nb
+        self.plan = ctypes.c_void_p()
+        self.workspace = None
+        if nb:
+            native.check(self.lib.sa_plan_create(descs, nb, ctypes.byref(self.plan)), "sa_plan_create")
+            need = int(self.lib.sa_plan_workspace_bytes(self.plan))
+            self.workspace = torch.empty(need, dtype=torch.uint8, device=self.device)
+            native.check(
+                self.lib.sa_plan_bind_workspace(self.plan, self.workspace.data_ptr(), need), "sa_plan_bind_workspace"
+            )
+            self.n_factors = int(self.lib.sa_plan_num_factors(self.plan))
+            assert self.n_factors == len(self.factor_names)
+        else:
+            self.n_factors = 0
+        self.iterations = (ctypes.c_int32 * max(self.n_factors, 1))()
+        self.status = (ctypes.c_int32 * max(self.n_factors, 1))()
+        self.grad_ptrs = (ctypes.c_void_p * max(nb, 1))()
+        self.last_newton_iterations: list[int] = []
+
+        # one CPU step counter per group, aliased under every parameter (distributed_shampoo.py:790-815)
+        self.step_tensor = torch.tensor(0, dtype=torch.int64, device="cpu")
+        for p in params:
+            optimizer.state[p][STEP] = self.step_tensor
+        self.stream: torch.cuda.Stream | None = None
+
+    def close(self) -> None:
+        if self.plan:
+            self.lib.sa_plan_destroy(self.plan)
+            self.plan = ctypes.c_void_p()
+
+    # -- configuration helpers ---------------------------------------------------------------
+
+    @staticmethod
+    def _check_supported(group: dict[str, Any], pc: PreconditionerConfig) -> None:
+        if not isinstance(group[DISTRIBUTED_CONFIG], SingleDeviceDistributedConfig):
+            raise NotImplementedError(f"{group[DISTRIBUTED_CONFIG]=} not supported!")
+        if not isinstance(pc, RootInvShampooPreconditionerConfig):
+            raise NotImplementedError(f"{pc=} not supported!")
+        if not isinstance(pc.amortized_computation_config, CoupledNewtonConfig):
+            raise NotImplementedError(
+                f"Root inverse config is not implemented! Specified root inverse config is {pc.amortized_computation_config=}."
+            )
+        if not pc.use_symmetric_packing:
+            raise NotImplementedError("use_symmetric_packing=False: the native step keeps factors packed")
+        if pc.factor_matrix_dtype != torch.float32 or pc.inv_factor_matrix_dtype != torch.float32:
+            raise NotImplementedError("factor matrices are fp32 in the native step")
+        if pc.use_trace_scaling:
+            raise NotImplementedError("use_trace_scaling is not built")
+        if group[ITERATE_AVERAGING_CONFIG] is not None and not isinstance(
+            group[ITERATE_AVERAGING_CONFIG], ClassicMomentumConfig
+        ):
+            raise NotImplementedError(
+                f"{group[ITERATE_AVERAGING_CONFIG]=} is not supported! Supported configs: ClassicMomentumConfig."
+            )
+
+    @staticmethod
+    def _inverse_exponent(pc: RootInvShampooPreconditionerConfig, dimension: int, order: int) -> float:
+        """shampoo_preconditioner_list.py:1726-1747."""
+        override = pc.inverse_exponent_override.get(order, {})
+        if isinstance(override, dict):
+            return override.get(dimension, 1 / (2 * max(order, 1)))
+        return override
+
+    @staticmethod
+    def _graft_setup(graft: PreconditionerConfig | None) -> tuple[int, float, float, bool, float]:
+        """(type, beta2, weighting factor, bias correction, epsilon), distributed_shampoo.py:673-714."""
+        if graft is None:
+            return native.SA_GRAFT_NONE, 1.0, 1.0, False, 0.0
+        if isinstance(graft, SGDPreconditionerConfig):
+            return native.SA_GRAFT_SGD, 1.0, 1.0, False, 0.0
+        if isinstance(graft, RMSpropPreconditionerConfig) and graft.drop_weighting_factor_on_gsquare:
+            return native.SA_GRAFT_ADAGRAD, graft.beta2, 1.0, False, graft.epsilon
+        if isinstance(graft, AdamPreconditionerConfig):
+            return native.SA_GRAFT_ADAGRAD, graft.beta2, 1 - graft.beta2, True, graft.epsilon
+        if isinstance(graft, RMSpropPreconditionerConfig):
+            return native.SA_GRAFT_ADAGRAD, graft.beta2, 1 - graft.beta2, False, graft.epsilon
+        if isinstance(graft, AdaGradPreconditionerConfig):
+            return native.SA_GRAFT_ADAGRAD, 1.0, 1.0, False, graft.epsilon
+        raise NotImplementedError(f"{graft=} not supported!")
+
+    # -- one step ----------------------------------------------------------------------------
+
+    def _bind_gradients(self, eager_nan_check: bool) -> int:
+        """Per-block gradient pointers; a parameter without a (non-empty) gradient masks its blocks
+        (shampoo_distributor.py:259-299).  Returns the number of active blocks."""
+        grads: list[torch.Tensor | None] = []
+        for p in self.params:
+            g = p.grad
+            if g is None or g.numel() == 0:
+                grads.append(None)
+                continue
+            if g.dtype != torch.float32 or g.device != p.device:
+                raise NotImplementedError("gradients must be fp32 on the parameter's device")
+            if not g.is_contiguous():
+                raise ValueError("gradients must be contiguous (the reference views them with merged shapes)")
+            if eager_nan_check:
+                assert torch.isfinite(g).all(), (
+                    f"Encountered gradient containing NaN/Inf in parameter with shape {g.shape}. "
+                    "Check your model for numerical instability or consider gradient clipping."
+                )
+            grads.append(g)
+        active = 0
+        for k, i in enumerate(self.native_index):
+            s = self.block_specs[i]
+            g = grads[s.param_index]
+            if g is None:
+                self.grad_ptrs[k] = None
+            else:
+                self.grad_ptrs[k] = g.data_ptr() + 4 * s.offset
+                active += 1
+        self._grads_alive = grads  # keep the tensors alive until the step has been enqueued
+        return active
+
+    def step(self, group: dict[str, Any], runtime: ShampooRuntimeConfig) -> None:
+        lib = self.lib
+        active = self._bind_gradients(runtime.eager_nan_check) if self.n_native else 0
+        step = self.step_tensor.add_(1)
+        step_val = int(step.item())
+        if not active:
+            self._grads_alive = None
+            return
+        stream = native.current_stream_ptr(self.device)
+        native.check(lib.sa_plan_bind_gradients(self.plan, self.grad_ptrs, stream), "sa_plan_bind_gradients")
+
+        beta1, beta2 = group[BETAS]
+        beta3 = group[BETA3]
+        lr = torch.tensor(group[LR], dtype=torch.float32).item()
+        weight_decay = group[WEIGHT_DECAY]
+        wd_type = group[WEIGHT_DECAY_TYPE]
+        start = group[START_PRECONDITIONING_STEP]
+        freq = group[PRECONDITION_FREQUENCY]
+        use_bc = group[USE_BIAS_CORRECTION]
+        pc = self.preconditioner_config
+        amortize = (step_val % freq == 0 and step_val > start) or step_val == start
+        graft_only = step_val < start and group[GRAFTING_CONFIG] is not None
+
+        if weight_decay != 0.0 and wd_type == WeightDecayType.L2:
+            native.check(lib.sa_add_l2_regularization(self.plan, weight_decay, stream), "sa_add_l2_regularization")
+
+        drop = pc.drop_weighting_factor_on_gsquare
+        weighting = 1.0 if (drop or beta2 == 1.0) else 1 - beta2
+        native.check(lib.sa_update_factor_matrices(self.plan, beta2, weighting, stream), "sa_update_factor_matrices")
+
+        # fp32 scalars evaluated with the very torch expressions the reference uses
+        bc2 = 1.0
+        if use_bc and beta2 < 1.0 and not drop:
+            bc2 = float(torch.tensor(1.0) - beta2**step)
+        if amortize:
+            self._amortized_computation(group, bc2, stream)
+
+        s = native.StepScalars()
+        s.lr = lr
+        s.beta1 = beta1
+        s.beta3 = beta3 if beta1 != 0.0 else 0.0
+        s.bias_correction1 = float(1.0 - beta3 * beta1 ** (step - 1)) if (use_bc and beta1 != 0.0) else 1.0
+        s.graft_type = self.graft_type
+        s.graft_beta2 = self.graft_beta2
+        s.graft_weight = self.graft_weight
+        s.graft_bias_correction2 = (
+            float(torch.tensor(1.0) - self.graft_beta2**step) if (self.graft_bias and self.graft_beta2 < 1.0) else 1.0
+        )
+        s.graft_epsilon = self.graft_eps
+        alpha = 0.0
+        if weight_decay != 0.0 and wd_type != WeightDecayType.L2:
+            if wd_type == WeightDecayType.DECOUPLED:
+                alpha = weight_decay
+            elif wd_type == WeightDecayType.CORRECTED:
+                alpha = weight_decay * lr / group[PEAK_LR]
+            elif wd_type == WeightDecayType.INDEPENDENT:
+                alpha = weight_decay / group[PEAK_LR]
+            else:
+                raise ValueError(f"Invalid weight decay type: {wd_type=}!")
+        s.weight_decay_alpha = alpha
+        mom = group[ITERATE_AVERAGING_CONFIG]
+        if isinstance(mom, ClassicMomentumConfig):
+            s.momentum, s.dampening, s.use_nesterov = mom.momentum, mom.dampening, int(mom.use_nesterov)
+        else:
+            s.momentum, s.dampening, s.use_nesterov = 0.0, 0.0, 0
+
+        ref = ctypes.byref(s)
+        if graft_only:
+            native.check(lib.sa_grafting_only_step(self.plan, ref, stream), "sa_grafting_only_step")
+        else:
+            native.check(
+                lib.sa_update_grafting_and_filtered_grad(self.plan, ref, stream),
+                "sa_update_grafting_and_filtered_grad",
+            )
+            native.check(lib.sa_precondition(self.plan, ref, stream), "sa_precondition")
+            native.check(lib.sa_apply_update(self.plan, ref, stream), "sa_apply_update")
+        # drop the references so param.grad can be freed (distributed_shampoo.py:1666-1667)
+        self._grads_alive = None
+
+    def _amortized_computation(self, group: dict[str, Any], bc2: float, stream: int) -> None:
+        """Batched inverse roots + the reference's error semantics
+        (shampoo_preconditioner_list.py:314-443)."""
+        pc = self.preconditioner_config
+        cfg: CoupledNewtonConfig = pc.amortized_computation_config
+        native.check(
+            self.lib.sa_compute_root_inverses_newton(
+                self.plan, bc2, group[EPSILON], cfg.max_iterations, cfg.tolerance, self.iterations, self.status, stream
+            ),
+            "sa_compute_root_inverses_newton",
+        )
+        self.last_newton_iterations = [int(self.iterations[i]) for i in range(self.n_factors)]
+        for i in range(self.n_factors):
+            st = int(self.status[i])
+            name = self.factor_names[i]
+            if st == native.SA_FACTOR_INPUT_NONFINITE:
+                raise PreconditionerValueError(
+                    f"Encountered nan/inf values in factor matrix {name}! "
+                    "To mitigate, check if nan inputs are being passed into the network or nan gradients are being passed to the optimizer. "
+                    "Otherwise, in some cases, this may be due to divergence of the algorithm. To mitigate, try decreasing the learning rate or increasing grafting epsilon."
+                )
+            if st == native.SA_FACTOR_RESULT_NONFINITE:
+                raise PreconditionerValueError(
+                    f"Encountered nan or inf values in name of factor matrix {name}! "
+                    "To mitigate, check factor matrix before the matrix computation."
+                )
+            if st == native.SA_FACTOR_NOT_CONVERGED:
+                logger.warning("Newton did not converge and reached maximum number of iterations!")
+        # blocks whose root cannot be used by the coupled Newton iteration fail every time
+        for k, message in self.bad_root_blocks.items():
+            count = self.failed_counter.get(k, 0) + 1
+            self.failed_counter[k] = count
+            logger.warning(f"Matrix computation failed with exception={message!r}. Using previous preconditioner and continuing...")
+            if count > pc.num_tolerated_failed_amortized_computations:
+                names = tuple(n for n, b in zip(self.factor_names, self.factor_block) if b == k)
+                raise ValueError(
+                    f"The number of failed amortized computations for factors {names} exceeded the allowed tolerance. "
+                    f"The last seen exception was {message}."
+                )
+
+
+class DistributedShampoo(torch.optim.Optimizer):
+    """Distributed Shampoo on one MI355X.
+
+    Arguments, defaults and validation follow the reference constructor
+    (distributed_shampoo/distributed_shampoo.py:361-535).  Built natively:
+    `RootInvShampooPreconditionerConfig` with `CoupledNewtonConfig`, grafting with
+    SGD / AdaGrad / RMSprop / Adam, every `WeightDecayType`, `ClassicMomentumConfig`,
+    `SingleDeviceDistributedConfig`.  Anything else raises NotImplementedError at construction.
+    """
+
+    def __init__(
+        self,
+        params,
+        lr: float = 1e-2,
+        betas: tuple[float, float] = (0.9, 1.0),
+        beta3: float = -1.0,
+        epsilon: float = 1e-12,
+        weight_decay: float = 0.0,
+        weight_decay_type: WeightDecayType = WeightDecayType.DECOUPLED,
+        max_preconditioner_dim: int | float = 1024,
+        precondition_frequency: int = 1,
+        start_preconditioning_step: int = -1,
+        use_bias_correction: bool = True,
+        iterate_averaging_config: IterateAveragingConfig | None = None,
+        grafting_config: PreconditionerConfig | None = None,
+        use_pin_memory: bool = False,
+        shampoo_pt2_compile_config: object | None = None,
+        distributed_config: DistributedConfig = DefaultSingleDeviceDistributedConfig,
+        preconditioner_config: PreconditionerConfig = DefaultShampooConfig,
+        shampoo_runtime_config: ShampooRuntimeConfig = DefaultShampooRuntimeConfig,
+        concurrency_config: ConcurrencyConfig = DefaultConcurrencyConfig,
+    ) -> None:
+        super().__init__(
+            params,
+            {
+                LR: lr,
+                BETAS: betas,
+                BETA3: beta3,
+                EPSILON: epsilon,
+                WEIGHT_DECAY: weight_decay,
+                PEAK_LR: lr,
+                WEIGHT_DECAY_TYPE: weight_decay_type,
+                MAX_PRECONDITIONER_DIM: max_preconditioner_dim,
+                PRECONDITION_FREQUENCY: precondition_frequency,
+                START_PRECONDITIONING_STEP: start_preconditioning_step,
+                USE_BIAS_CORRECTION: use_bias_correction,
+                ITERATE_AVERAGING_CONFIG: iterate_averaging_config,
+                GRAFTING_CONFIG: grafting_config,
+                USE_PIN_MEMORY: use_pin_memory,
+                DISTRIBUTED_CONFIG: distributed_config,
+                PRECONDITIONER_CONFIG: preconditioner_config,
+            },
+        )
+        if shampoo_pt2_compile_config is not None:
+            raise NotImplementedError("shampoo_pt2_compile_config: the native step is not traced by torch.compile")
+        for i, group in enumerate(self.param_groups):
+            logger.info(f"Checking param_group {i} hyperparameters...")
+            self._check_group(group)
+        self._runtime_config = shampoo_runtime_config
+        self._concurrency_config = concurrency_config
+        self._groups: list[_NativeGroup] = [_NativeGroup(self, g, i) for i, g in enumerate(self.param_groups)]
+        all_cuda = all(g[PARAMS][0].device.type == "cuda" for g in self.param_groups)
+        self._use_streams = bool(concurrency_config.enable_cuda_stream_for_param_groups and all_cuda)
+        if self._use_streams:
+            for ng in self._groups:
+                ng.stream = torch.cuda.Stream(device=ng.device)
+        self.register_load_state_dict_post_hook(DistributedShampoo._after_load_state_dict)
+
+    def __del__(self) -> None:
+        for ng in getattr(self, "_groups", []):
+            try:
+                ng.close()
+            except Exception:  # noqa: BLE001 - interpreter shutdown
+                pass
+
+    @staticmethod
+    def _check_group(group: dict[str, Any]) -> None:
+        """distributed_shampoo.py:411-530, same conditions and messages."""
+        if not group[LR] >= 0.0:
+            raise ValueError(f"Invalid {group[LR]=}. Must be >= 0.0.")
+        if not 0.0 <= group[BETAS][0] < 1.0:
+            raise ValueError(f"Invalid {group[BETAS][0]=}. Must be in [0.0, 1.0).")
+        if not 0.0 <= group[BETAS][1] <= 1.0:
+            raise ValueError(f"Invalid {group[BETAS][1]=}. Must be in [0.0, 1.0].")
+        if group[BETA3] == -1.0:
+            group[BETA3] = group[BETAS][0]
+        elif not 0.0 <= group[BETA3] < 1.0:
+            raise ValueError(f"Invalid {group[BETA3]=}. Must be in [0.0, 1.0).")
+        pc = group[PRECONDITIONER_CONFIG]
+        if (
+            isinstance(pc, BaseShampooPreconditionerConfig)
+            and isinstance(pc.amortized_computation_config, EigendecompositionConfig)
+            and isinstance(pc.amortized_computation_config.rank_deficient_stability_config, PseudoInverseConfig)
+        ):
+            if group[EPSILON] != 0.0:
+                raise ValueError(f"Invalid {group[EPSILON]=}. Must be == 0.0 when PseudoInverseConfig is used.")
+        elif not group[EPSILON] > 0.0:
+            raise ValueError(f"Invalid {group[EPSILON]=}. Must be > 0.0.")
+        if not group[WEIGHT_DECAY] >= 0.0:
+            raise ValueError(f"Invalid {group[WEIGHT_DECAY]=}. Must be >= 0.0.")
+        if (
+            group[WEIGHT_DECAY_TYPE] in (WeightDecayType.CORRECTED, WeightDecayType.INDEPENDENT)
+            and not group[PEAK_LR] > 0.0
+        ):
+            raise ValueError(
+                f"Invalid {group[PEAK_LR]=}. Must be > 0.0 when using WeightDecayType.CORRECTED or WeightDecayType.INDEPENDENT."
+            )
+        if isinstance(group[MAX_PRECONDITIONER_DIM], float) and group[MAX_PRECONDITIONER_DIM] != math.inf:
+            raise ValueError(f"Invalid {group[MAX_PRECONDITIONER_DIM]=}. Must be an integer or math.inf.")
+        if not group[MAX_PRECONDITIONER_DIM] >= 1:
+            raise ValueError(f"Invalid {group[MAX_PRECONDITIONER_DIM]=}. Must be >= 1.")
+        if not group[PRECONDITION_FREQUENCY] >= 1:
+            raise ValueError(f"Invalid {group[PRECONDITION_FREQUENCY]=}. Must be >= 1.")
+        if not group[START_PRECONDITIONING_STEP] >= -1:
+            raise ValueError(f"Invalid {group[START_PRECONDITIONING_STEP]=}. Must be >= -1.")
+        if group[START_PRECONDITIONING_STEP] == -1:
+            group[START_PRECONDITIONING_STEP] = group[PRECONDITION_FREQUENCY]
+            logger.warning(
+                f"start_preconditioning_step set to -1. Setting start_preconditioning_step equal to {group[PRECONDITION_FREQUENCY]=} by default."
+            )
+        if group[START_PRECONDITIONING_STEP] < group[PRECONDITION_FREQUENCY]:
+            raise ValueError(
+                f"Invalid {group[START_PRECONDITIONING_STEP]=}. Must be >= {group[PRECONDITION_FREQUENCY]=}."
+            )
+
+    @torch.no_grad()
+    def step(self, closure: Callable[[], float] | None = None) -> float | None:
+        """One optimization step (distributed_shampoo.py:1677-1711)."""
+        loss = None
+        if closure is not None:
+            with torch.enable_grad():
+                loss = closure()
+        for ng, group in zip(self._groups, self.param_groups, strict=True):
+            if self._use_streams:
+                ng.stream.wait_stream(torch.cuda.current_stream(ng.device))
+                ctx = torch.cuda.stream(ng.stream)
+            else:
+                ctx = nullcontext()
+            with ctx:
+                ng.step(group, self._runtime_config)
+        if self._use_streams:
+            for ng in self._groups:
+                torch.cuda.current_stream(ng.device).wait_stream(ng.stream)
+        return loss
+
+    # -- checkpointing ----------------------------------------------------------------------
+
+    @staticmethod
+    def _after_load_state_dict(optimizer: "DistributedShampoo") -> None:
+        """torch's load_state_dict replaces the state tensors with copies; move the loaded values
+        back into the arenas the kernels own and re-alias the state (the reference copies in place
+        too, distributed_shampoo.py:1803-1889)."""
+        for ng in optimizer._groups:
+            ng.restore_state(optimizer)
+
+
+def _restore_state(self: _NativeGroup, optimizer: DistributedShampoo) -> None:
+    loaded_steps = []
+    fi = 0
+    for k, i in enumerate(self.native_index):
+        s = self.block_specs[i]
+        p = self.params[s.param_index]
+        st = optimizer.state[p]
+        block = st.get(s.block_key, {})
+        slot = 0
+        sh = block.get(SHAMPOO, {"factor_matrices": {}, "inv_factor_matrices": {}})
+        for dim in range(s.order):
+            if not self.selectors[k][dim]:
+                continue
+            n = s.shape[dim]
+            shape = (n * (n + 1) // 2,)
+            for key, arena in (("factor_matrices", self.factor_arena), ("inv_factor_matrices", self.inv_arena)):
+                mine = arena.view(fi, shape)
+                src = sh[key].get(slot, sh[key].get(str(slot))) if key in sh else None
+                if src is not None and src.data_ptr() != mine.data_ptr():
+                    mine.copy_(src)
+                sh.setdefault(key, {})[slot] = mine
+                sh[key].pop(str(slot), None)
+            slot += 1
+            fi += 1
+        block[SHAMPOO] = sh
+        for key, arena in ((ADAGRAD, self.adagrad_arena), (FILTERED_GRAD, self.filtered_arena), (MOMENTUM_BUFFER, self.momentum_arena)):
+            if arena is None:
+                continue
+            mine = arena.view(k, s.shape)
+            src = block.get(key)
+            if src is not None and src.data_ptr() != mine.data_ptr():
+                mine.copy_(src)
+            block[key] = mine
+        st[s.block_key] = block
+    for p in self.params:
+        if STEP in optimizer.state[p]:
+            loaded_steps.append(int(optimizer.state[p][STEP]))
+    if loaded_steps:
+        assert len(set(loaded_steps)) == 1, f"parameters of one group disagree on step: {sorted(set(loaded_steps))}"
+        self.step_tensor.fill_(loaded_steps[0])
+    for p in self.params:
+        optimizer.state[p][STEP] = self.step_tensor
+    if self.plan:
+        native.check(self.lib.sa_plan_invalidate_inverse_cache(self.plan), "sa_plan_invalidate_inverse_cache")
+
+
+_NativeGroup.restore_state = _restore_state  # type: ignore[attr-defined]
