@@ -151,6 +151,9 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="llama3_8b_layer", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 1 GiB copy kernel (sa::copy_kernel) so that rocprofv3 --pmc FETCH_SIZE / "
+                         "WRITE_SIZE readings can be scaled against a kernel of known traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build targets one MI355X; --gpus must be 1 (no collectives, no sharding).")
@@ -180,6 +183,12 @@ def main() -> None:
     for i in range(args.warmup):
         one_step(i)
     torch.cuda.synchronize()
+    if args.calibrate_copy:
+        src = torch.ones(1 << 28, device=device)  # 1 GiB
+        dst = torch.empty_like(src)
+        native.check(lib.sa_copy_f32(src.data_ptr(), dst.data_ptr(), src.numel(), native.current_stream_ptr(device)), "sa_copy_f32")
+        torch.cuda.synchronize()
+        del src, dst
 
     lib.sa_set_profiling(1)
     phases = ("newton_gemm", "syrk", "precondition_gemm", "grafting", "apply")

@@ -153,6 +153,10 @@ int32_t sa_gemm_f32(const float* A, const float* B, float* C, int32_t M, int32_t
                     int64_t lda, int64_t ldb, int64_t ldc, int32_t a_layout, int32_t b_layout,
                     int32_t batch, int64_t stride_a, int64_t stride_b, int64_t stride_c, void* stream);
 
+/* dst[i] = src[i] for n floats with a plain float4 copy kernel (n % 4 == 0, 16-byte aligned): the
+ * known-traffic kernel that hardware HBM counters are calibrated against. */
+int32_t sa_copy_f32(const float* src, float* dst, int64_t n, void* stream);
+
 /* Averaged duration (milliseconds, HIP events on `stream`) of the kernels of the named phase during
  * the most recent call that ran it: "newton_gemm", "syrk", "precondition_gemm", "grafting", "apply".
  * Timing is off unless sa_set_profiling(1) was called; returns a negative value if unavailable. */

@@ -517,6 +517,12 @@ __global__ void newton_control_kernel(NewtonCtl c, const int* __restrict__ ids, 
   if (threadIdx.x == 0) *n_active = cnt;
 }
 
+// Plain float4 copy of n4 vectors: the known-traffic kernel HBM counters are scaled against.
+__global__ __launch_bounds__(256) void copy_kernel(const float4* __restrict__ src, float4* __restrict__ dst, long long n4) {
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (long long)gridDim.x * blockDim.x)
+    dst[i] = src[i];
+}
+
 __global__ void copy_strided_kernel(const float* __restrict__ src, long long lds_, float* __restrict__ dst,
                                     int rows, int cols) {
   const long long n = (long long)rows * cols;

@@ -1035,4 +1035,15 @@ int32_t sa_gemm_f32(const float* A, const float* B, float* C, int32_t M, int32_t
   return fail(SA_ERR_INVALID, "sa_gemm_f32: layouts must be 0 or 1");
 }
 
+int32_t sa_copy_f32(const float* src, float* dst, int64_t n, void* stream) {
+  if (!src || !dst || n <= 0 || (n & 3) || ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15))
+    return fail(SA_ERR_INVALID, "sa_copy_f32: need 16-byte aligned pointers and n a multiple of 4");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  Span span("copy", s, 8.0 * (double)n, 1, true);
+  hipLaunchKernelGGL(copy_kernel, dim3(256 * 16), dim3(256), 0, s, reinterpret_cast<const float4*>(src),
+                     reinterpret_cast<float4*>(dst), (long long)(n / 4));
+  HIPCHECK(hipGetLastError());
+  return SA_OK;
+}
+
 }  // extern "C"

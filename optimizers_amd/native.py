@@ -31,7 +31,7 @@ EXPORTS = (
     "sa_plan_bind_gradients", "sa_add_l2_regularization", "sa_update_factor_matrices",
     "sa_compute_root_inverses_newton", "sa_update_grafting_and_filtered_grad", "sa_precondition",
     "sa_apply_update", "sa_grafting_only_step", "sa_plan_read_norms", "sa_plan_read_preconditioned",
-    "sa_gemm_f32", "sa_set_profiling", "sa_phase_ms", "sa_phase_flops", "sa_phase_launches",
+    "sa_gemm_f32", "sa_copy_f32", "sa_set_profiling", "sa_phase_ms", "sa_phase_flops", "sa_phase_launches",
 )
 
 
@@ -110,6 +110,7 @@ def load() -> ctypes.CDLL:
         c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int64, c_int64, c_int64, c_int32, c_int32,
         c_int32, c_int64, c_int64, c_int64, c_void_p,
     ]
+    lib.sa_copy_f32.argtypes = [c_void_p, c_void_p, c_int64, c_void_p]
     lib.sa_set_profiling.argtypes = [c_int32]
     lib.sa_phase_ms.argtypes = [c_char_p]
     lib.sa_phase_ms.restype = c_double
