@@ -543,53 +543,53 @@ class DistributedShampoo(torch.optim.Optimizer):
                 pass
 
     @staticmethod
-    def _check_group(group: dict[str, Any]) -> None:
+    def _check_group(param_group: dict[str, Any]) -> None:
         """distributed_shampoo.py:411-530, same conditions and messages."""
-        if not group[LR] >= 0.0:
-            raise ValueError(f"Invalid {group[LR]=}. Must be >= 0.0.")
-        if not 0.0 <= group[BETAS][0] < 1.0:
-            raise ValueError(f"Invalid {group[BETAS][0]=}. Must be in [0.0, 1.0).")
-        if not 0.0 <= group[BETAS][1] <= 1.0:
-            raise ValueError(f"Invalid {group[BETAS][1]=}. Must be in [0.0, 1.0].")
-        if group[BETA3] == -1.0:
-            group[BETA3] = group[BETAS][0]
-        elif not 0.0 <= group[BETA3] < 1.0:
-            raise ValueError(f"Invalid {group[BETA3]=}. Must be in [0.0, 1.0).")
-        pc = group[PRECONDITIONER_CONFIG]
+        if not param_group[LR] >= 0.0:
+            raise ValueError(f"Invalid {param_group[LR]=}. Must be >= 0.0.")
+        if not 0.0 <= param_group[BETAS][0] < 1.0:
+            raise ValueError(f"Invalid {param_group[BETAS][0]=}. Must be in [0.0, 1.0).")
+        if not 0.0 <= param_group[BETAS][1] <= 1.0:
+            raise ValueError(f"Invalid {param_group[BETAS][1]=}. Must be in [0.0, 1.0].")
+        if param_group[BETA3] == -1.0:
+            param_group[BETA3] = param_group[BETAS][0]
+        elif not 0.0 <= param_group[BETA3] < 1.0:
+            raise ValueError(f"Invalid {param_group[BETA3]=}. Must be in [0.0, 1.0).")
+        pc = param_group[PRECONDITIONER_CONFIG]
         if (
             isinstance(pc, BaseShampooPreconditionerConfig)
             and isinstance(pc.amortized_computation_config, EigendecompositionConfig)
             and isinstance(pc.amortized_computation_config.rank_deficient_stability_config, PseudoInverseConfig)
         ):
-            if group[EPSILON] != 0.0:
-                raise ValueError(f"Invalid {group[EPSILON]=}. Must be == 0.0 when PseudoInverseConfig is used.")
-        elif not group[EPSILON] > 0.0:
-            raise ValueError(f"Invalid {group[EPSILON]=}. Must be > 0.0.")
-        if not group[WEIGHT_DECAY] >= 0.0:
-            raise ValueError(f"Invalid {group[WEIGHT_DECAY]=}. Must be >= 0.0.")
+            if param_group[EPSILON] != 0.0:
+                raise ValueError(f"Invalid {param_group[EPSILON]=}. Must be == 0.0 when PseudoInverseConfig is used.")
+        elif not param_group[EPSILON] > 0.0:
+            raise ValueError(f"Invalid {param_group[EPSILON]=}. Must be > 0.0.")
+        if not param_group[WEIGHT_DECAY] >= 0.0:
+            raise ValueError(f"Invalid {param_group[WEIGHT_DECAY]=}. Must be >= 0.0.")
         if (
-            group[WEIGHT_DECAY_TYPE] in (WeightDecayType.CORRECTED, WeightDecayType.INDEPENDENT)
-            and not group[PEAK_LR] > 0.0
+            param_group[WEIGHT_DECAY_TYPE] in (WeightDecayType.CORRECTED, WeightDecayType.INDEPENDENT)
+            and not param_group[PEAK_LR] > 0.0
         ):
             raise ValueError(
-                f"Invalid {group[PEAK_LR]=}. Must be > 0.0 when using WeightDecayType.CORRECTED or WeightDecayType.INDEPENDENT."
+                f"Invalid {param_group[PEAK_LR]=}. Must be > 0.0 when using WeightDecayType.CORRECTED or WeightDecayType.INDEPENDENT."
             )
-        if isinstance(group[MAX_PRECONDITIONER_DIM], float) and group[MAX_PRECONDITIONER_DIM] != math.inf:
-            raise ValueError(f"Invalid {group[MAX_PRECONDITIONER_DIM]=}. Must be an integer or math.inf.")
-        if not group[MAX_PRECONDITIONER_DIM] >= 1:
-            raise ValueError(f"Invalid {group[MAX_PRECONDITIONER_DIM]=}. Must be >= 1.")
-        if not group[PRECONDITION_FREQUENCY] >= 1:
-            raise ValueError(f"Invalid {group[PRECONDITION_FREQUENCY]=}. Must be >= 1.")
-        if not group[START_PRECONDITIONING_STEP] >= -1:
-            raise ValueError(f"Invalid {group[START_PRECONDITIONING_STEP]=}. Must be >= -1.")
-        if group[START_PRECONDITIONING_STEP] == -1:
-            group[START_PRECONDITIONING_STEP] = group[PRECONDITION_FREQUENCY]
+        if isinstance(param_group[MAX_PRECONDITIONER_DIM], float) and param_group[MAX_PRECONDITIONER_DIM] != math.inf:
+            raise ValueError(f"Invalid {param_group[MAX_PRECONDITIONER_DIM]=}. Must be an integer or math.inf.")
+        if not param_group[MAX_PRECONDITIONER_DIM] >= 1:
+            raise ValueError(f"Invalid {param_group[MAX_PRECONDITIONER_DIM]=}. Must be >= 1.")
+        if not param_group[PRECONDITION_FREQUENCY] >= 1:
+            raise ValueError(f"Invalid {param_group[PRECONDITION_FREQUENCY]=}. Must be >= 1.")
+        if not param_group[START_PRECONDITIONING_STEP] >= -1:
+            raise ValueError(f"Invalid {param_group[START_PRECONDITIONING_STEP]=}. Must be >= -1.")
+        if param_group[START_PRECONDITIONING_STEP] == -1:
+            param_group[START_PRECONDITIONING_STEP] = param_group[PRECONDITION_FREQUENCY]
             logger.warning(
-                f"start_preconditioning_step set to -1. Setting start_preconditioning_step equal to {group[PRECONDITION_FREQUENCY]=} by default."
+                f"start_preconditioning_step set to -1. Setting start_preconditioning_step equal to {param_group[PRECONDITION_FREQUENCY]=} by default."
             )
-        if group[START_PRECONDITIONING_STEP] < group[PRECONDITION_FREQUENCY]:
+        if param_group[START_PRECONDITIONING_STEP] < param_group[PRECONDITION_FREQUENCY]:
             raise ValueError(
-                f"Invalid {group[START_PRECONDITIONING_STEP]=}. Must be >= {group[PRECONDITION_FREQUENCY]=}."
+                f"Invalid {param_group[START_PRECONDITIONING_STEP]=}. Must be >= {param_group[PRECONDITION_FREQUENCY]=}."
             )
 
     @torch.no_grad()

@@ -1,0 +1,250 @@
+"""Host-visible behaviour of the native optimizer on the GPU: library equivalences, masking,
+weight-decay flavours, checkpoint round trip, failure semantics."""
+
+import copy
+import math
+
+import pytest
+import torch
+
+from tests.golden_cases import rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _newton(**kw):
+    import optimizers_amd as oa
+
+    return oa.RootInvShampooPreconditionerConfig(amortized_computation_config=oa.CoupledNewtonConfig(), **kw)
+
+
+def _oracle(params, **kw):
+    from oracle.shampoo_oracle import OracleConfig, ShampooOracle
+
+    return ShampooOracle(params, OracleConfig(preconditioner="newton", **kw))
+
+
+@pytest.mark.parametrize("decoupled", [True, False])
+def test_grafting_only_equals_torch_adam(decoupled):
+    """gpu_tests/shampoo_grafting_test.py:68-266 idea: preconditioning never starts."""
+    import optimizers_amd as oa
+
+    torch.manual_seed(0)
+    shapes = [(70, 33), (33,), (5, 1, 7)]
+    init = [torch.randn(*s) for s in shapes]
+    lr, betas, eps, wd = 0.01, (0.9, 0.999), 1e-8, 0.05
+    ref_p = [torch.nn.Parameter(t.clone()) for t in init]
+    ref = (torch.optim.AdamW if decoupled else torch.optim.Adam)(ref_p, lr=lr, betas=betas, eps=eps, weight_decay=wd)
+    params = [torch.nn.Parameter(t.clone().to(DEV)) for t in init]
+    opt = oa.DistributedShampoo(
+        params, lr=lr, betas=betas, epsilon=1e-12, weight_decay=wd,
+        weight_decay_type=oa.WeightDecayType.DECOUPLED if decoupled else oa.WeightDecayType.L2,
+        max_preconditioner_dim=32, precondition_frequency=1, start_preconditioning_step=10**9,
+        preconditioner_config=_newton(), grafting_config=oa.AdamPreconditionerConfig(beta2=betas[1], epsilon=eps),
+    )
+    for _ in range(6):
+        grads = [torch.randn(*s) for s in shapes]
+        for p, q, g in zip(ref_p, params, grads):
+            p.grad = g.clone()
+            q.grad = g.to(DEV)
+        ref.step()
+        opt.step()
+    for q, p in zip(params, ref_p):
+        torch.testing.assert_close(q.detach().cpu(), p.detach(), rtol=2e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("wd_type", ["DECOUPLED", "CORRECTED", "INDEPENDENT", "L2"])
+@pytest.mark.parametrize("graft", ["adam", "rmsprop", "adagrad", "sgd", None])
+def test_weight_decay_and_grafting_flavours_match_oracle(wd_type, graft):
+    import optimizers_amd as oa
+
+    g = torch.Generator().manual_seed(11)
+    shapes = [(40, 24), (24,)]
+    init = [torch.randn(*s, generator=g) for s in shapes]
+    kw = dict(lr=0.02, betas=(0.9, 0.99), epsilon=1e-8, weight_decay=0.01, max_preconditioner_dim=16,
+              precondition_frequency=2, start_preconditioning_step=4)
+    gcfg = {"adam": oa.AdamPreconditionerConfig(beta2=0.95, epsilon=1e-7), "rmsprop": oa.RMSpropPreconditionerConfig(beta2=0.95, epsilon=1e-7),
+            "adagrad": oa.AdaGradPreconditionerConfig(epsilon=1e-7), "sgd": oa.SGDPreconditionerConfig(), None: None}[graft]
+    params = [torch.nn.Parameter(t.clone().to(DEV)) for t in init]
+    opt = oa.DistributedShampoo(params, weight_decay_type=oa.WeightDecayType[wd_type],
+                                preconditioner_config=_newton(inverse_exponent_override={1: {0: 0.0}}), grafting_config=gcfg, **kw)
+    ref_p = [t.clone() for t in init]
+    ref = _oracle(ref_p, weight_decay_type=wd_type, inverse_exponent_override={1: {0: 0.0}}, grafting=graft,
+                  grafting_beta2=0.95, grafting_epsilon=1e-7, **kw)
+    for step in range(8):
+        grads = [torch.randn(*s, generator=g) for s in shapes]
+        if step == 3:
+            opt.param_groups[0]["lr"] = 0.01  # exercises CORRECTED (lr / peak_lr)
+            ref.cfg.lr = 0.01
+        for q, gr in zip(params, grads):
+            q.grad = gr.to(DEV)
+        opt.step()
+        ref.step([x.clone() for x in grads])
+    for q, r in zip(params, ref_p):
+        assert rel_err(q.detach().cpu(), r) < 1e-4
+
+
+def test_none_and_empty_gradients_mask_their_blocks():
+    """shampoo_distributor.py:269-277 / tests/distributed_shampoo_test.py:1533-1579."""
+    import optimizers_amd as oa
+
+    g = torch.Generator().manual_seed(3)
+    shapes = [(20, 12), (12,), (9, 9)]
+    init = [torch.randn(*s, generator=g) for s in shapes]
+    # epsilon is large enough that the few-gradient factors of the small blocks are well posed
+    kw = dict(lr=0.01, betas=(0.9, 0.99), epsilon=1e-2, max_preconditioner_dim=8, precondition_frequency=1,
+              start_preconditioning_step=2)
+    params = [torch.nn.Parameter(t.clone().to(DEV)) for t in init]
+    opt = oa.DistributedShampoo(params, preconditioner_config=_newton(inverse_exponent_override={1: {0: 0.0}}),
+                                grafting_config=oa.AdaGradPreconditionerConfig(epsilon=1e-8), **kw)
+    ref_p = [t.clone() for t in init]
+    ref = _oracle(ref_p, inverse_exponent_override={1: {0: 0.0}}, grafting="adagrad", grafting_epsilon=1e-8, **kw)
+    masks = [(1, 1, 1), (1, 0, 1), (0, 1, 1), (1, 1, 0), (1, 1, 1), (0, 0, 0), (1, 1, 1)]
+    for m in masks:
+        grads = [torch.randn(*s, generator=g) if keep else None for s, keep in zip(shapes, m)]
+        for q, gr in zip(params, grads):
+            q.grad = None if gr is None else gr.to(DEV)
+        before = [q.detach().clone() for q in params]
+        opt.step()
+        ref.step([None if x is None else x.clone() for x in grads])
+        for q, b, keep in zip(params, before, m):
+            if not keep:
+                assert torch.equal(q.detach(), b)
+    for q, r in zip(params, ref_p):
+        assert rel_err(q.detach().cpu(), r) < 1e-4
+    assert int(opt.state[params[0]]["step"]) == len(masks) == int(ref.step_t)
+
+
+def test_state_dict_layout_and_round_trip():
+    """Golden layout tests/distributed_shampoo_test.py:516-622; resume must continue bit-identically."""
+    import optimizers_amd as oa
+
+    def make(init):
+        ps = [torch.nn.Parameter(t.clone().to(DEV)) for t in init]
+        o = oa.DistributedShampoo(ps, lr=0.01, betas=(0.9, 0.99), epsilon=1e-6, max_preconditioner_dim=5,
+                                  precondition_frequency=1, start_preconditioning_step=1,
+                                  preconditioner_config=_newton(), grafting_config=oa.AdaGradPreconditionerConfig(epsilon=1e-3))
+        return ps, o
+
+    g = torch.Generator().manual_seed(5)
+    init = [torch.randn(5, 10, generator=g)]
+    params, opt = make(init)
+    sd = opt.state_dict()
+    blk = sd["state"][0]["block_0"]
+    assert set(sd["state"][0]) == {"block_0", "block_1", "step"}
+    assert set(blk) == {"shampoo", "adagrad", "filtered_grad"}
+    assert set(blk["shampoo"]) == {"factor_matrices", "inv_factor_matrices"}
+    assert blk["shampoo"]["factor_matrices"][0].shape == (15,) and blk["adagrad"].shape == (5, 5)
+    eye = torch.zeros(15)
+    eye[[0, 5, 9, 12, 14]] = 1
+    assert torch.equal(blk["shampoo"]["inv_factor_matrices"][1].cpu(), eye)
+    assert sd["param_groups"][0]["beta3"] == 0.9 and sd["param_groups"][0]["start_preconditioning_step"] == 1
+    grads = [torch.randn(5, 10, generator=g) for _ in range(6)]
+    for gr in grads[:3]:
+        params[0].grad = gr.to(DEV)
+        opt.step()
+    saved = copy.deepcopy(opt.state_dict())
+    saved_w = params[0].detach().clone()
+    for gr in grads[3:]:
+        params[0].grad = gr.to(DEV)
+        opt.step()
+    # resume in a fresh optimizer
+    params2, opt2 = make([saved_w.cpu()])
+    opt2.load_state_dict(saved)
+    assert int(opt2.state[params2[0]]["step"]) == 3
+    for gr in grads[3:]:
+        params2[0].grad = gr.to(DEV)
+        opt2.step()
+    assert torch.equal(params2[0].detach(), params[0].detach())
+
+
+def test_two_param_groups_and_streams():
+    import optimizers_amd as oa
+
+    g = torch.Generator().manual_seed(8)
+    a0, b0 = torch.randn(24, 16, generator=g), torch.randn(16, 40, generator=g)
+    pa, pb = torch.nn.Parameter(a0.clone().to(DEV)), torch.nn.Parameter(b0.clone().to(DEV))
+    opt = oa.DistributedShampoo(
+        [{"params": [pa], "lr": 0.01}, {"params": [pb], "lr": 0.03, "max_preconditioner_dim": 8}],
+        betas=(0.9, 0.99), epsilon=1e-6, max_preconditioner_dim=16, precondition_frequency=1,
+        start_preconditioning_step=2, preconditioner_config=_newton(), grafting_config=oa.AdamPreconditionerConfig(beta2=0.99, epsilon=1e-8))
+    ra, rb = [a0.clone()], [b0.clone()]
+    common = dict(betas=(0.9, 0.99), epsilon=1e-6, precondition_frequency=1, start_preconditioning_step=2,
+                  grafting="adam", grafting_beta2=0.99, grafting_epsilon=1e-8)
+    oa_ = _oracle(ra, lr=0.01, max_preconditioner_dim=16, **common)
+    ob_ = _oracle(rb, lr=0.03, max_preconditioner_dim=8, **common)
+    for _ in range(5):
+        ga, gb = torch.randn(24, 16, generator=g), torch.randn(16, 40, generator=g)
+        pa.grad, pb.grad = ga.to(DEV), gb.to(DEV)
+        opt.step()
+        oa_.step([ga.clone()])
+        ob_.step([gb.clone()])
+    assert rel_err(pa.detach().cpu(), ra[0]) < 1e-4 and rel_err(pb.detach().cpu(), rb[0]) < 1e-4
+
+
+def test_non_integer_root_fails_like_reference_after_tolerance():
+    """matrix_functions.py:670-673 raises inside the tolerated region of shampoo_preconditioner_list.py:430-443."""
+    import optimizers_amd as oa
+
+    p = torch.nn.Parameter(torch.randn(6, 6).to(DEV))
+    opt = oa.DistributedShampoo([p], lr=0.01, betas=(0.0, 1.0), epsilon=1e-6, max_preconditioner_dim=8,
+                                precondition_frequency=1, start_preconditioning_step=1,
+                                preconditioner_config=_newton(inverse_exponent_override={2: 0.3}))
+    for i in range(3):
+        p.grad = torch.randn(6, 6).to(DEV)
+        opt.step()  # tolerated: 3 failures
+    p.grad = torch.randn(6, 6).to(DEV)
+    with pytest.raises(ValueError, match="exceeded the allowed tolerance"):
+        opt.step()
+
+
+def test_nonfinite_gradient_raises_preconditioner_value_error():
+    import optimizers_amd as oa
+
+    p = torch.nn.Parameter(torch.randn(8, 8).to(DEV))
+    opt = oa.DistributedShampoo([p], lr=0.01, betas=(0.9, 0.99), epsilon=1e-6, max_preconditioner_dim=8,
+                                precondition_frequency=1, start_preconditioning_step=1, preconditioner_config=_newton())
+    g = torch.randn(8, 8)
+    g[2, 3] = float("nan")
+    p.grad = g.to(DEV)
+    with pytest.raises(oa.PreconditionerValueError, match="Encountered nan/inf values in factor matrix 0.block_0.0"):
+        opt.step()
+    opt2 = oa.DistributedShampoo([p], lr=0.01, epsilon=1e-6, preconditioner_config=_newton(),
+                                 shampoo_runtime_config=oa.ShampooRuntimeConfig(eager_nan_check=True))
+    with pytest.raises(AssertionError, match="Encountered gradient containing NaN/Inf"):
+        opt2.step()
+
+
+def test_large_ragged_kronecker_update_and_precondition():
+    """GPT-2-like ragged blocks (81x768, 256x768, 1024x768) for two steps against the oracle."""
+    import optimizers_amd as oa
+
+    g = torch.Generator().manual_seed(21)
+    shapes = [(1105, 768), (768, 1300), (768,)]
+    init = [0.02 * torch.randn(*s, generator=g) for s in shapes]
+    # epsilon = 1e-3 keeps the rank-deficient factors (81 or 337 rows feeding a 768 x 768 factor) well posed;
+    # with 1e-12 the reference's Newton iteration returns rounding noise or raises on them
+    kw = dict(lr=1e-3, betas=(0.9, 0.999), epsilon=1e-3, max_preconditioner_dim=1024, precondition_frequency=1,
+              start_preconditioning_step=2)
+    params = [torch.nn.Parameter(t.clone().to(DEV)) for t in init]
+    opt = oa.DistributedShampoo(params, preconditioner_config=_newton(inverse_exponent_override={1: {0: 0.0}}),
+                                grafting_config=oa.AdamPreconditionerConfig(beta2=0.999, epsilon=1e-8), **kw)
+    ref_p = [t.clone() for t in init]
+    ref = _oracle(ref_p, inverse_exponent_override={1: {0: 0.0}}, grafting="adam", grafting_beta2=0.999, grafting_epsilon=1e-8, **kw)
+    for _ in range(3):
+        grads = [0.02 * torch.randn(*s, generator=g) for s in shapes]
+        for q, gr in zip(params, grads):
+            q.grad = gr.to(DEV)
+        opt.step()
+        ref.step([x.clone() for x in grads])
+    ng = opt._groups[0]
+    for k, bi in enumerate(ng.native_index):
+        spec = ng.block_specs[bi]
+        st = opt.state[params[spec.param_index]][spec.block_key]
+        for j, f in enumerate(ref.state[bi]["factors"]):
+            assert rel_err(st["shampoo"]["factor_matrices"][j].cpu(), f) < 1e-5
+        for j, f in enumerate(ref.state[bi]["inv"]):
+            assert rel_err(st["shampoo"]["inv_factor_matrices"][j].cpu(), f) < 1e-3
+    for q, r in zip(params, ref_p):
+        assert rel_err(q.detach().cpu(), r) < 1e-4
