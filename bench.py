@@ -151,6 +151,9 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="llama3_8b_layer", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--symmetric-newton", action="store_true",
+                    help="compute only the upper triangle of every coupled-Newton product and mirror it (not the "
+                         "reference's arithmetic on ill-conditioned factors; off by default)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB copy kernel (sa::copy_kernel) so that rocprofv3 --pmc FETCH_SIZE / "
                          "WRITE_SIZE readings can be scaled against a kernel of known traffic")
@@ -168,6 +171,7 @@ def main() -> None:
     device = torch.device("cuda:0")
     workload = WORKLOADS[args.workload]
     lib = native.load()
+    lib.sa_set_symmetric_newton(1 if args.symmetric_newton else 0)
     params, opt = build(workload, device)
     n_params = sum(p.numel() for p in params)
 
@@ -193,6 +197,7 @@ def main() -> None:
     lib.sa_set_profiling(1)
     phases = ("newton_gemm", "syrk", "precondition_gemm", "grafting", "apply")
     acc = {ph: [0.0, 0.0, 0] for ph in phases}  # ms, work, launches
+    executed = 0.0
     iters = []
     t0 = time.perf_counter()
     for i in range(args.warmup, total):
@@ -204,6 +209,7 @@ def main() -> None:
                 acc[ph][0] += ms
                 acc[ph][1] += lib.sa_phase_flops(ph.encode())
                 acc[ph][2] += lib.sa_phase_launches(ph.encode())
+        executed += max(lib.sa_phase_executed_flops(b"newton_gemm"), 0.0)
         iters.append(list(opt._groups[0].last_newton_iterations))
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
@@ -220,6 +226,11 @@ def main() -> None:
         "unit": "TFLOP/s",
         "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
         "traffic": None,
+        # `achieved` bills the full-GEMM algorithmic flops (2 d^3 per product); `executed_frac` is what the
+        # matrix cores really sustained (they differ only with --symmetric-newton and through tile padding).
+        "symmetric_products": bool(args.symmetric_newton),
+        "executed_TFLOP/s": executed / (ng_ms * 1e-3) / 1e12 if ng_ms > 0 else 0.0,
+        "executed_frac": executed / (ng_ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS if ng_ms > 0 else 0.0,
         "avg_launch_ms": ng_ms / max(ng_launches, 1),
         "flop_per_launch": ng_flops / max(ng_launches, 1),
         "launches": ng_launches,

@@ -163,7 +163,16 @@ int32_t sa_copy_f32(const float* src, float* dst, int64_t n, void* stream);
 int32_t sa_set_profiling(int32_t enabled);
 double sa_phase_ms(const char* phase);
 double sa_phase_flops(const char* phase); /* algorithmic flops (or bytes for HBM-bound phases) of that call */
-int32_t sa_phase_launches(const char* phase); /* kernel launches the phase issued in that call */
+int32_t sa_phase_launches(const char* phase);
+double sa_phase_executed_flops(const char* phase); /* flops actually issued by "newton_gemm" (symmetric products are halved) */
+
+/* Coupled Newton products are symmetric in exact arithmetic (every operand is a polynomial in the
+ * factor).  When enabled only the tiles on or above the diagonal of each product are computed and
+ * mirrored (1.9x fewer MFMA flops at d = 2048).  Off by default: every product is a full GEMM like the
+ * reference's `@` (matrix_functions.py:426-427).  Measured: identical results (1e-6) on well conditioned
+ * factors, but on factors with condition number > 1e5 the mirrored iteration deviates ~10x more from
+ * exact arithmetic than the reference does.  Process-wide switch. */
+int32_t sa_set_symmetric_newton(int32_t enabled); /* kernel launches the phase issued in that call */
 
 #ifdef __cplusplus
 }

@@ -145,7 +145,10 @@ __device__ __forceinline__ float wave_max_nan(float v) {
   return v;
 }
 
-template <int AL, int BL, int EPI, bool EDGE>
+// TRI: the product is known to be symmetric (coupled Newton: every operand is a polynomial in the
+// same matrix).  Only tiles on or above the diagonal are computed; an off-diagonal tile is stored
+// twice, as computed and transposed, which halves the MFMA work of a square product.
+template <int AL, int BL, int EPI, bool EDGE, bool TRI = (EPI == EPI_SYRK_EMA)>
 __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(
     const GemmProblem* __restrict__ problems, int n_problems, int total_tiles, GemmScalars sc) {
   __shared__ __attribute__((aligned(16))) float As[2][BK * LDS_STRIDE];
@@ -169,7 +172,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(
   int tm, tn;
   {
     int t = logical - P.tile_begin;
-    if (EPI == EPI_SYRK_EMA) {
+    if (TRI) {
       // upper-triangular tile enumeration, row by row
       tm = 0;
       int rowlen = P.tiles_n;
@@ -272,6 +275,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(
         const float v = acc[i][j][e];
         if (EPI == EPI_STORE) {
           if (!EDGE || (row < M && col < N)) C[(long long)row * ldc + col] = v;
+          if (TRI && tm != tn && (!EDGE || (row < M && col < N))) C[(long long)col * ldc + row] = v;
         } else if (EPI == EPI_STORE_SQNORM) {
           if (!EDGE || (row < M && col < N)) {
             C[(long long)row * ldc + col] = v;
@@ -291,6 +295,10 @@ __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(
           float mp = __fmul_rn(v, sc.mp_scale);
           if (row == col && row < P.d) mp = __fadd_rn(mp, sc.mp_diag);
           P.C2[(long long)row * ldc + col] = mp;
+          if (TRI && tm != tn) {
+            C[(long long)col * ldc + row] = v;
+            P.C2[(long long)col * ldc + row] = mp;
+          }
           if (row < P.d && col < P.d) {
             const float dv = fabsf(v - (row == col ? 1.0f : 0.0f));
             if (dv != dv) local_nan = true;

@@ -127,11 +127,11 @@ struct GemmTable {
 
 inline int vec_ok(const void* p, long long ld) { return ((reinterpret_cast<uintptr_t>(p) & 15) == 0 && (ld % 4) == 0) ? 1 : 0; }
 
-template <int AL, int BL, int EPI, bool EDGE>
+template <int AL, int BL, int EPI, bool EDGE, bool TRI = (EPI == EPI_SYRK_EMA)>
 int launch_gemm(const GemmTable& g, GemmScalars sc, hipStream_t s) {
   if (g.total_tiles == 0) return SA_OK;
   const int per = (g.total_tiles + NUM_XCD - 1) / NUM_XCD;
-  hipLaunchKernelGGL((grouped_gemm_kernel<AL, BL, EPI, EDGE>), dim3(per * NUM_XCD), dim3(GEMM_THREADS), 0, s,
+  hipLaunchKernelGGL((grouped_gemm_kernel<AL, BL, EPI, EDGE, TRI>), dim3(per * NUM_XCD), dim3(GEMM_THREADS), 0, s,
                      g.t.dev, (int)g.t.n, g.total_tiles, sc);
   HIPCHECK(hipGetLastError());
   return SA_OK;
@@ -147,10 +147,12 @@ GemmScalars unit_scalars() { return GemmScalars{1.0f, 1.0f, 1.0f, 0.0f, 0.0f, 0.
 struct Phase {
   std::vector<std::pair<hipEvent_t, hipEvent_t>> spans;
   size_t used = 0;
-  double work = 0.0;  // flops or bytes
+  double work = 0.0;      // algorithmic flops or bytes
+  double executed = 0.0;  // flops actually issued (differs when symmetric products are halved)
   int launches = 0;
 };
 bool g_profiling = false;
+bool g_symmetric_newton = false;
 std::map<std::string, Phase> g_phases;
 
 struct Span {
@@ -160,7 +162,7 @@ struct Span {
   Span(const char* name, hipStream_t st, double work, int launches, bool reset) {
     if (!g_profiling) return;
     ph = &g_phases[name];
-    if (reset) { ph->used = 0; ph->work = 0.0; ph->launches = 0; }
+    if (reset) { ph->used = 0; ph->work = 0.0; ph->executed = 0.0; ph->launches = 0; }
     if (ph->used == ph->spans.size()) {
       hipEvent_t a, b;
       if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) { ph = nullptr; return; }
@@ -470,6 +472,14 @@ double sa_phase_flops(const char* phase) {
   auto it = g_phases.find(phase ? phase : "");
   return it == g_phases.end() ? -1.0 : it->second.work;
 }
+double sa_phase_executed_flops(const char* phase) {
+  auto it = g_phases.find(phase ? phase : "");
+  return it == g_phases.end() ? -1.0 : it->second.executed;
+}
+int32_t sa_set_symmetric_newton(int32_t enabled) {
+  g_symmetric_newton = enabled != 0;
+  return SA_OK;
+}
 int32_t sa_phase_launches(const char* phase) {
   auto it = g_phases.find(phase ? phase : "");
   return it == g_phases.end() ? -1 : it->second.launches;
@@ -751,6 +761,7 @@ static int newton_batch(sa_plan* p, const std::vector<int>& ids, int root, float
     }
   }
   if (std::max(squarings - 1, 0) + (cube ? 1 : 0) > 4) return fail(SA_ERR_UNSUPPORTED, "root too large for the power chain");
+  const bool sym = g_symmetric_newton;
   const float alpha = (float)(-1.0 / root);          // M.mul(alpha)
   const float one_minus_alpha = (float)(1.0 - (-1.0 / root));  // .add_(I, alpha = 1 - alpha)
 
@@ -807,27 +818,27 @@ static int newton_batch(sa_plan* p, const std::vector<int>& ids, int root, float
       float* S1 = newton_buf(p, NB_S1, f);
       float* S2 = newton_buf(p, NB_S2, f);
       // launch A: X <- X M_p, and the first squaring if the root needs one
-      p->nt_a[par].add(prob(f, X, Mp, Xn), false);
-      if (squarings >= 1) p->nt_a[par].add(prob(f, Mp, Mp, S1), false);
+      p->nt_a[par].add(prob(f, X, Mp, Xn), sym);
+      if (squarings >= 1) p->nt_a[par].add(prob(f, Mp, Mp, S1), sym);
       // remaining chain reads only S1/S2/Mp of this parity; build it for parity-specific Mp when cube
       const float* cur = (squarings >= 1) ? S1 : Mp;
       int slot = par * 4;  // nt_pow[0..3] parity 0, [4..7] parity 1
       float* pong[2] = {S2, S1};
       int which = 0;
       for (int q = 1; q < squarings; ++q) {
-        p->nt_pow[slot++].add(prob(f, cur, cur, pong[which]), false);
+        p->nt_pow[slot++].add(prob(f, cur, cur, pong[which]), sym);
         cur = pong[which];
         which ^= 1;
       }
       if (cube) {
-        p->nt_pow[slot++].add(prob(f, cur, Mp, pong[which]), false);
+        p->nt_pow[slot++].add(prob(f, cur, Mp, pong[which]), sym);
         cur = pong[which];
       }
       power = cur;
       GemmProblem m = prob(f, power, M, Mn);
       m.C2 = Mpn;
       m.err_bits = p->d_err + ids[i];
-      p->nt_m[par].add(m, false);
+      p->nt_m[par].add(m, sym);
     }
   }
   for (int par = 0; par < 2; ++par) { SACHECK(p->nt_a[par].commit(s)); SACHECK(p->nt_m[par].commit(s)); }
@@ -847,18 +858,31 @@ static int newton_batch(sa_plan* p, const std::vector<int>& ids, int root, float
   msc.mp_diag = one_minus_alpha;
   const int gemms_per_iter = 1 + squarings + (cube ? 1 : 0) + 1;
   for (int it = 0; it < max_iter; ++it) {
-    double flops = 0.0;
+    double flops = 0.0, executed = 0.0;
     int live = 0;
     for (int i = 0; i < n; ++i)
-      if (h_active[ids[i]]) { const double d = p->factors[ids[i]].d; flops += 2.0 * d * d * d * gemms_per_iter; ++live; }
+      if (h_active[ids[i]]) {
+        const Factor& f = p->factors[ids[i]];
+        const double d = f.d, t = f.dpad / BM;
+        flops += 2.0 * d * d * d * gemms_per_iter;
+        executed += 2.0 * BM * BN * (double)f.dpad * (sym ? t * (t + 1) / 2 : t * t) * gemms_per_iter;
+        ++live;
+      }
     if (!live) break;
     {
       int nl = 2;
       for (int k = 0; k < 4; ++k) nl += p->nt_pow[parity * 4 + k].total_tiles ? 1 : 0;
       Span span("newton_gemm", s, flops, nl, false);
-      SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false>(p->nt_a[parity], unit, s)));
-      for (int k = 0; k < 4; ++k) SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false>(p->nt_pow[parity * 4 + k], unit, s)));
-      SACHECK((launch_gemm<A_MK, B_KN, EPI_NEWTON_M, false>(p->nt_m[parity], msc, s)));
+      if (g_profiling) g_phases["newton_gemm"].executed += executed;
+      if (sym) {
+        SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, true>(p->nt_a[parity], unit, s)));
+        for (int k = 0; k < 4; ++k) SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, true>(p->nt_pow[parity * 4 + k], unit, s)));
+        SACHECK((launch_gemm<A_MK, B_KN, EPI_NEWTON_M, false, true>(p->nt_m[parity], msc, s)));
+      } else {
+        SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, false>(p->nt_a[parity], unit, s)));
+        for (int k = 0; k < 4; ++k) SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, false>(p->nt_pow[parity * 4 + k], unit, s)));
+        SACHECK((launch_gemm<A_MK, B_KN, EPI_NEWTON_M, false, false>(p->nt_m[parity], msc, s)));
+      }
       *flops_acc += flops;
       *launches_acc += nl;
     }
@@ -879,7 +903,7 @@ int32_t sa_compute_root_inverses_newton(sa_plan* p, float bias_correction2, floa
   SACHECK(ensure_tables(p, nullptr, s));
   const int F = (int)p->factors.size();
   if (F == 0) return SA_OK;
-  if (g_profiling) { Phase& ph = g_phases["newton_gemm"]; ph.used = 0; ph.work = 0.0; ph.launches = 0; }
+  if (g_profiling) { Phase& ph = g_phases["newton_gemm"]; ph.used = 0; ph.work = 0.0; ph.executed = 0.0; ph.launches = 0; }
 
   // factors of masked blocks are left alone (shampoo_preconditioner_list.py:1426)
   std::vector<int> todo;

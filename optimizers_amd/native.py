@@ -31,7 +31,7 @@ EXPORTS = (
     "sa_plan_bind_gradients", "sa_add_l2_regularization", "sa_update_factor_matrices",
     "sa_compute_root_inverses_newton", "sa_update_grafting_and_filtered_grad", "sa_precondition",
     "sa_apply_update", "sa_grafting_only_step", "sa_plan_read_norms", "sa_plan_read_preconditioned",
-    "sa_gemm_f32", "sa_copy_f32", "sa_set_profiling", "sa_phase_ms", "sa_phase_flops", "sa_phase_launches",
+    "sa_gemm_f32", "sa_copy_f32", "sa_set_profiling", "sa_phase_ms", "sa_phase_flops", "sa_phase_launches", "sa_phase_executed_flops", "sa_set_symmetric_newton",
 )
 
 
@@ -116,6 +116,9 @@ def load() -> ctypes.CDLL:
     lib.sa_phase_ms.restype = c_double
     lib.sa_phase_flops.argtypes = [c_char_p]
     lib.sa_phase_flops.restype = c_double
+    lib.sa_phase_executed_flops.argtypes = [c_char_p]
+    lib.sa_phase_executed_flops.restype = c_double
+    lib.sa_set_symmetric_newton.argtypes = [c_int32]
     lib.sa_phase_launches.argtypes = [c_char_p]
     lib.sa_phase_launches.restype = c_int32
     for name in EXPORTS:
