@@ -123,6 +123,16 @@ int32_t sa_compute_root_inverses_newton(sa_plan* plan, float bias_correction2, f
                                         int32_t max_iterations, float tolerance,
                                         int32_t* iterations_out, int32_t* status_out, void* stream);
 
+/* Batched symmetric eigendecomposition root inverse on every factor (two-sided block Jacobi):
+ * A = unpack(factor / bias_correction2) (+ epsilon I when perturb_before_computation), (lambda, Q) = eigh(A),
+ * spectrum shifted as the reference does when min(lambda) < epsilon, X = Q diag(lambda^(-1/root)) Q^T
+ * (matrix_functions.py:306-366, 698-770, 179-279 via shampoo_preconditioner_list.py:314-443, 631-680).
+ * roots: host array, one (possibly fractional) root per factor.  sweeps_out / status_out as for the Newton call;
+ * SA_FACTOR_NOT_CONVERGED means rotations were still being applied in sweep max_sweeps. */
+int32_t sa_compute_root_inverses_eigh(sa_plan* plan, float bias_correction2, float epsilon, const float* roots,
+                                      int32_t perturb_before_computation, int32_t max_sweeps,
+                                      int32_t* sweeps_out, int32_t* status_out, void* stream);
+
 /* Grafting second moment, filtered gradient and the grafted direction's squared norm per block
  * (adagrad_preconditioner_list.py:122-162, distributed_shampoo.py:1162-1199, 1110-1114). */
 int32_t sa_update_grafting_and_filtered_grad(sa_plan* plan, const sa_step_scalars* s, void* stream);

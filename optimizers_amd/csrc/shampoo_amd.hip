@@ -13,6 +13,7 @@
 #include <vector>
 
 #include "../../include/shampoo_amd.h"
+#include "eigh.h"
 #include "elementwise.h"
 #include "gemm.h"
 
@@ -221,6 +222,11 @@ struct sa_plan {
   Table<SymFactor> t_sym;
   Table<NormJob> t_normjobs;
   Table<int> t_ids;
+  Table<JacobiFactor> t_jacobi;
+  Table<int2> t_sched;
+  Table<EigInit> t_eiginit;
+  Table<EigFinal> t_eigfinal;
+  GemmTable eig_gemm;
   int n_active_blocks = 0;
 
   // Newton control state (device) and pinned readback
@@ -566,6 +572,7 @@ void sa_plan_destroy(sa_plan* p) {
     g->t.destroy();
   for (auto& g : p->nt_pow) g.t.destroy();
   p->t_sym.destroy(); p->t_normjobs.destroy(); p->t_ids.destroy();
+  p->t_jacobi.destroy(); p->t_sched.destroy(); p->t_eiginit.destroy(); p->t_eigfinal.destroy(); p->eig_gemm.t.destroy();
   for (void* q : {(void*)p->d_err, (void*)p->d_active, (void*)p->d_iters, (void*)p->d_final_parity,
                   (void*)p->d_final_err, (void*)p->d_flags, (void*)p->d_nactive})
     if (q) (void)hipFree(q);
@@ -895,43 +902,35 @@ static int newton_batch(sa_plan* p, const std::vector<int>& ids, int root, float
   return SA_OK;
 }
 
-int32_t sa_compute_root_inverses_newton(sa_plan* p, float bias_correction2, float epsilon, int32_t max_iterations,
-                                        float tolerance, int32_t* iterations_out, int32_t* status_out, void* stream) {
-  if (!p || !iterations_out || !status_out) return fail(SA_ERR_INVALID, "sa_compute_root_inverses_newton: NULL argument");
-  if (!(bias_correction2 != 0.0f) || max_iterations < 0) return fail(SA_ERR_INVALID, "bad bias correction or max_iterations");
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  SACHECK(ensure_tables(p, nullptr, s));
+// Shared front end of the root-inverse paths: which factors are to be recomputed, Frobenius norm
+// partials of the ridged, bias-corrected factor, and the finiteness check of the input.  On return `todo`
+// holds the factors that precede the first non-finite one (the reference raises there).
+static int root_inverse_prologue(sa_plan* p, float bias_correction2, float norm_eps, int32_t* iterations_out,
+                                 int32_t* status_out, hipStream_t s, std::vector<int>* todo) {
   const int F = (int)p->factors.size();
-  if (F == 0) return SA_OK;
-  if (g_profiling) { Phase& ph = g_phases["newton_gemm"]; ph.used = 0; ph.work = 0.0; ph.executed = 0.0; ph.launches = 0; }
-
-  // factors of masked blocks are left alone (shampoo_preconditioner_list.py:1426)
-  std::vector<int> todo;
+  todo->clear();
   for (int i = 0; i < F; ++i) {
     iterations_out[i] = 0;
     status_out[i] = SA_FACTOR_SKIPPED;
-    if (block_active(p, p->factors[i].block)) todo.push_back(i);
+    if (block_active(p, p->factors[i].block)) todo->push_back(i);
   }
-  if (todo.empty()) return SA_OK;
+  if (todo->empty()) return SA_OK;
   // factors that are not recomputed below must keep a valid dense copy of their stored inverse
   SACHECK(refresh_inverse_cache(p, s));
-
   HIPCHECK(hipMemsetAsync(p->d_flags, 0, F * sizeof(int), s));
   HIPCHECK(hipMemsetAsync(p->d_err, 0, F * sizeof(int), s));
   HIPCHECK(hipMemsetAsync(p->d_iters, 0, F * sizeof(int), s));
   HIPCHECK(hipMemsetAsync(p->d_active, 0, F * sizeof(int), s));
   HIPCHECK(hipMemsetAsync(p->d_final_parity, 0, F * sizeof(int), s));
-
-  // 1. Frobenius norms of the ridged, bias-corrected factors + finiteness of the input
-  SACHECK(p->t_normjobs.begin(todo.size()));
+  SACHECK(p->t_normjobs.begin(todo->size()));
   int chunks = 0;
-  for (size_t i = 0; i < todo.size(); ++i) {
-    const Factor& f = p->factors[todo[i]];
+  for (size_t i = 0; i < todo->size(); ++i) {
+    const Factor& f = p->factors[(*todo)[i]];
     NormJob& J = p->t_normjobs.host[i];
     std::memset(&J, 0, sizeof(J));
     J.src = f.factor;
     J.partial = p->f(p->off_norm_partial) + f.norm_off;
-    J.nonfinite = p->d_flags + todo[i];
+    J.nonfinite = p->d_flags + (*todo)[i];
     J.d = f.d; J.dpad = f.dpad; J.dense = 0;
     J.chunk_begin = chunks;
     J.n_chunks = f.norm_chunks;
@@ -939,50 +938,33 @@ int32_t sa_compute_root_inverses_newton(sa_plan* p, float bias_correction2, floa
     chunks += f.norm_chunks;
   }
   SACHECK(p->t_normjobs.upload(s));
-  hipLaunchKernelGGL((factor_norm_kernel<false>), dim3(chunks), dim3(256), 0, s, p->t_normjobs.dev, (int)todo.size(),
-                     bias_correction2, epsilon);
+  hipLaunchKernelGGL((factor_norm_kernel<false>), dim3(chunks), dim3(256), 0, s, p->t_normjobs.dev, (int)todo->size(),
+                     bias_correction2, norm_eps);
   HIPCHECK(hipGetLastError());
   int* h_flags = p->h_pinned + F;
   HIPCHECK(hipMemcpyAsync(h_flags, p->d_flags, F * sizeof(int), hipMemcpyDeviceToHost, s));
   HIPCHECK(hipStreamSynchronize(s));
-  // the reference walks factors in order and raises at the first non-finite one
-  size_t limit = todo.size();
-  for (size_t i = 0; i < todo.size(); ++i)
-    if (h_flags[todo[i]]) { status_out[todo[i]] = SA_FACTOR_INPUT_NONFINITE; limit = i; break; }
-  todo.resize(limit);
-  if (todo.empty()) return SA_OK;
+  size_t limit = todo->size();
+  for (size_t i = 0; i < todo->size(); ++i)
+    if (h_flags[(*todo)[i]]) { status_out[(*todo)[i]] = SA_FACTOR_INPUT_NONFINITE; limit = i; break; }
+  todo->resize(limit);
+  return SA_OK;
+}
 
-  // 2. iterate, one batch per distinct root
-  std::vector<int> ones(F, 0);
-  for (int i : todo) ones[i] = 1;
-  HIPCHECK(hipMemcpyAsync(p->d_active, ones.data(), F * sizeof(int), hipMemcpyHostToDevice, s));
-  HIPCHECK(hipStreamSynchronize(s));
-  std::map<int, std::vector<int>> by_root;
-  for (int i : todo) by_root[p->factors[i].root].push_back(i);
-  double flops = 0.0;
-  int launches = 0;
-  for (auto& kv : by_root)
-    SACHECK(newton_batch(p, kv.second, kv.first, epsilon, bias_correction2, max_iterations, tolerance, s, &flops, &launches));
-
-  // 3. read back iteration counts, final errors, parities
-  int* h_iters = p->h_pinned;
-  int* h_par = p->h_pinned + F;
-  float* h_err = reinterpret_cast<float*>(p->h_pinned + 2 * F);
+// Shared back end: finiteness of every result X (dense, dpad-strided), then pack + mirror the results that
+// precede the first non-finite one into inv_factor and the dense inverse cache.
+static int root_inverse_epilogue(sa_plan* p, const std::vector<int>& todo, const std::vector<const float*>& X,
+                                 int32_t* status_out, hipStream_t s, size_t* n_ok) {
+  const int F = (int)p->factors.size();
   int* h_bad = p->h_pinned + 3 * F;
-  HIPCHECK(hipMemcpyAsync(h_iters, p->d_iters, F * sizeof(int), hipMemcpyDeviceToHost, s));
-  HIPCHECK(hipMemcpyAsync(h_par, p->d_final_parity, F * sizeof(int), hipMemcpyDeviceToHost, s));
-  HIPCHECK(hipMemcpyAsync(h_err, p->d_final_err, F * sizeof(float), hipMemcpyDeviceToHost, s));
-  HIPCHECK(hipStreamSynchronize(s));
-
-  // 4. finiteness of every result
   HIPCHECK(hipMemsetAsync(p->d_flags, 0, F * sizeof(int), s));
   SACHECK(p->t_normjobs.begin(todo.size()));
-  chunks = 0;
+  int chunks = 0;
   for (size_t i = 0; i < todo.size(); ++i) {
     const Factor& f = p->factors[todo[i]];
     NormJob& J = p->t_normjobs.host[i];
     std::memset(&J, 0, sizeof(J));
-    J.src = newton_buf(p, h_par[todo[i]] ? NB_X1 : NB_X0, f);
+    J.src = X[i];
     J.partial = nullptr;
     J.nonfinite = p->d_flags + todo[i];
     J.d = f.d; J.dpad = f.dpad; J.dense = 1;
@@ -996,16 +978,10 @@ int32_t sa_compute_root_inverses_newton(sa_plan* p, float bias_correction2, floa
   HIPCHECK(hipGetLastError());
   HIPCHECK(hipMemcpyAsync(h_bad, p->d_flags, F * sizeof(int), hipMemcpyDeviceToHost, s));
   HIPCHECK(hipStreamSynchronize(s));
-
-  // 5. commit the results that precede the first non-finite one
   size_t ok = todo.size();
-  for (size_t i = 0; i < todo.size(); ++i) {
-    const int fi = todo[i];
-    iterations_out[fi] = h_iters[fi];
-    if (h_bad[fi]) { status_out[fi] = SA_FACTOR_RESULT_NONFINITE; ok = i; break; }
-    status_out[fi] = (h_err[fi] <= tolerance) ? SA_FACTOR_OK : SA_FACTOR_NOT_CONVERGED;
-  }
-  for (size_t i = ok + 1; i < todo.size(); ++i) iterations_out[todo[i]] = h_iters[todo[i]];
+  for (size_t i = 0; i < todo.size(); ++i)
+    if (h_bad[todo[i]]) { status_out[todo[i]] = SA_FACTOR_RESULT_NONFINITE; ok = i; break; }
+  *n_ok = ok;
   if (ok > 0) {
     SACHECK(p->t_sym.begin(ok));
     int tiles = 0;
@@ -1013,7 +989,7 @@ int32_t sa_compute_root_inverses_newton(sa_plan* p, float bias_correction2, floa
       const Factor& f = p->factors[todo[i]];
       SymFactor& S = p->t_sym.host[i];
       std::memset(&S, 0, sizeof(S));
-      S.dense_in = newton_buf(p, h_par[todo[i]] ? NB_X1 : NB_X0, f);
+      S.dense_in = X[i];
       S.packed_out = f.inv;
       S.dense_out[0] = p->f(p->off_inv_dense) + f.dense_off;
       S.d = f.d; S.dpad = f.dpad; S.tiles = f.dpad / ST; S.root = f.root; S.enabled = 1;
@@ -1025,6 +1001,221 @@ int32_t sa_compute_root_inverses_newton(sa_plan* p, float bias_correction2, floa
     HIPCHECK(hipGetLastError());
     HIPCHECK(hipStreamSynchronize(s));
   }
+  return SA_OK;
+}
+
+int32_t sa_compute_root_inverses_newton(sa_plan* p, float bias_correction2, float epsilon, int32_t max_iterations,
+                                        float tolerance, int32_t* iterations_out, int32_t* status_out, void* stream) {
+  if (!p || !iterations_out || !status_out) return fail(SA_ERR_INVALID, "sa_compute_root_inverses_newton: NULL argument");
+  if (!(bias_correction2 != 0.0f) || max_iterations < 0) return fail(SA_ERR_INVALID, "bad bias correction or max_iterations");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SACHECK(ensure_tables(p, nullptr, s));
+  const int F = (int)p->factors.size();
+  if (F == 0) return SA_OK;
+  if (g_profiling) { Phase& ph = g_phases["newton_gemm"]; ph.used = 0; ph.work = 0.0; ph.executed = 0.0; ph.launches = 0; }
+  std::vector<int> todo;
+  SACHECK(root_inverse_prologue(p, bias_correction2, epsilon, iterations_out, status_out, s, &todo));
+  if (todo.empty()) return SA_OK;
+
+  // iterate, one batch per distinct root
+  std::vector<int> ones(F, 0);
+  for (int i : todo) ones[i] = 1;
+  HIPCHECK(hipMemcpyAsync(p->d_active, ones.data(), F * sizeof(int), hipMemcpyHostToDevice, s));
+  HIPCHECK(hipStreamSynchronize(s));
+  std::map<int, std::vector<int>> by_root;
+  for (int i : todo) by_root[p->factors[i].root].push_back(i);
+  double flops = 0.0;
+  int launches = 0;
+  for (auto& kv : by_root)
+    SACHECK(newton_batch(p, kv.second, kv.first, epsilon, bias_correction2, max_iterations, tolerance, s, &flops, &launches));
+
+  // iteration counts, final errors, parities
+  std::vector<int> iters(F), par(F);
+  std::vector<float> errs(F);
+  HIPCHECK(hipMemcpyAsync(p->h_pinned, p->d_iters, F * sizeof(int), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipMemcpyAsync(p->h_pinned + F, p->d_final_parity, F * sizeof(int), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipMemcpyAsync(p->h_pinned + 2 * F, p->d_final_err, F * sizeof(float), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipStreamSynchronize(s));
+  std::memcpy(iters.data(), p->h_pinned, F * sizeof(int));
+  std::memcpy(par.data(), p->h_pinned + F, F * sizeof(int));
+  std::memcpy(errs.data(), p->h_pinned + 2 * F, F * sizeof(float));
+
+  std::vector<const float*> X(todo.size());
+  for (size_t i = 0; i < todo.size(); ++i) X[i] = newton_buf(p, par[todo[i]] ? NB_X1 : NB_X0, p->factors[todo[i]]);
+  size_t ok = 0;
+  SACHECK(root_inverse_epilogue(p, todo, X, status_out, s, &ok));
+  for (size_t i = 0; i < todo.size(); ++i) {
+    const int fi = todo[i];
+    iterations_out[fi] = iters[fi];
+    if (i < ok) status_out[fi] = (errs[fi] <= tolerance) ? SA_FACTOR_OK : SA_FACTOR_NOT_CONVERGED;
+  }
+  return SA_OK;
+}
+
+// --------------------------------------------------------------------------------------------
+// Batched eigendecomposition root inverse (block Jacobi)
+// --------------------------------------------------------------------------------------------
+
+int32_t sa_compute_root_inverses_eigh(sa_plan* p, float bias_correction2, float epsilon, const float* roots,
+                                      int32_t perturb_before_computation, int32_t max_sweeps, int32_t* sweeps_out,
+                                      int32_t* status_out, void* stream) {
+  if (!p || !roots || !sweeps_out || !status_out) return fail(SA_ERR_INVALID, "sa_compute_root_inverses_eigh: NULL argument");
+  if (!(bias_correction2 != 0.0f) || max_sweeps < 1) return fail(SA_ERR_INVALID, "bad bias correction or max_sweeps");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SACHECK(ensure_tables(p, nullptr, s));
+  const int F = (int)p->factors.size();
+  if (F == 0) return SA_OK;
+  for (int i = 0; i < F; ++i)
+    if (!(roots[i] > 0.0f)) return fail(SA_ERR_INVALID, "Root " + std::to_string(roots[i]) + " should be positive!");
+  const float ridge = perturb_before_computation ? epsilon : 0.0f;
+  std::vector<int> todo;
+  SACHECK(root_inverse_prologue(p, bias_correction2, ridge, sweeps_out, status_out, s, &todo));
+  if (todo.empty()) return SA_OK;
+  const int n = (int)todo.size();
+
+  // Frobenius norms (for the absolute rotation threshold)
+  std::vector<float> fro(n);
+  {
+    std::vector<float> partials(p->norm_partials_total);
+    HIPCHECK(hipMemcpyAsync(partials.data(), p->f(p->off_norm_partial), partials.size() * sizeof(float), hipMemcpyDeviceToHost, s));
+    HIPCHECK(hipStreamSynchronize(s));
+    for (int i = 0; i < n; ++i) {
+      const Factor& f = p->factors[todo[i]];
+      double acc = 0.0;
+      for (int c = 0; c < f.norm_chunks; ++c) acc += partials[f.norm_off + c];
+      fro[i] = (float)std::sqrt(acc);
+    }
+  }
+
+  // A <- unpack(factor / bc2) + ridge I, V <- I
+  SACHECK(p->t_eiginit.begin(n));
+  int tiles = 0;
+  for (int i = 0; i < n; ++i) {
+    const Factor& f = p->factors[todo[i]];
+    EigInit& J = p->t_eiginit.host[i];
+    std::memset(&J, 0, sizeof(J));
+    J.packed = f.factor;
+    J.A = newton_buf(p, NB_M0, f);
+    J.V = newton_buf(p, NB_X0, f);
+    J.d = f.d; J.dpad = f.dpad; J.tiles = f.dpad / 64; J.enabled = 1;
+    J.tile_begin = tiles;
+    tiles += J.tiles * J.tiles;
+  }
+  SACHECK(p->t_eiginit.upload(s));
+  hipLaunchKernelGGL(eig_init_kernel, dim3(tiles), dim3(256), 0, s, p->t_eiginit.dev, n, bias_correction2, ridge);
+  HIPCHECK(hipGetLastError());
+
+  // tournament schedules, one per distinct block count
+  std::map<int, size_t> sched_off;
+  std::vector<int2> sched;
+  int max_nb = 0, max_dpad = 0;
+  for (int i = 0; i < n; ++i) {
+    const int nb = p->factors[todo[i]].dpad / JB;
+    max_nb = std::max(max_nb, nb);
+    max_dpad = std::max(max_dpad, p->factors[todo[i]].dpad);
+    if (sched_off.count(nb)) continue;
+    sched_off[nb] = sched.size();
+    const int m = nb - 1;
+    for (int r = 0; r < nb - 1; ++r)
+      for (int k = 0; k < nb / 2; ++k) {
+        int a, b;
+        if (k == 0) { a = 0; b = (r % m) + 1; }
+        else { a = ((r + k) % m) + 1; b = ((r - k + m) % m) + 1; }
+        sched.push_back(make_int2(std::min(a, b), std::max(a, b)));
+      }
+  }
+  SACHECK(p->t_sched.begin(sched.size()));
+  std::memcpy(p->t_sched.host, sched.data(), sched.size() * sizeof(int2));
+  SACHECK(p->t_sched.upload(s));
+  SACHECK(p->t_jacobi.begin(n));
+  int pairs = 0;
+  for (int i = 0; i < n; ++i) {
+    const Factor& f = p->factors[todo[i]];
+    JacobiFactor& J = p->t_jacobi.host[i];
+    std::memset(&J, 0, sizeof(J));
+    J.A = newton_buf(p, NB_M0, f);
+    J.V = newton_buf(p, NB_X0, f);
+    J.U = newton_buf(p, NB_S2, f);
+    J.nb = f.dpad / JB;
+    J.sched = p->t_sched.dev + sched_off[J.nb];
+    J.rotations = p->d_iters + todo[i];
+    J.active = p->d_active + todo[i];
+    J.thr_abs = 1e-9f * fro[i];
+    J.thr_diag = 2.4e-7f * fro[i];  // 2^-22 ||A||_F: below the eigenvalue resolution of an fp32 matrix
+    J.d = f.d; J.dpad = f.dpad;
+    J.pair_begin = pairs;
+    pairs += J.nb / 2;
+  }
+  SACHECK(p->t_jacobi.upload(s));
+  std::vector<int> active(F, 0);
+  for (int i : todo) active[i] = 1;
+  HIPCHECK(hipMemcpyAsync(p->d_active, active.data(), F * sizeof(int), hipMemcpyHostToDevice, s));
+  HIPCHECK(hipStreamSynchronize(s));
+
+  int live = n;
+  for (int sweep = 0; sweep < max_sweeps && live > 0; ++sweep) {
+    HIPCHECK(hipMemsetAsync(p->d_iters, 0, F * sizeof(int), s));
+    double work = 0.0;
+    for (int i = 0; i < n; ++i)
+      if (active[todo[i]]) { const double d = p->factors[todo[i]].dpad; work += 3.0 * 2.0 * d * d * JP * (d / JB - 1); }
+    {
+      Span span("jacobi", s, work, 3 * (max_nb - 1), sweep == 0);
+      for (int r = 0; r < max_nb - 1; ++r) {
+        hipLaunchKernelGGL(jacobi_pivot_kernel, dim3(pairs), dim3(256), 0, s, p->t_jacobi.dev, n, r);
+        hipLaunchKernelGGL(jacobi_cols_kernel, dim3(pairs, max_dpad / 128, 2), dim3(256), 0, s, p->t_jacobi.dev, n, r);
+        hipLaunchKernelGGL(jacobi_rows_kernel, dim3(pairs, max_dpad / 128, 1), dim3(256), 0, s, p->t_jacobi.dev, n, r);
+      }
+      HIPCHECK(hipGetLastError());
+    }
+    HIPCHECK(hipMemcpyAsync(p->h_pinned, p->d_iters, F * sizeof(int), hipMemcpyDeviceToHost, s));
+    HIPCHECK(hipStreamSynchronize(s));
+    live = 0;
+    for (int i : todo) {
+      if (!active[i]) continue;
+      sweeps_out[i] = sweep + 1;
+      if (p->h_pinned[i] == 0) active[i] = 0; else ++live;
+    }
+    HIPCHECK(hipMemcpyAsync(p->d_active, active.data(), F * sizeof(int), hipMemcpyHostToDevice, s));
+    HIPCHECK(hipStreamSynchronize(s));
+  }
+
+  // X = V diag(f(lambda)) V^T
+  SACHECK(p->t_eigfinal.begin(n));
+  p->eig_gemm.clear();
+  int slabs = 0;
+  for (int i = 0; i < n; ++i) {
+    const Factor& f = p->factors[todo[i]];
+    EigFinal& J = p->t_eigfinal.host[i];
+    std::memset(&J, 0, sizeof(J));
+    J.A = newton_buf(p, NB_M0, f);
+    J.V = newton_buf(p, NB_X0, f);
+    J.Vs = newton_buf(p, NB_S1, f);
+    J.lambda_out = newton_buf(p, NB_MP0, f);
+    J.weight_out = newton_buf(p, NB_MP0, f) + f.dpad;
+    J.d = f.d; J.dpad = f.dpad;
+    J.exponent = -1.0f / roots[todo[i]];
+    J.row_begin = slabs;
+    J.enabled = 1;
+    slabs += f.dpad / 8;
+    GemmProblem q{};
+    q.A = J.Vs; q.B = J.V; q.C = newton_buf(p, NB_X1, f);
+    q.lda = q.ldb = q.ldc = f.dpad;
+    q.M = q.N = q.K = f.dpad;
+    q.a_vec = q.b_vec = 1;
+    p->eig_gemm.add(q, false);
+  }
+  SACHECK(p->t_eigfinal.upload(s));
+  SACHECK(p->eig_gemm.commit(s));
+  hipLaunchKernelGGL(eig_weights_kernel, dim3(n), dim3(256), 0, s, p->t_eigfinal.dev, epsilon, perturb_before_computation ? 1 : 0);
+  hipLaunchKernelGGL(eig_scale_cols_kernel, dim3(slabs), dim3(256), 0, s, p->t_eigfinal.dev, n);
+  HIPCHECK(hipGetLastError());
+  SACHECK((launch_gemm<A_MK, B_NK, EPI_STORE, false, false>(p->eig_gemm, unit_scalars(), s)));
+
+  std::vector<const float*> X(n);
+  for (int i = 0; i < n; ++i) X[i] = newton_buf(p, NB_X1, p->factors[todo[i]]);
+  size_t ok = 0;
+  SACHECK(root_inverse_epilogue(p, todo, X, status_out, s, &ok));
+  for (size_t i = 0; i < ok; ++i) status_out[todo[i]] = active[todo[i]] ? SA_FACTOR_NOT_CONVERGED : SA_FACTOR_OK;
   return SA_OK;
 }
 

@@ -26,6 +26,7 @@ from optimizers_amd.matrix_functions_types import (
     CoupledNewtonConfig,
     EigenConfig,
     EigendecompositionConfig,
+    PerturbationConfig,
     PseudoInverseConfig,
 )
 from optimizers_amd.shampoo_types import (
@@ -174,6 +175,8 @@ class _NativeGroup:
         descs = (native.BlockDesc * max(nb, 1))()
         self.factor_names: list[str] = []
         self.factor_block: list[int] = []
+        self.factor_roots: list[float] = []
+        self.use_eigh = isinstance(pc.amortized_computation_config, EigenConfig)
         self.bad_root_blocks: dict[int, str] = {}
         self.failed_counter: dict[int, int] = {}
         fi = 0
@@ -202,7 +205,10 @@ class _NativeGroup:
                 d.factor[dim] = f.data_ptr()
                 d.inv_factor[dim] = inv.data_ptr()
                 root = Fraction(self.roots[k][slot])
-                if root.denominator != 1:
+                self.factor_roots.append(float(self.roots[k][slot]))
+                if self.use_eigh:
+                    d.root[dim] = max(int(round(self.roots[k][slot])), 1)  # unused by the eigh path
+                elif root.denominator != 1:
                     # the reference raises inside matrix_inverse_root at every amortized step and
                     # tolerates it num_tolerated_failed_amortized_computations times
                     self.bad_root_blocks[k] = (
@@ -252,6 +258,7 @@ class _NativeGroup:
         self.status = (ctypes.c_int32 * max(self.n_factors, 1))()
         self.grad_ptrs = (ctypes.c_void_p * max(nb, 1))()
         self.last_newton_iterations: list[int] = []
+        self.max_jacobi_sweeps = 16
 
         # one CPU step counter per group, aliased under every parameter (distributed_shampoo.py:790-815)
         self.step_tensor = torch.tensor(0, dtype=torch.int64, device="cpu")
@@ -272,9 +279,15 @@ class _NativeGroup:
             raise NotImplementedError(f"{group[DISTRIBUTED_CONFIG]=} not supported!")
         if not isinstance(pc, RootInvShampooPreconditionerConfig):
             raise NotImplementedError(f"{pc=} not supported!")
-        if not isinstance(pc.amortized_computation_config, CoupledNewtonConfig):
+        acc = pc.amortized_computation_config
+        if isinstance(acc, EigenConfig):
+            if not isinstance(acc.rank_deficient_stability_config, PerturbationConfig):
+                raise NotImplementedError(f"{acc.rank_deficient_stability_config=} is not supported.")
+            if acc.eigendecomposition_offload_device != "":
+                raise NotImplementedError("eigendecomposition_offload_device: the decomposition runs on the MI355X")
+        elif not isinstance(acc, CoupledNewtonConfig):
             raise NotImplementedError(
-                f"Root inverse config is not implemented! Specified root inverse config is {pc.amortized_computation_config=}."
+                f"Root inverse config is not implemented! Specified root inverse config is {acc=}."
             )
         if not pc.use_symmetric_packing:
             raise NotImplementedError("use_symmetric_packing=False: the native step keeps factors packed")
@@ -430,13 +443,24 @@ class _NativeGroup:
         """Batched inverse roots + the reference's error semantics
         (shampoo_preconditioner_list.py:314-443)."""
         pc = self.preconditioner_config
-        cfg: CoupledNewtonConfig = pc.amortized_computation_config
-        native.check(
-            self.lib.sa_compute_root_inverses_newton(
-                self.plan, bc2, group[EPSILON], cfg.max_iterations, cfg.tolerance, self.iterations, self.status, stream
-            ),
-            "sa_compute_root_inverses_newton",
-        )
+        cfg = pc.amortized_computation_config
+        if self.use_eigh:
+            roots = (ctypes.c_float * max(self.n_factors, 1))(*self.factor_roots)
+            native.check(
+                self.lib.sa_compute_root_inverses_eigh(
+                    self.plan, bc2, group[EPSILON], roots,
+                    int(cfg.rank_deficient_stability_config.perturb_before_computation), self.max_jacobi_sweeps,
+                    self.iterations, self.status, stream,
+                ),
+                "sa_compute_root_inverses_eigh",
+            )
+        else:
+            native.check(
+                self.lib.sa_compute_root_inverses_newton(
+                    self.plan, bc2, group[EPSILON], cfg.max_iterations, cfg.tolerance, self.iterations, self.status, stream
+                ),
+                "sa_compute_root_inverses_newton",
+            )
         self.last_newton_iterations = [int(self.iterations[i]) for i in range(self.n_factors)]
         for i in range(self.n_factors):
             st = int(self.status[i])
@@ -453,7 +477,10 @@ class _NativeGroup:
                     "To mitigate, check factor matrix before the matrix computation."
                 )
             if st == native.SA_FACTOR_NOT_CONVERGED:
-                logger.warning("Newton did not converge and reached maximum number of iterations!")
+                if self.use_eigh:
+                    logger.warning(f"Jacobi eigensolver still rotating after {self.max_jacobi_sweeps} sweeps for factor matrix {name}.")
+                else:
+                    logger.warning("Newton did not converge and reached maximum number of iterations!")
         # blocks whose root cannot be used by the coupled Newton iteration fail every time
         for k, message in self.bad_root_blocks.items():
             count = self.failed_counter.get(k, 0) + 1
