@@ -31,6 +31,7 @@ struct JacobiFactor {
   float* U;            // (nb/2) x 64 x 64 rotations of the current round
   const int2* sched;   // (nb-1) x (nb/2) block pairs (I < J)
   int* rotations;      // number of rotations applied in the current sweep
+  float* rot_mass;     // sum of 2 a_pq^2 over those rotations = decrease of the off-diagonal norm^2
   const int* active;   // skip the factor when *active == 0
   float thr_abs;       // |a_pq| below this is treated as zero
   float thr_diag;      // a pair whose two diagonal entries are both below this (in magnitude) lies in the
@@ -65,6 +66,7 @@ __global__ __launch_bounds__(256) void jacobi_pivot_kernel(const JacobiFactor* _
   __shared__ float cs[2][JB];
   __shared__ int pq[2][JB];
   __shared__ int nrot;
+  __shared__ float nmass;
   const int fi = jacobi_locate(factors, n_factors, blockIdx.x);
   const JacobiFactor& F = factors[fi];
   if (*F.active == 0 || round >= F.nb - 1) return;
@@ -72,7 +74,7 @@ __global__ __launch_bounds__(256) void jacobi_pivot_kernel(const JacobiFactor* _
   const int2 ij = F.sched[round * (F.nb / 2) + pair];
   const int tid = threadIdx.x;
   const long long ld = F.dpad;
-  if (tid == 0) nrot = 0;
+  if (tid == 0) { nrot = 0; nmass = 0.0f; }
   for (int e = tid; e < JP * JP; e += 256) {
     const int i = e >> 6, j = e & 63;
     const int gi = (i < JB ? ij.x * JB + i : ij.y * JB + i - JB);
@@ -96,8 +98,12 @@ __global__ __launch_bounds__(256) void jacobi_pivot_kernel(const JacobiFactor* _
         c = 1.0f / sqrtf(1.0f + t * t);
         s = t * c;
         atomicAdd(&nrot, 1);
+        atomicAdd(&nmass, 2.0f * apq * apq);
       }
-      cs[0][tid] = c;
+      // Rutishauser's form: x' = x - s (y + tq x), y' = y + s (x - tq y) with tq = tan(theta/2) = s / (1 + c).
+      // It adds the small term (1 - c) x to the other small term before touching x, so tiny rotations do not
+      // bias the column norms (c alone rounds to 1 for |t| < 2.4e-4).
+      cs[0][tid] = s / (1.0f + c);
       cs[1][tid] = s;
       pq[0][tid] = p;
       pq[1][tid] = q;
@@ -108,13 +114,13 @@ __global__ __launch_bounds__(256) void jacobi_pivot_kernel(const JacobiFactor* _
 #pragma unroll
       for (int kk = 0; kk < 8; ++kk) {
         const int k = k0 + kk, p = pq[0][k], q = pq[1][k];
-        const float c = cs[0][k], s = cs[1][k];
+        const float tq = cs[0][k], s = cs[1][k];
         const float gp = G[i][p], gq = G[i][q];
-        G[i][p] = c * gp - s * gq;
-        G[i][q] = s * gp + c * gq;
+        G[i][p] = gp - s * (gq + tq * gp);
+        G[i][q] = gq + s * (gp - tq * gq);
         const float up = U[i][p], uq = U[i][q];
-        U[i][p] = c * up - s * uq;
-        U[i][q] = s * up + c * uq;
+        U[i][p] = up - s * (uq + tq * up);
+        U[i][q] = uq + s * (up - tq * uq);
       }
     }
     __syncthreads();
@@ -123,17 +129,20 @@ __global__ __launch_bounds__(256) void jacobi_pivot_kernel(const JacobiFactor* _
 #pragma unroll
       for (int kk = 0; kk < 8; ++kk) {
         const int k = k0 + kk, p = pq[0][k], q = pq[1][k];
-        const float c = cs[0][k], s = cs[1][k];
+        const float tq = cs[0][k], s = cs[1][k];
         const float gp = G[p][j], gq = G[q][j];
-        G[p][j] = c * gp - s * gq;
-        G[q][j] = s * gp + c * gq;
+        G[p][j] = gp - s * (gq + tq * gp);
+        G[q][j] = gq + s * (gp - tq * gq);
       }
     }
     __syncthreads();
   }
   float* Uout = F.U + (long long)pair * JP * JP;
   for (int e = tid; e < JP * JP; e += 256) Uout[e] = U[e >> 6][e & 63];
-  if (tid == 0 && nrot) atomicAdd(F.rotations, nrot);
+  if (tid == 0 && nrot) {
+    atomicAdd(F.rotations, nrot);
+    atomicAdd(F.rot_mass, nmass);
+  }
 }
 
 // which: 0 -> A, 1 -> V.  Grid: (pairs of all factors, dpad_max/128 row slabs, 2)

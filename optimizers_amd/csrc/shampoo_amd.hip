@@ -1139,6 +1139,7 @@ int32_t sa_compute_root_inverses_eigh(sa_plan* p, float bias_correction2, float 
     J.nb = f.dpad / JB;
     J.sched = p->t_sched.dev + sched_off[J.nb];
     J.rotations = p->d_iters + todo[i];
+    J.rot_mass = p->d_final_err + todo[i];
     J.active = p->d_active + todo[i];
     J.thr_abs = 1e-9f * fro[i];
     J.thr_diag = 2.4e-7f * fro[i];  // 2^-22 ||A||_F: below the eigenvalue resolution of an fp32 matrix
@@ -1155,6 +1156,7 @@ int32_t sa_compute_root_inverses_eigh(sa_plan* p, float bias_correction2, float 
   int live = n;
   for (int sweep = 0; sweep < max_sweeps && live > 0; ++sweep) {
     HIPCHECK(hipMemsetAsync(p->d_iters, 0, F * sizeof(int), s));
+    HIPCHECK(hipMemsetAsync(p->d_final_err, 0, F * sizeof(float), s));
     double work = 0.0;
     for (int i = 0; i < n; ++i)
       if (active[todo[i]]) { const double d = p->factors[todo[i]].dpad; work += 3.0 * 2.0 * d * d * JP * (d / JB - 1); }
@@ -1168,12 +1170,17 @@ int32_t sa_compute_root_inverses_eigh(sa_plan* p, float bias_correction2, float 
       HIPCHECK(hipGetLastError());
     }
     HIPCHECK(hipMemcpyAsync(p->h_pinned, p->d_iters, F * sizeof(int), hipMemcpyDeviceToHost, s));
+    HIPCHECK(hipMemcpyAsync(p->h_pinned + F, p->d_final_err, F * sizeof(float), hipMemcpyDeviceToHost, s));
     HIPCHECK(hipStreamSynchronize(s));
     live = 0;
-    for (int i : todo) {
+    const float* mass = reinterpret_cast<const float*>(p->h_pinned + F);
+    for (int k = 0; k < n; ++k) {
+      const int i = todo[k];
       if (!active[i]) continue;
       sweeps_out[i] = sweep + 1;
-      if (p->h_pinned[i] == 0) active[i] = 0; else ++live;
+      // converged when the sweep removed less than (5e-7 ||A||_F)^2 of off-diagonal mass
+      const double tol = 5e-7 * (double)fro[k];
+      if (p->h_pinned[i] == 0 || (double)mass[i] < tol * tol) active[i] = 0; else ++live;
     }
     HIPCHECK(hipMemcpyAsync(p->d_active, active.data(), F * sizeof(int), hipMemcpyHostToDevice, s));
     HIPCHECK(hipStreamSynchronize(s));

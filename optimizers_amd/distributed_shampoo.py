@@ -258,7 +258,7 @@ class _NativeGroup:
         self.status = (ctypes.c_int32 * max(self.n_factors, 1))()
         self.grad_ptrs = (ctypes.c_void_p * max(nb, 1))()
         self.last_newton_iterations: list[int] = []
-        self.max_jacobi_sweeps = 16
+        self.max_jacobi_sweeps = 30
 
         # one CPU step counter per group, aliased under every parameter (distributed_shampoo.py:790-815)
         self.step_tensor = torch.tensor(0, dtype=torch.int64, device="cpu")
