@@ -61,8 +61,13 @@ typedef struct sa_block_desc {
   float* adagrad;         /* grafting second moment, or NULL */
   float* momentum_buffer; /* classic momentum buffer, or NULL */
   float* factor[2];       /* packed upper-triangular Kronecker factor of dim 0 / dim 1; NULL = dim not preconditioned */
-  float* inv_factor[2];   /* packed upper-triangular inverse root of that factor */
+  float* inv_factor[2];   /* packed upper-triangular inverse root of that factor (root-inverse Shampoo), or NULL */
   int32_t root[2];        /* integer inverse root (4 for matrices, 2 for vectors by default) */
+  /* eigenvalue-corrected Shampoo / SOAP (shampoo_preconditioner_list.py:942-1007): dense d x d eigenbasis of
+   * each factor (row-major, columns are eigenvectors) and the second moment kept in the rotated basis
+   * (rows x cols, contiguous).  NULL for root-inverse Shampoo. */
+  float* eigenvectors[2];
+  float* corrected_eigenvalues;
 } sa_block_desc;
 
 /* Scalars of one step, already evaluated by the host exactly as the reference evaluates
@@ -132,6 +137,23 @@ int32_t sa_compute_root_inverses_newton(sa_plan* plan, float bias_correction2, f
 int32_t sa_compute_root_inverses_eigh(sa_plan* plan, float bias_correction2, float epsilon, const float* roots,
                                       int32_t perturb_before_computation, int32_t max_sweeps,
                                       int32_t* sweeps_out, int32_t* status_out, void* stream);
+
+/* Eigenbasis refresh of eigenvalue-corrected Shampoo with the QR algorithm: B = Q^T A Q with
+ * A = unpack(factor / bias_correction2) + epsilon I; while ||B - diag(B)||_F > tolerance ||B||_F and fewer than
+ * max_iterations were done: (Q', R) = qr(B) (blocked Householder), Q <- Q Q', B <- Q^T A Q; finally the columns
+ * of Q are ordered by ascending diag(B) with a stable sort (matrix_functions.py:799-852 via
+ * shampoo_preconditioner_list.py:314-443, 1137-1198).  iterations_out / status_out as for the Newton call. */
+int32_t sa_refresh_eigenbases_qr(sa_plan* plan, float bias_correction2, float epsilon, int32_t max_iterations,
+                                 float tolerance, int32_t* iterations_out, int32_t* status_out, void* stream);
+
+/* corrected_eigenvalues <- beta2 * corrected_eigenvalues + w * (Q_L^T G Q_R)^2 with the raw gradient
+ * (shampoo_preconditioner_list.py:1891-1912). */
+int32_t sa_update_corrected_eigenvalues(sa_plan* plan, float beta2, float weighting_factor, void* stream);
+
+/* P = Q_L [ (Q_L^T Ghat Q_R) / ((corrected_eigenvalues / bias_correction2)^(1/root) + epsilon) ] Q_R^T into the
+ * workspace plus its squared norm per block (shampoo_preconditioner_list.py:1914-1942). */
+int32_t sa_precondition_eigenvalue_corrected(sa_plan* plan, const sa_step_scalars* s, float bias_correction2,
+                                             float epsilon, float root, void* stream);
 
 /* Grafting second moment, filtered gradient and the grafted direction's squared norm per block
  * (adagrad_preconditioner_list.py:122-162, distributed_shampoo.py:1162-1199, 1110-1114). */

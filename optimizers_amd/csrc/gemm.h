@@ -41,6 +41,9 @@ enum Epilogue {
   EPI_STORE_SQNORM = 1, // C = acc, partial[tile] = sum(acc^2) over the tile
   EPI_SYRK_EMA = 2,     // packed upper triangle: C = beta*C + alpha*acc   (tiles tn >= tm only)
   EPI_NEWTON_M = 3,     // C = acc (new M), C2 = acc*mp_scale + mp_diag*I, err = max|acc - I| over d x d
+  EPI_SQ_EMA = 4,       // C = beta*C + alpha*acc^2        (second moment in the eigenbasis)
+  EPI_DIVPOW = 5,       // C = acc / ((C2 / div)^pow_exp + eps)   (C2 has the layout of C)
+  EPI_SUB = 6,          // C -= acc                         (block-reflector updates of the QR refresh)
 };
 
 struct GemmProblem {
@@ -63,6 +66,7 @@ struct GemmScalars {
   float a_div, b_div;      // operand is divided by this on load (1.0f = as stored)
   float alpha, beta;       // EPI_SYRK_EMA: C = beta*C + alpha*acc
   float mp_scale, mp_diag; // EPI_NEWTON_M: M_p = M*mp_scale + mp_diag*I
+  float div, pow_exp, eps; // EPI_DIVPOW
 };
 
 __device__ __forceinline__ float4 load4_guarded(const float* p, bool vec, int valid) {
@@ -288,6 +292,23 @@ __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(
             const long long off = (long long)row * N - ((long long)row * (row - 1)) / 2 + (col - row);
             const float old = C[off];
             C[off] = __fadd_rn(__fmul_rn(old, sc.beta), __fmul_rn(v, sc.alpha));
+          }
+        } else if (EPI == EPI_SQ_EMA) {
+          if (!EDGE || (row < M && col < N)) {
+            const long long o = (long long)row * ldc + col;
+            C[o] = __fadd_rn(__fmul_rn(C[o], sc.beta), __fmul_rn(__fmul_rn(sc.alpha, v), v));
+          }
+        } else if (EPI == EPI_DIVPOW) {
+          if (!EDGE || (row < M && col < N)) {
+            const long long o = (long long)row * ldc + col;
+            const float x = P.C2[o] / sc.div;
+            const float r = (sc.pow_exp == 0.5f) ? sqrtf(x) : powf(x, sc.pow_exp);
+            C[o] = v / (r + sc.eps);
+          }
+        } else if (EPI == EPI_SUB) {
+          if (!EDGE || (row < M && col < N)) {
+            const long long o = (long long)row * ldc + col;
+            C[o] = C[o] - v;
           }
         } else if (EPI == EPI_NEWTON_M) {
           // operands are zero padded to the tile grid, so every (row, col) is in bounds

@@ -1,0 +1,210 @@
+// Batched blocked Householder QR for the eigenbasis refresh of eigenvalue-corrected Shampoo.
+//
+// One refresh factors B = Q^T A Q (d x d) for every factor at once.  Columns are processed in panels;
+// a panel (all rows below the diagonal x up to 32 columns) is factored by ONE workgroup entirely in LDS
+// (up to 135 KB of the 160 KB a CU has), producing the Householder vectors V (unit lower trapezoid) and
+// the triangular factor T of the compact WY form H_1...H_k = I - V T V^T.  The trailing matrix and the
+// accumulated eigenbasis are then updated with the grouped MFMA GEMM (EPI_SUB).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "gemm.h"
+
+namespace sa {
+
+constexpr int QR_MAX_PANEL = 32;
+constexpr int QR_THREADS = 256;
+
+struct QrPanel {
+  const float* B;   // matrix being factored, row stride ldb
+  float* V;         // rows x pcols, row stride QR_MAX_PANEL: Householder vectors (unit diagonal, zeros above)
+  float* T;         // QR_MAX_PANEL x QR_MAX_PANEL upper triangular
+  long long ldb;
+  int d;            // matrix dimension
+  int j0;           // first column / row of the panel
+  int pcols;        // columns in this panel
+  const int* active;
+};
+
+// dynamic LDS: rows * (pcols + 1) floats for the panel
+__global__ __launch_bounds__(QR_THREADS) void qr_panel_kernel(const QrPanel* __restrict__ jobs) {
+  extern __shared__ float lds[];
+  __shared__ float wred[4][QR_MAX_PANEL];
+  __shared__ float tau_s[QR_MAX_PANEL];
+  __shared__ float S[QR_MAX_PANEL][QR_MAX_PANEL + 1];
+  __shared__ float Tm[QR_MAX_PANEL][QR_MAX_PANEL + 1];
+  __shared__ float bcast[2];
+  const QrPanel& J = jobs[blockIdx.x];
+  if (J.active != nullptr && *J.active == 0) return;
+  const int rows = J.d - J.j0, pc = J.pcols, st = pc + 1;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float* P = lds;
+  for (int e = tid; e < rows * pc; e += QR_THREADS) {
+    const int r = e / pc, c = e - r * pc;
+    P[r * st + c] = J.B[(long long)(J.j0 + r) * J.ldb + J.j0 + c];
+  }
+  __syncthreads();
+  for (int c = 0; c < pc; ++c) {
+    // --- Householder vector of column c (LAPACK slarfg): rows c..rows-1
+    float part = 0.f;
+    for (int r = c + 1 + tid; r < rows; r += QR_THREADS) { const float x = P[r * st + c]; part += x * x; }
+    part = wave_sum(part);
+    if (lane == 0) wred[wave][0] = part;
+    __syncthreads();
+    if (tid == 0) {
+      const float sigma2 = (wred[0][0] + wred[1][0]) + (wred[2][0] + wred[3][0]);
+      const float alpha = (c < rows) ? P[c * st + c] : 0.f;
+      float tau = 0.f, scale = 0.f, beta = alpha;
+      if (sigma2 != 0.f && c < rows) {
+        beta = -copysignf(sqrtf(alpha * alpha + sigma2), alpha);
+        tau = (beta - alpha) / beta;
+        scale = 1.0f / (alpha - beta);
+      }
+      tau_s[c] = tau;
+      bcast[0] = scale;
+      bcast[1] = beta;
+    }
+    __syncthreads();
+    const float scale = bcast[0], tau = tau_s[c];
+    for (int r = c + 1 + tid; r < rows; r += QR_THREADS) P[r * st + c] *= scale;
+    if (tid == 0 && c < rows) P[c * st + c] = bcast[1];
+    __syncthreads();
+    if (tau != 0.f) {
+      // --- apply H_c to the remaining panel columns: w = v^T P[:, c'] ; P[:, c'] -= tau w v
+      for (int cc = c + 1; cc < pc; ++cc) {
+        float w = 0.f;
+        for (int r = c + 1 + tid; r < rows; r += QR_THREADS) w += P[r * st + c] * P[r * st + cc];
+        w = wave_sum(w);
+        if (lane == 0) wred[wave][cc] = w;
+      }
+      __syncthreads();
+      for (int cc = c + 1; cc < pc; ++cc) {
+        const float w = tau * (P[c * st + cc] + (wred[0][cc] + wred[1][cc]) + (wred[2][cc] + wred[3][cc]));
+        for (int r = c + 1 + tid; r < rows; r += QR_THREADS) P[r * st + cc] -= w * P[r * st + c];
+      }
+      __syncthreads();
+      if (tid < pc - (c + 1)) {
+        // row c itself (v[c] = 1); row c and the partial sums are still untouched
+        const int cc = c + 1 + tid;
+        const float w = tau * (P[c * st + cc] + (wred[0][cc] + wred[1][cc]) + (wred[2][cc] + wred[3][cc]));
+        P[c * st + cc] -= w;
+      }
+      __syncthreads();
+    }
+  }
+  // --- S = V^T V (strict upper part), v_k has an implicit 1 at row k and zeros above
+  for (int e = tid; e < pc * pc; e += QR_THREADS) {
+    const int i = e / pc, k = e - i * pc;
+    float acc = 0.f;
+    if (i < k && k < rows) {
+      acc = P[k * st + i];  // v_i[k] * v_k[k] with v_k[k] = 1
+      for (int r = k + 1; r < rows; ++r) acc += P[r * st + i] * P[r * st + k];
+    }
+    S[i][k] = acc;
+  }
+  for (int e = tid; e < QR_MAX_PANEL * QR_MAX_PANEL; e += QR_THREADS) Tm[e / QR_MAX_PANEL][e % QR_MAX_PANEL] = 0.f;
+  __syncthreads();
+  // --- T (LAPACK slarft, forward columnwise): T[i][i] = tau_i, T[0:i, i] = -tau_i T[0:i,0:i] S[0:i, i]
+  for (int i = 0; i < pc; ++i) {
+    if (tid < i) {
+      float acc = 0.f;
+      for (int m = tid; m < i; ++m) acc += Tm[tid][m] * S[m][i];
+      Tm[tid][i] = -tau_s[i] * acc;
+    }
+    if (tid == i) Tm[i][i] = tau_s[i];
+    __syncthreads();
+  }
+  for (int e = tid; e < QR_MAX_PANEL * QR_MAX_PANEL; e += QR_THREADS)
+    J.T[e] = Tm[e / QR_MAX_PANEL][e % QR_MAX_PANEL];
+  for (int e = tid; e < rows * QR_MAX_PANEL; e += QR_THREADS) {
+    const int r = e / QR_MAX_PANEL, c = e % QR_MAX_PANEL;
+    float v = 0.f;
+    if (c < pc) v = (r > c) ? P[r * st + c] : (r == c ? 1.0f : 0.0f);
+    J.V[(long long)r * QR_MAX_PANEL + c] = v;
+  }
+}
+
+// Generic strided 2-D copy: dst[r][c] = src[r][c]
+struct Copy2D {
+  const float* src;
+  float* dst;
+  long long lds_, ldd;
+  int rows, cols;
+  const int* perm;  // optional: dst[r][c] = src[r][perm[c]]
+};
+__global__ __launch_bounds__(256) void copy2d_kernel(const Copy2D* __restrict__ jobs) {
+  const Copy2D& J = jobs[blockIdx.y];
+  const long long n = (long long)J.rows * J.cols;
+  for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < n; e += (long long)gridDim.x * 256) {
+    const int r = (int)(e / J.cols), c = (int)(e % J.cols);
+    const int sc = J.perm ? min(max(J.perm[c], 0), J.cols - 1) : c;  // clamp: a NaN spectrum leaves ranks undefined
+    J.dst[r * J.ldd + c] = J.src[r * J.lds_ + sc];
+  }
+}
+
+// Per factor: sum of squares of all entries and of the diagonal of a d x d matrix (criterion of
+// matrix_functions.py:772-797); one workgroup per factor.
+struct NormPair {
+  const float* B;
+  float* out_all;   // sum B^2
+  float* out_diag;  // sum diag(B)^2
+  long long ldb;
+  int d;
+};
+__global__ __launch_bounds__(256) void diag_off_norm_kernel(const NormPair* __restrict__ jobs) {
+  __shared__ float red[4];
+  const NormPair& J = jobs[blockIdx.x];
+  float a = 0.f, dg = 0.f;
+  const long long n = (long long)J.d * J.d;
+  for (long long e = threadIdx.x; e < n; e += 256) {
+    const int r = (int)(e / J.d), c = (int)(e % J.d);
+    const float v = J.B[r * J.ldb + c];
+    a += v * v;
+    if (r == c) dg += v * v;
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  a = wave_sum(a);
+  if (lane == 0) red[wave] = a;
+  __syncthreads();
+  const float ta = (red[0] + red[1]) + (red[2] + red[3]);
+  __syncthreads();
+  dg = wave_sum(dg);
+  if (lane == 0) red[wave] = dg;
+  __syncthreads();
+  if (threadIdx.x == 0) { *J.out_all = ta; *J.out_diag = (red[0] + red[1]) + (red[2] + red[3]); }
+}
+
+// Rayleigh quotients ev[i] = sum_r Q[r][i] * Y[r][i], stable ascending rank of ev, and its inverse
+// permutation: order[k] = index of the k-th smallest (ties keep their original order, like
+// torch.sort(stable=True), matrix_functions.py:849).  One workgroup per factor, d <= 4096.
+struct SortJob {
+  const float* Q;
+  const float* Y;
+  float* ev;     // d floats
+  int* order;    // d ints
+  long long ldq, ldy;
+  int d;
+};
+__global__ __launch_bounds__(256) void rayleigh_sort_kernel(const SortJob* __restrict__ jobs) {
+  const SortJob& J = jobs[blockIdx.x];
+  const int d = J.d;
+  for (int i = threadIdx.x; i < d; i += 256) {
+    float acc = 0.f;
+    for (int r = 0; r < d; ++r) acc += J.Q[r * J.ldq + i] * J.Y[r * J.ldy + i];
+    J.ev[i] = acc;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < d; i += 256) {
+    const float x = J.ev[i];
+    int rank = 0;
+    for (int j = 0; j < d; ++j) {
+      const float y = J.ev[j];
+      rank += (y < x || (y == x && j < i)) ? 1 : 0;
+    }
+    J.order[rank] = i;
+  }
+}
+
+}  // namespace sa

@@ -16,6 +16,7 @@
 #include "eigh.h"
 #include "elementwise.h"
 #include "gemm.h"
+#include "qr.h"
 
 using namespace sa;
 
@@ -142,7 +143,7 @@ int launch_gemm_auto(const GemmTable& g, GemmScalars sc, hipStream_t s) {
   return g.aligned ? launch_gemm<AL, BL, EPI, false>(g, sc, s) : launch_gemm<AL, BL, EPI, true>(g, sc, s);
 }
 
-GemmScalars unit_scalars() { return GemmScalars{1.0f, 1.0f, 1.0f, 0.0f, 0.0f, 0.0f}; }
+GemmScalars unit_scalars() { return GemmScalars{1.0f, 1.0f, 1.0f, 0.0f, 0.0f, 0.0f, 1.0f, 1.0f, 0.0f}; }
 
 // ---- phase timing -------------------------------------------------------------------------
 struct Phase {
@@ -185,6 +186,7 @@ struct Factor {
   int block, side, d, dpad, root;
   float* factor;
   float* inv;
+  float* eigvec;
   long long dense_off;   // offset (floats) of this factor inside every dense array
   long long norm_off;    // offset into the norm-partial array
   int norm_chunks;
@@ -227,6 +229,14 @@ struct sa_plan {
   Table<EigInit> t_eiginit;
   Table<EigFinal> t_eigfinal;
   GemmTable eig_gemm;
+  GemmTable ec_stat1, ec_stat2, ec_stat_l, ec_stat_r;          // corrected-eigenvalue update
+  GemmTable ec_p1, ec_p1d, ec_p2, ec_p2d, ec_p3, ec_p3n, ec_p4, ec_p4n;  // eigenvalue-corrected preconditioning
+  GemmTable qr_g[6], qr_aq, qr_b;
+  Table<QrPanel> t_qrpanel;
+  Table<Copy2D> t_copy;
+  Table<NormPair> t_normpair;
+  Table<SortJob> t_sort;
+  bool eigenvalue_corrected = false;
   int n_active_blocks = 0;
 
   // Newton control state (device) and pinned readback
@@ -253,7 +263,7 @@ void compute_layout(sa_plan* p) {
   p->off_ghat_partial = take(p->total_chunks_all);
   p->off_ptile_partial = take(p->total_ptiles_all);
   p->off_norm_partial = take(p->norm_partials_total);
-  p->scratch_floats = std::max(8LL * p->dense_total, 3LL * round_up(p->total_elems, 64) + 192);
+  p->scratch_floats = std::max(8LL * p->dense_total, 4LL * round_up(p->total_elems, 64) + 256);
   p->off_scratch = take(p->scratch_floats);
   p->ws_needed = o * (long long)sizeof(float);
 }
@@ -267,6 +277,7 @@ enum { NB_X0 = 0, NB_X1 = 1, NB_M0 = 2, NB_M1 = 3, NB_MP0 = 4, NB_MP1 = 5, NB_S1
 inline float* tbuf(const sa_plan* p) { return p->f(p->off_scratch); }
 inline float* pbuf(const sa_plan* p) { return p->f(p->off_scratch + round_up(p->total_elems, 64) + 64); }
 inline float* ghbuf(const sa_plan* p) { return p->f(p->off_scratch + 2 * (round_up(p->total_elems, 64) + 64)); }
+inline float* t2buf(const sa_plan* p) { return p->f(p->off_scratch + 3 * (round_up(p->total_elems, 64) + 64)); }
 
 int need_ws(const sa_plan* p) {
   if (!p->ws) return fail(SA_ERR_WORKSPACE, "no workspace bound (sa_plan_bind_workspace)");
@@ -357,9 +368,58 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
   SACHECK(p->syrk0.commit(s));
   SACHECK(p->syrk1.commit(s));
 
-  // preconditioning tables
+  // eigenvalue-corrected tables
+  for (GemmTable* g : {&p->ec_stat1, &p->ec_stat2, &p->ec_stat_l, &p->ec_stat_r, &p->ec_p1, &p->ec_p1d, &p->ec_p2, &p->ec_p2d,
+                       &p->ec_p3, &p->ec_p3n, &p->ec_p4, &p->ec_p4n})
+    g->clear();
+  if (p->eigenvalue_corrected) {
+    for (int b : active) {
+      const sa_block_desc& d = p->blocks[b];
+      const BlockDev& B = p->t_blocks.host[b];
+      const int f0 = p->block_factor[0][b], f1 = p->block_factor[1][b];
+      if (f0 < 0 && f1 < 0) continue;
+      const long long eo = p->elem_off[b];
+      float* part = p->f(p->off_ptile_partial) + p->ptile_begin_all[b];
+      const float* QL = f0 >= 0 ? p->factors[f0].eigvec : nullptr;
+      const float* QR = f1 >= 0 ? p->factors[f1].eigvec : nullptr;
+      const float* G = p->grads[b];
+      auto mk = [&](const float* A, long long lda, const float* Bm, long long ldb, float* C, float* C2, int K) {
+        GemmProblem q{};
+        q.A = A; q.lda = lda; q.a_vec = vec_ok(A, lda);
+        q.B = Bm; q.ldb = ldb; q.b_vec = vec_ok(Bm, ldb);
+        q.C = C; q.C2 = C2; q.ldc = d.cols;
+        q.M = d.rows; q.N = d.cols; q.K = K;
+        return q;
+      };
+      float* T = tbuf(p) + eo;
+      float* T2 = t2buf(p) + eo;
+      float* Pb = pbuf(p) + eo;
+      if (f0 >= 0 && f1 >= 0) {
+        p->ec_stat1.add(mk(QL, d.rows, G, d.ld, T, nullptr, d.rows), false);                       // T = QL^T G   (A_KM)
+        p->ec_stat2.add(mk(T, d.cols, QR, d.cols, d.corrected_eigenvalues, nullptr, d.cols), false);  // corr <- EMA (T QR)^2
+        p->ec_p1.add(mk(QL, d.rows, B.ghat_src, B.ghat_ld, T, nullptr, d.rows), false);             // T = QL^T Ghat (b_div)
+        p->ec_p2.add(mk(T, d.cols, QR, d.cols, T2, d.corrected_eigenvalues, d.cols), false);         // T2 = (T QR)/den
+        p->ec_p3.add(mk(QL, d.rows, T2, d.cols, T, nullptr, d.rows), false);                         // T = QL T2
+        p->ec_p4.add(mk(T, d.cols, QR, d.cols, Pb, part, d.cols), false);                            // P = T QR^T (B_NK)
+      } else if (f0 >= 0) {
+        p->ec_stat_l.add(mk(QL, d.rows, G, d.ld, d.corrected_eigenvalues, nullptr, d.rows), false);
+        p->ec_p1d.add(mk(QL, d.rows, B.ghat_src, B.ghat_ld, T2, d.corrected_eigenvalues, d.rows), false);
+        p->ec_p3n.add(mk(QL, d.rows, T2, d.cols, Pb, part, d.rows), false);
+      } else {
+        p->ec_stat_r.add(mk(G, d.ld, QR, d.cols, d.corrected_eigenvalues, nullptr, d.cols), false);
+        p->ec_p2d.add(mk(B.ghat_src, B.ghat_ld, QR, d.cols, T2, d.corrected_eigenvalues, d.cols), false);
+        p->ec_p4n.add(mk(T2, d.cols, QR, d.cols, Pb, part, d.cols), false);
+      }
+    }
+  }
+  for (GemmTable* g : {&p->ec_stat1, &p->ec_stat2, &p->ec_stat_l, &p->ec_stat_r, &p->ec_p1, &p->ec_p1d, &p->ec_p2, &p->ec_p2d,
+                       &p->ec_p3, &p->ec_p3n, &p->ec_p4, &p->ec_p4n})
+    SACHECK(g->commit(s));
+
+  // preconditioning tables (root-inverse Shampoo)
   p->g1_store.clear(); p->g1_norm.clear(); p->g2_norm.clear(); p->g2g_norm.clear();
   for (int b : active) {
+    if (p->eigenvalue_corrected) break;
     const sa_block_desc& d = p->blocks[b];
     const BlockDev& B = p->t_blocks.host[b];
     const int f0 = p->block_factor[0][b], f1 = p->block_factor[1][b];
@@ -425,7 +485,7 @@ int validate_scalars(const sa_plan* p, const sa_step_scalars* s) {
 
 // packed -> dense mirrored cache of every inverse root
 int refresh_inverse_cache(sa_plan* p, hipStream_t s) {
-  if (p->inv_cache_valid || p->factors.empty()) { p->inv_cache_valid = true; return SA_OK; }
+  if (p->inv_cache_valid || p->factors.empty() || p->eigenvalue_corrected) { p->inv_cache_valid = true; return SA_OK; }
   const int F = (int)p->factors.size();
   SACHECK(p->t_sym.begin(F));
   int tiles = 0;
@@ -522,9 +582,13 @@ int32_t sa_plan_create(const sa_block_desc* blocks, int32_t n_blocks, sa_plan** 
     ptiles += ((d.rows + BM - 1) / BM) * ((d.cols + BN - 1) / BN);
     for (int side = 0; side < 2; ++side) {
       if (!d.factor[side]) continue;
-      if (!d.inv_factor[side] || d.root[side] < 1) {
+      if ((!d.inv_factor[side] && !d.eigenvectors[side]) || (d.inv_factor[side] && d.root[side] < 1)) {
         delete p;
-        return fail(SA_ERR_INVALID, "sa_plan_create: factor without inverse storage or with root < 1");
+        return fail(SA_ERR_INVALID, "sa_plan_create: factor without inverse / eigenvector storage or with root < 1");
+      }
+      if (d.eigenvectors[side] && !d.corrected_eigenvalues) {
+        delete p;
+        return fail(SA_ERR_INVALID, "sa_plan_create: eigenvectors without corrected_eigenvalues");
       }
       Factor f{};
       f.block = b; f.side = side;
@@ -533,11 +597,13 @@ int32_t sa_plan_create(const sa_block_desc* blocks, int32_t n_blocks, sa_plan** 
       f.root = d.root[side];
       f.factor = d.factor[side];
       f.inv = d.inv_factor[side];
+      f.eigvec = d.eigenvectors[side];
       f.dense_off = dense;
       dense += (long long)f.dpad * f.dpad;
       f.norm_off = normp;
       f.norm_chunks = (int)(((long long)f.d * (f.d + 1) / 2 + NORM_CHUNK - 1) / NORM_CHUNK);
       normp += f.norm_chunks;
+      if (f.eigvec) p->eigenvalue_corrected = true;
       p->block_factor[side][b] = (int)p->factors.size();
       p->factors.push_back(f);
     }
@@ -573,6 +639,11 @@ void sa_plan_destroy(sa_plan* p) {
   for (auto& g : p->nt_pow) g.t.destroy();
   p->t_sym.destroy(); p->t_normjobs.destroy(); p->t_ids.destroy();
   p->t_jacobi.destroy(); p->t_sched.destroy(); p->t_eiginit.destroy(); p->t_eigfinal.destroy(); p->eig_gemm.t.destroy();
+  for (GemmTable* g : {&p->ec_stat1, &p->ec_stat2, &p->ec_stat_l, &p->ec_stat_r, &p->ec_p1, &p->ec_p1d, &p->ec_p2, &p->ec_p2d,
+                       &p->ec_p3, &p->ec_p3n, &p->ec_p4, &p->ec_p4n, &p->qr_aq, &p->qr_b})
+    g->t.destroy();
+  for (auto& g : p->qr_g) g.t.destroy();
+  p->t_qrpanel.destroy(); p->t_copy.destroy(); p->t_normpair.destroy(); p->t_sort.destroy();
   for (void* q : {(void*)p->d_err, (void*)p->d_active, (void*)p->d_iters, (void*)p->d_final_parity,
                   (void*)p->d_final_err, (void*)p->d_flags, (void*)p->d_nactive})
     if (q) (void)hipFree(q);
@@ -1223,6 +1294,303 @@ int32_t sa_compute_root_inverses_eigh(sa_plan* p, float bias_correction2, float 
   size_t ok = 0;
   SACHECK(root_inverse_epilogue(p, todo, X, status_out, s, &ok));
   for (size_t i = 0; i < ok; ++i) status_out[todo[i]] = active[todo[i]] ? SA_FACTOR_NOT_CONVERGED : SA_FACTOR_OK;
+  return SA_OK;
+}
+
+// --------------------------------------------------------------------------------------------
+// Eigenvalue-corrected Shampoo (SOAP)
+// --------------------------------------------------------------------------------------------
+
+int32_t sa_update_corrected_eigenvalues(sa_plan* p, float beta2, float weighting_factor, void* stream) {
+  if (!p) return fail(SA_ERR_INVALID, "NULL plan");
+  if (!p->eigenvalue_corrected) return fail(SA_ERR_STATE, "plan has no eigenvector state");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SACHECK(ensure_tables(p, nullptr, s));
+  GemmScalars sc = unit_scalars();
+  sc.alpha = weighting_factor;
+  sc.beta = beta2;
+  double flops = 0.0;
+  for (const GemmTable* g : {&p->ec_stat1, &p->ec_stat2, &p->ec_stat_l, &p->ec_stat_r})
+    for (const GemmProblem& q : g->build) flops += 2.0 * q.M * q.N * q.K;
+  Span span("eigenbasis_rotation", s, flops, 4, true);
+  SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_STORE>(p->ec_stat1, unit_scalars(), s)));
+  SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_SQ_EMA>(p->ec_stat2, sc, s)));
+  SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_SQ_EMA>(p->ec_stat_l, sc, s)));
+  SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_SQ_EMA>(p->ec_stat_r, sc, s)));
+  return SA_OK;
+}
+
+int32_t sa_precondition_eigenvalue_corrected(sa_plan* p, const sa_step_scalars* sc, float bias_correction2, float epsilon,
+                                             float root, void* stream) {
+  if (!p) return fail(SA_ERR_INVALID, "NULL plan");
+  if (!p->eigenvalue_corrected) return fail(SA_ERR_STATE, "plan has no eigenvector state");
+  if (!(root > 0.0f) || !(bias_correction2 != 0.0f)) return fail(SA_ERR_INVALID, "bad root or bias correction");
+  SACHECK(validate_scalars(p, sc));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SACHECK(ensure_tables(p, sc, s));
+  double flops = 0.0;
+  for (const GemmTable* g : {&p->ec_p1, &p->ec_p1d, &p->ec_p2, &p->ec_p2d, &p->ec_p3, &p->ec_p3n, &p->ec_p4, &p->ec_p4n})
+    for (const GemmProblem& q : g->build) flops += 2.0 * q.M * q.N * q.K;
+  {
+    Span span("precondition_gemm", s, flops, 8, true);
+    GemmScalars u = unit_scalars();
+    GemmScalars bdiv = u; bdiv.b_div = sc->bias_correction1;
+    GemmScalars den = u; den.div = bias_correction2; den.pow_exp = 1.0f / root; den.eps = epsilon;
+    GemmScalars den_b = den; den_b.b_div = sc->bias_correction1;
+    GemmScalars den_a = den; den_a.a_div = sc->bias_correction1;
+    SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_STORE>(p->ec_p1, bdiv, s)));
+    SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_DIVPOW>(p->ec_p1d, den_b, s)));
+    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_DIVPOW>(p->ec_p2, den, s)));
+    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_DIVPOW>(p->ec_p2d, den_a, s)));
+    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE>(p->ec_p3, u, s)));
+    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE_SQNORM>(p->ec_p3n, u, s)));
+    SACHECK((launch_gemm_auto<A_MK, B_NK, EPI_STORE_SQNORM>(p->ec_p4, u, s)));
+    SACHECK((launch_gemm_auto<A_MK, B_NK, EPI_STORE_SQNORM>(p->ec_p4n, u, s)));
+  }
+  if (p->n_active_blocks) {
+    hipLaunchKernelGGL(reduce_norms_kernel, dim3(p->n_active_blocks), dim3(EW_THREADS), 0, s, p->t_blocks.dev,
+                       p->t_active_blocks.dev, p->n_blocks, p->f(p->off_graft_partial), p->f(p->off_ghat_partial),
+                       p->f(p->off_ptile_partial), p->f(p->off_norms));
+    HIPCHECK(hipGetLastError());
+  }
+  return SA_OK;
+}
+
+// Blocked Householder QR of B (NB_X0) for the active factors; the reflectors are applied from the right to
+// Qacc (NB_X1):  Qacc <- Qacc H_1 H_2 ... H_d.
+static int qr_accumulate(sa_plan* p, const std::vector<int>& ids, hipStream_t s) {
+  const int n = (int)ids.size();
+  int dmax = 0;
+  for (int i : ids) dmax = std::max(dmax, p->factors[i].d);
+  const int lds_floats = 34816;  // 136 KB for the panel, the rest of the 160 KB holds the small arrays
+  int pc_max = std::min(QR_MAX_PANEL, lds_floats / dmax - 1);
+  if (pc_max < 1) return fail(SA_ERR_UNSUPPORTED, "QR refresh: factor dimension too large for an LDS resident panel");
+  static bool attr_set = false;
+  if (!attr_set) {
+    HIPCHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(qr_panel_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                 lds_floats * (int)sizeof(float)));
+    attr_set = true;
+  }
+  for (int j0 = 0; j0 < dmax; j0 += pc_max) {
+    SACHECK(p->t_qrpanel.begin(n));
+    for (int k = 0; k < 6; ++k) p->qr_g[k].clear();
+    int jobs = 0, max_rows = 0;
+    for (int i : ids) {
+      const Factor& f = p->factors[i];
+      if (j0 >= f.d) continue;
+      const int pc = std::min(pc_max, f.d - j0), rows = f.d - j0, ntrail = f.d - j0 - pc;
+      float* B = newton_buf(p, NB_X0, f);
+      float* Qacc = newton_buf(p, NB_X1, f);
+      float* V = newton_buf(p, NB_S1, f);
+      float* T = V + (long long)f.dpad * QR_MAX_PANEL;
+      float* W = T + QR_MAX_PANEL * QR_MAX_PANEL;
+      float* W2 = W + (long long)QR_MAX_PANEL * f.dpad;
+      float* Z = newton_buf(p, NB_S2, f);
+      float* Z2 = Z + (long long)f.dpad * QR_MAX_PANEL;
+      QrPanel& J = p->t_qrpanel.host[jobs++];
+      std::memset(&J, 0, sizeof(J));
+      J.B = B; J.V = V; J.T = T; J.ldb = f.dpad; J.d = f.d; J.j0 = j0; J.pcols = pc; J.active = p->d_active + i;
+      max_rows = std::max(max_rows, rows);
+      auto mk = [&](const float* A, long long lda, const float* Bm, long long ldb, float* C, long long ldc, int M, int N, int K) {
+        GemmProblem q{};
+        q.A = A; q.lda = lda; q.a_vec = vec_ok(A, lda);
+        q.B = Bm; q.ldb = ldb; q.b_vec = vec_ok(Bm, ldb);
+        q.C = C; q.ldc = ldc; q.M = M; q.N = N; q.K = K;
+        q.active = p->d_active + i;
+        return q;
+      };
+      if (ntrail > 0) {
+        float* Bt = B + (long long)j0 * f.dpad + j0 + pc;  // trailing matrix B[j0:, j0+pc:]
+        p->qr_g[0].add(mk(V, QR_MAX_PANEL, Bt, f.dpad, W, f.dpad, pc, ntrail, rows), false);   // W = V^T Bt      (A_KM)
+        p->qr_g[1].add(mk(T, QR_MAX_PANEL, W, f.dpad, W2, f.dpad, pc, ntrail, pc), false);      // W2 = T^T W     (A_KM)
+        p->qr_g[2].add(mk(V, QR_MAX_PANEL, W2, f.dpad, Bt, f.dpad, rows, ntrail, pc), false);   // Bt -= V W2     (A_MK, SUB)
+      }
+      float* Qt = Qacc + j0;  // Qacc[:, j0:]
+      p->qr_g[3].add(mk(Qt, f.dpad, V, QR_MAX_PANEL, Z, QR_MAX_PANEL, f.d, pc, rows), false);   // Z = Qt V       (NN)
+      p->qr_g[4].add(mk(Z, QR_MAX_PANEL, T, QR_MAX_PANEL, Z2, QR_MAX_PANEL, f.d, pc, pc), false);  // Z2 = Z T     (NN)
+      p->qr_g[5].add(mk(Z2, QR_MAX_PANEL, V, QR_MAX_PANEL, Qt, f.dpad, f.d, rows, pc), false);  // Qt -= Z2 V^T   (B_NK, SUB)
+    }
+    if (!jobs) break;
+    p->t_qrpanel.n = jobs;
+    SACHECK(p->t_qrpanel.upload(s));
+    for (int k = 0; k < 6; ++k) SACHECK(p->qr_g[k].commit(s));
+    const size_t lds_bytes = (size_t)max_rows * (pc_max + 1) * sizeof(float);
+    hipLaunchKernelGGL(qr_panel_kernel, dim3(jobs), dim3(QR_THREADS), lds_bytes, s, p->t_qrpanel.dev);
+    HIPCHECK(hipGetLastError());
+    GemmScalars u = unit_scalars();
+    SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, true>(p->qr_g[0], u, s)));
+    SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, true>(p->qr_g[1], u, s)));
+    SACHECK((launch_gemm<A_MK, B_KN, EPI_SUB, true>(p->qr_g[2], u, s)));
+    SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, true>(p->qr_g[3], u, s)));
+    SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, true>(p->qr_g[4], u, s)));
+    SACHECK((launch_gemm<A_MK, B_NK, EPI_SUB, true>(p->qr_g[5], u, s)));
+  }
+  return SA_OK;
+}
+
+int32_t sa_refresh_eigenbases_qr(sa_plan* p, float bias_correction2, float epsilon, int32_t max_iterations, float tolerance,
+                                 int32_t* iterations_out, int32_t* status_out, void* stream) {
+  if (!p || !iterations_out || !status_out) return fail(SA_ERR_INVALID, "sa_refresh_eigenbases_qr: NULL argument");
+  if (!p->eigenvalue_corrected) return fail(SA_ERR_STATE, "plan has no eigenvector state");
+  if (!(bias_correction2 != 0.0f) || max_iterations < 0) return fail(SA_ERR_INVALID, "bad bias correction or max_iterations");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SACHECK(ensure_tables(p, nullptr, s));
+  const int F = (int)p->factors.size();
+  if (F == 0) return SA_OK;
+  std::vector<int> todo;
+  SACHECK(root_inverse_prologue(p, bias_correction2, epsilon, iterations_out, status_out, s, &todo));
+  if (todo.empty()) return SA_OK;
+  const int n = (int)todo.size();
+
+  // A = unpack(factor / bc2) + eps I (NB_M0); Qacc = current eigenbasis (NB_X1)
+  SACHECK(p->t_eiginit.begin(n));
+  SACHECK(p->t_copy.begin(n));
+  int tiles = 0;
+  for (int i = 0; i < n; ++i) {
+    const Factor& f = p->factors[todo[i]];
+    EigInit& J = p->t_eiginit.host[i];
+    std::memset(&J, 0, sizeof(J));
+    J.packed = f.factor; J.A = newton_buf(p, NB_M0, f); J.V = newton_buf(p, NB_MP0, f);
+    J.d = f.d; J.dpad = f.dpad; J.tiles = f.dpad / 64; J.enabled = 1; J.tile_begin = tiles;
+    tiles += J.tiles * J.tiles;
+    Copy2D& C = p->t_copy.host[i];
+    std::memset(&C, 0, sizeof(C));
+    C.src = f.eigvec; C.lds_ = f.d; C.dst = newton_buf(p, NB_X1, f); C.ldd = f.dpad; C.rows = f.d; C.cols = f.d;
+  }
+  SACHECK(p->t_eiginit.upload(s));
+  SACHECK(p->t_copy.upload(s));
+  hipLaunchKernelGGL(eig_init_kernel, dim3(tiles), dim3(256), 0, s, p->t_eiginit.dev, n, bias_correction2, epsilon);
+  hipLaunchKernelGGL(copy2d_kernel, dim3(64, n), dim3(256), 0, s, p->t_copy.dev);
+  HIPCHECK(hipGetLastError());
+
+  std::vector<int> active(F, 0), iters(F, 0);
+  for (int i : todo) active[i] = 1;
+  auto build_AQ = [&](bool also_B) -> int {
+    p->qr_aq.clear();
+    p->qr_b.clear();
+    for (int i : todo) {
+      const Factor& f = p->factors[i];
+      GemmProblem q{};
+      q.A = newton_buf(p, NB_M0, f); q.lda = f.dpad; q.a_vec = 1;
+      q.B = newton_buf(p, NB_X1, f); q.ldb = f.dpad; q.b_vec = 1;
+      q.C = newton_buf(p, NB_M1, f); q.ldc = f.dpad; q.M = q.N = q.K = f.d;
+      p->qr_aq.add(q, false);  // Y = A Qacc
+      if (also_B) {
+        GemmProblem b{};
+        b.A = newton_buf(p, NB_X1, f); b.lda = f.dpad; b.a_vec = 1;   // Qacc^T (A_KM)
+        b.B = newton_buf(p, NB_M1, f); b.ldb = f.dpad; b.b_vec = 1;
+        b.C = newton_buf(p, NB_X0, f); b.ldc = f.dpad; b.M = b.N = b.K = f.d;
+        p->qr_b.add(b, false);  // B = Qacc^T Y
+      }
+    }
+    SACHECK(p->qr_aq.commit(s));
+    SACHECK(p->qr_b.commit(s));
+    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE>(p->qr_aq, unit_scalars(), s)));
+    if (also_B) SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_STORE>(p->qr_b, unit_scalars(), s)));
+    return SA_OK;
+  };
+
+  for (int it = 0; it < max_iterations; ++it) {
+    SACHECK(build_AQ(true));
+    // criterion ||B - diag B||_F <= tol ||B||_F, evaluated like the reference (fp32, sqrt of a difference)
+    SACHECK(p->t_normpair.begin(n));
+    for (int k = 0; k < n; ++k) {
+      const Factor& f = p->factors[todo[k]];
+      NormPair& J = p->t_normpair.host[k];
+      J.B = newton_buf(p, NB_X0, f); J.ldb = f.dpad; J.d = f.d;
+      J.out_all = p->d_final_err + todo[k];
+      J.out_diag = reinterpret_cast<float*>(p->d_err) + todo[k];
+    }
+    SACHECK(p->t_normpair.upload(s));
+    hipLaunchKernelGGL(diag_off_norm_kernel, dim3(n), dim3(256), 0, s, p->t_normpair.dev);
+    HIPCHECK(hipGetLastError());
+    HIPCHECK(hipMemcpyAsync(p->h_pinned, p->d_final_err, F * sizeof(float), hipMemcpyDeviceToHost, s));
+    HIPCHECK(hipMemcpyAsync(p->h_pinned + F, p->d_err, F * sizeof(float), hipMemcpyDeviceToHost, s));
+    HIPCHECK(hipStreamSynchronize(s));
+    const float* h_all = reinterpret_cast<const float*>(p->h_pinned);
+    const float* h_diag = reinterpret_cast<const float*>(p->h_pinned + F);
+    std::vector<int> go;
+    for (int k = 0; k < n; ++k) {
+      const int i = todo[k];
+      if (!active[i]) continue;
+      const float norm = std::sqrt(h_all[i]), dnorm = std::sqrt(h_diag[i]);
+      const float off = std::sqrt(norm * norm - dnorm * dnorm);  // NaN when rounding makes it negative: iterate
+      const bool below = off <= tolerance * norm;
+      if (below) active[i] = 0; else go.push_back(i);
+    }
+    if (go.empty()) break;
+    HIPCHECK(hipMemcpyAsync(p->d_active, active.data(), F * sizeof(int), hipMemcpyHostToDevice, s));
+    HIPCHECK(hipStreamSynchronize(s));
+    double flops = 0.0;
+    for (int i : go) { const double d = p->factors[i].d; flops += (4.0 / 3.0 + 2.0) * d * d * d; }
+    {
+      Span span("qr_refresh", s, flops, 7 * ((p->factors[go[0]].d + 31) / 32), it == 0);
+      SACHECK(qr_accumulate(p, go, s));
+    }
+    for (int i : go) iters[i] += 1;
+  }
+  // eigenvalue estimates = Rayleigh quotients of the final basis, stable ascending order, permuted columns
+  SACHECK(build_AQ(false));
+  SACHECK(p->t_sort.begin(n));
+  SACHECK(p->t_copy.begin(n));
+  for (int k = 0; k < n; ++k) {
+    const Factor& f = p->factors[todo[k]];
+    SortJob& J = p->t_sort.host[k];
+    J.Q = newton_buf(p, NB_X1, f); J.ldq = f.dpad;
+    J.Y = newton_buf(p, NB_M1, f); J.ldy = f.dpad;
+    J.ev = newton_buf(p, NB_S2, f) + 2LL * f.dpad * QR_MAX_PANEL;
+    J.order = reinterpret_cast<int*>(J.ev + f.dpad);
+    J.d = f.d;
+    Copy2D& C = p->t_copy.host[k];
+    std::memset(&C, 0, sizeof(C));
+    C.src = newton_buf(p, NB_X1, f); C.lds_ = f.dpad; C.dst = newton_buf(p, NB_X0, f); C.ldd = f.dpad;
+    C.rows = f.d; C.cols = f.d; C.perm = J.order;
+  }
+  SACHECK(p->t_sort.upload(s));
+  SACHECK(p->t_copy.upload(s));
+  hipLaunchKernelGGL(rayleigh_sort_kernel, dim3(n), dim3(256), 0, s, p->t_sort.dev);
+  hipLaunchKernelGGL(copy2d_kernel, dim3(64, n), dim3(256), 0, s, p->t_copy.dev);  // sorted basis -> NB_X0
+  HIPCHECK(hipGetLastError());
+
+  // finiteness of the new bases, then copy those that precede the first bad one into the state
+  const int Fall = F;
+  int* h_bad = p->h_pinned + 3 * Fall;
+  HIPCHECK(hipMemsetAsync(p->d_flags, 0, Fall * sizeof(int), s));
+  SACHECK(p->t_normjobs.begin(n));
+  int chunks = 0;
+  for (int k = 0; k < n; ++k) {
+    const Factor& f = p->factors[todo[k]];
+    NormJob& J = p->t_normjobs.host[k];
+    std::memset(&J, 0, sizeof(J));
+    J.src = newton_buf(p, NB_X0, f); J.nonfinite = p->d_flags + todo[k];
+    J.d = f.d; J.dpad = f.dpad; J.dense = 1; J.chunk_begin = chunks;
+    J.n_chunks = (int)(((long long)f.d * f.d + NORM_CHUNK - 1) / NORM_CHUNK); J.enabled = 1;
+    chunks += J.n_chunks;
+  }
+  SACHECK(p->t_normjobs.upload(s));
+  hipLaunchKernelGGL((factor_norm_kernel<true>), dim3(chunks), dim3(256), 0, s, p->t_normjobs.dev, n, 1.0f, 0.0f);
+  HIPCHECK(hipGetLastError());
+  HIPCHECK(hipMemcpyAsync(h_bad, p->d_flags, Fall * sizeof(int), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipStreamSynchronize(s));
+  int ok = n;
+  for (int k = 0; k < n; ++k) {
+    iterations_out[todo[k]] = iters[todo[k]];
+    if (k < ok && h_bad[todo[k]]) { status_out[todo[k]] = SA_FACTOR_RESULT_NONFINITE; ok = k; }
+  }
+  if (ok > 0) {
+    SACHECK(p->t_copy.begin(ok));
+    for (int k = 0; k < ok; ++k) {
+      const Factor& f = p->factors[todo[k]];
+      Copy2D& C = p->t_copy.host[k];
+      std::memset(&C, 0, sizeof(C));
+      C.src = newton_buf(p, NB_X0, f); C.lds_ = f.dpad; C.dst = f.eigvec; C.ldd = f.d; C.rows = f.d; C.cols = f.d;
+      status_out[todo[k]] = SA_FACTOR_OK;
+    }
+    SACHECK(p->t_copy.upload(s));
+    hipLaunchKernelGGL(copy2d_kernel, dim3(64, ok), dim3(256), 0, s, p->t_copy.dev);
+    HIPCHECK(hipGetLastError());
+    HIPCHECK(hipStreamSynchronize(s));
+  }
   return SA_OK;
 }
 

@@ -28,6 +28,7 @@ from optimizers_amd.matrix_functions_types import (
     EigendecompositionConfig,
     PerturbationConfig,
     PseudoInverseConfig,
+    QREigendecompositionConfig,
 )
 from optimizers_amd.shampoo_types import (
     ADAGRAD,
@@ -62,6 +63,7 @@ from optimizers_amd.shampoo_types import (
     DefaultShampooRuntimeConfig,
     DefaultSingleDeviceDistributedConfig,
     DistributedConfig,
+    EigenvalueCorrectedShampooPreconditionerConfig,
     IterateAveragingConfig,
     PreconditionerConfig,
     PreconditionerValueError,
@@ -153,11 +155,26 @@ class _NativeGroup:
         # which dims carry a Kronecker factor, and with which root
         self.selectors: list[tuple[bool, ...]] = []
         self.roots: list[tuple[float, ...]] = []
+        self.soap = isinstance(pc, EigenvalueCorrectedShampooPreconditionerConfig)
         for i in self.native_index:
             order = self.block_specs[i].order
-            exps = [self._inverse_exponent(pc, d, order) for d in range(order)]
-            self.selectors.append(tuple(e != 0.0 for e in exps))
-            self.roots.append(tuple(1 / e for e in exps if e != 0.0))
+            if self.soap:
+                # shampoo_preconditioner_list.py:1843-1865: one root for the corrected eigenvalues
+                ignored = pc.ignored_basis_change_dims.get(order, [])
+                sel = tuple(d not in ignored for d in range(order))
+                self.selectors.append(sel)
+                self.roots.append((1 / pc.inverse_exponent_override.get(order, 1 / 2),) * sum(sel))
+                if not any(sel):
+                    raise NotImplementedError("a block with every basis change ignored is not built natively")
+            else:
+                exps = [self._inverse_exponent(pc, d, order) for d in range(order)]
+                self.selectors.append(tuple(e != 0.0 for e in exps))
+                self.roots.append(tuple(1 / e for e in exps if e != 0.0))
+        if self.soap:
+            distinct = {1 / pc.inverse_exponent_override.get(self.block_specs[i].order, 1 / 2) for i in self.native_index}
+            if len(distinct) > 1:
+                raise NotImplementedError("different eigenvalue exponents per tensor order are not built natively")
+            self.soap_root = distinct.pop() if distinct else 2.0
 
         numels = [self.block_specs[i].numel for i in self.native_index]
         fdims: list[int] = []
@@ -166,7 +183,9 @@ class _NativeGroup:
             fdims.extend(s.shape[d] for d in range(s.order) if self.selectors[k][d])
         packed = [d * (d + 1) // 2 for d in fdims]
         self.factor_arena = _Arena(packed, self.device)
-        self.inv_arena = _Arena(packed, self.device)
+        self.inv_arena = _Arena(packed, self.device) if not self.soap else None
+        self.eigvec_arena = _Arena([d * d for d in fdims], self.device) if self.soap else None
+        self.corrected_arena = _Arena(numels, self.device) if self.soap else None
         self.filtered_arena = _Arena(numels, self.device) if beta1 != 0.0 else None
         self.adagrad_arena = _Arena(numels, self.device) if self.graft_type == native.SA_GRAFT_ADAGRAD else None
         self.momentum_arena = _Arena(numels, self.device) if isinstance(momentum_cfg, ClassicMomentumConfig) else None
@@ -177,6 +196,7 @@ class _NativeGroup:
         self.factor_block: list[int] = []
         self.factor_roots: list[float] = []
         self.use_eigh = isinstance(pc.amortized_computation_config, EigenConfig)
+        self._slots: list[tuple[torch.Tensor, str, tuple, torch.Tensor]] = []
         self.bad_root_blocks: dict[int, str] = {}
         self.failed_counter: dict[int, int] = {}
         fi = 0
@@ -190,23 +210,40 @@ class _NativeGroup:
             else:
                 d.rows, d.cols, d.ld = s.shape[0], s.shape[1], s.strides[0]
             d.param = p.data_ptr() + 4 * s.offset
-            shampoo_state: dict[str, dict[int, torch.Tensor]] = {"factor_matrices": {}, "inv_factor_matrices": {}}
+            shampoo_state: dict[str, Any] = (
+                {"factor_matrices": {}, "factor_matrices_eigenvectors": {}}
+                if self.soap
+                else {"factor_matrices": {}, "inv_factor_matrices": {}}
+            )
+            if self.soap:
+                shampoo_state["corrected_eigenvalues"] = self.corrected_arena.view(k, s.shape)
+                d.corrected_eigenvalues = shampoo_state["corrected_eigenvalues"].data_ptr()
+                self._slots.append((p, s.block_key, (SHAMPOO, "corrected_eigenvalues"), shampoo_state["corrected_eigenvalues"]))
             slot = 0
             for dim in range(s.order):
                 if not self.selectors[k][dim]:
                     continue
                 n = s.shape[dim]
                 f = self.factor_arena.view(fi, (n * (n + 1) // 2,))
-                inv = self.inv_arena.view(fi, (n * (n + 1) // 2,))
-                idx = torch.arange(n, device=self.device)
-                inv[idx * n - idx * (idx - 1) // 2] = 1.0  # packed identity
                 shampoo_state["factor_matrices"][slot] = f
-                shampoo_state["inv_factor_matrices"][slot] = inv
                 d.factor[dim] = f.data_ptr()
-                d.inv_factor[dim] = inv.data_ptr()
+                self._slots.append((p, s.block_key, (SHAMPOO, "factor_matrices", slot), f))
+                if self.soap:
+                    q = self.eigvec_arena.view(fi, (n, n))
+                    q.copy_(torch.eye(n, device=self.device))
+                    shampoo_state["factor_matrices_eigenvectors"][slot] = q
+                    d.eigenvectors[dim] = q.data_ptr()
+                    self._slots.append((p, s.block_key, (SHAMPOO, "factor_matrices_eigenvectors", slot), q))
+                else:
+                    inv = self.inv_arena.view(fi, (n * (n + 1) // 2,))
+                    idx = torch.arange(n, device=self.device)
+                    inv[idx * n - idx * (idx - 1) // 2] = 1.0  # packed identity
+                    shampoo_state["inv_factor_matrices"][slot] = inv
+                    d.inv_factor[dim] = inv.data_ptr()
+                    self._slots.append((p, s.block_key, (SHAMPOO, "inv_factor_matrices", slot), inv))
                 root = Fraction(self.roots[k][slot])
                 self.factor_roots.append(float(self.roots[k][slot]))
-                if self.use_eigh:
+                if self.use_eigh or self.soap:
                     d.root[dim] = max(int(round(self.roots[k][slot])), 1)  # unused by the eigh path
                 elif root.denominator != 1:
                     # the reference raises inside matrix_inverse_root at every amortized step and
@@ -225,12 +262,15 @@ class _NativeGroup:
             if self.adagrad_arena is not None:
                 block_state[ADAGRAD] = self.adagrad_arena.view(k, s.shape)
                 d.adagrad = block_state[ADAGRAD].data_ptr()
+                self._slots.append((p, s.block_key, (ADAGRAD,), block_state[ADAGRAD]))
             if self.filtered_arena is not None:
                 block_state[FILTERED_GRAD] = self.filtered_arena.view(k, s.shape)
                 d.filtered_grad = block_state[FILTERED_GRAD].data_ptr()
+                self._slots.append((p, s.block_key, (FILTERED_GRAD,), block_state[FILTERED_GRAD]))
             if self.momentum_arena is not None:
                 block_state[MOMENTUM_BUFFER] = self.momentum_arena.view(k, s.shape)
                 d.momentum_buffer = block_state[MOMENTUM_BUFFER].data_ptr()
+                self._slots.append((p, s.block_key, (MOMENTUM_BUFFER,), block_state[MOMENTUM_BUFFER]))
             logger.info(
                 f"Instantiated Shampoo Preconditioner {s.param_index}.{s.block_key} for Parameter {s.param_index} "
                 f"({tuple(p.shape)}), Block {s.block_key} ({s.shape})."
@@ -277,10 +317,17 @@ class _NativeGroup:
     def _check_supported(group: dict[str, Any], pc: PreconditionerConfig) -> None:
         if not isinstance(group[DISTRIBUTED_CONFIG], SingleDeviceDistributedConfig):
             raise NotImplementedError(f"{group[DISTRIBUTED_CONFIG]=} not supported!")
-        if not isinstance(pc, RootInvShampooPreconditionerConfig):
+        if not isinstance(pc, (RootInvShampooPreconditionerConfig, EigenvalueCorrectedShampooPreconditionerConfig)):
             raise NotImplementedError(f"{pc=} not supported!")
         acc = pc.amortized_computation_config
-        if isinstance(acc, EigenConfig):
+        if isinstance(pc, EigenvalueCorrectedShampooPreconditionerConfig):
+            if not isinstance(acc, QREigendecompositionConfig):
+                raise NotImplementedError(
+                    f"Eigendecomposition config is not implemented! Specified eigendecomposition config is {type(acc).__name__}."
+                )
+            if pc.factor_matrix_eigenvectors_dtype != torch.float32 or pc.corrected_eigenvalues_dtype != torch.float32:
+                raise NotImplementedError("eigenvectors and corrected eigenvalues are fp32 in the native step")
+        elif isinstance(acc, EigenConfig):
             if not isinstance(acc.rank_deficient_stability_config, PerturbationConfig):
                 raise NotImplementedError(f"{acc.rank_deficient_stability_config=} is not supported.")
             if acc.eigendecomposition_offload_device != "":
@@ -291,7 +338,7 @@ class _NativeGroup:
             )
         if not pc.use_symmetric_packing:
             raise NotImplementedError("use_symmetric_packing=False: the native step keeps factors packed")
-        if pc.factor_matrix_dtype != torch.float32 or pc.inv_factor_matrix_dtype != torch.float32:
+        if pc.factor_matrix_dtype != torch.float32 or getattr(pc, "inv_factor_matrix_dtype", torch.float32) != torch.float32:
             raise NotImplementedError("factor matrices are fp32 in the native step")
         if pc.use_trace_scaling:
             raise NotImplementedError("use_trace_scaling is not built")
@@ -396,6 +443,10 @@ class _NativeGroup:
             bc2 = float(torch.tensor(1.0) - beta2**step)
         if amortize:
             self._amortized_computation(group, bc2, stream)
+        if self.soap:
+            native.check(
+                lib.sa_update_corrected_eigenvalues(self.plan, beta2, weighting, stream), "sa_update_corrected_eigenvalues"
+            )
 
         s = native.StepScalars()
         s.lr = lr
@@ -434,7 +485,13 @@ class _NativeGroup:
                 lib.sa_update_grafting_and_filtered_grad(self.plan, ref, stream),
                 "sa_update_grafting_and_filtered_grad",
             )
-            native.check(lib.sa_precondition(self.plan, ref, stream), "sa_precondition")
+            if self.soap:
+                native.check(
+                    lib.sa_precondition_eigenvalue_corrected(self.plan, ref, bc2, group[EPSILON], self.soap_root, stream),
+                    "sa_precondition_eigenvalue_corrected",
+                )
+            else:
+                native.check(lib.sa_precondition(self.plan, ref, stream), "sa_precondition")
             native.check(lib.sa_apply_update(self.plan, ref, stream), "sa_apply_update")
         # drop the references so param.grad can be freed (distributed_shampoo.py:1666-1667)
         self._grads_alive = None
@@ -444,7 +501,14 @@ class _NativeGroup:
         (shampoo_preconditioner_list.py:314-443)."""
         pc = self.preconditioner_config
         cfg = pc.amortized_computation_config
-        if self.use_eigh:
+        if self.soap:
+            native.check(
+                self.lib.sa_refresh_eigenbases_qr(
+                    self.plan, bc2, group[EPSILON], cfg.max_iterations, cfg.tolerance, self.iterations, self.status, stream
+                ),
+                "sa_refresh_eigenbases_qr",
+            )
+        elif self.use_eigh:
             roots = (ctypes.c_float * max(self.n_factors, 1))(*self.factor_roots)
             native.check(
                 self.lib.sa_compute_root_inverses_eigh(
@@ -477,7 +541,9 @@ class _NativeGroup:
                     "To mitigate, check factor matrix before the matrix computation."
                 )
             if st == native.SA_FACTOR_NOT_CONVERGED:
-                if self.use_eigh:
+                if self.soap:
+                    pass
+                elif self.use_eigh:
                     logger.warning(f"Jacobi eigensolver still rotating after {self.max_jacobi_sweeps} sweeps for factor matrix {name}.")
                 else:
                     logger.warning("Newton did not converge and reached maximum number of iterations!")
@@ -651,42 +717,21 @@ class DistributedShampoo(torch.optim.Optimizer):
 
 
 def _restore_state(self: _NativeGroup, optimizer: DistributedShampoo) -> None:
-    loaded_steps = []
-    fi = 0
-    for k, i in enumerate(self.native_index):
-        s = self.block_specs[i]
-        p = self.params[s.param_index]
-        st = optimizer.state[p]
-        block = st.get(s.block_key, {})
-        slot = 0
-        sh = block.get(SHAMPOO, {"factor_matrices": {}, "inv_factor_matrices": {}})
-        for dim in range(s.order):
-            if not self.selectors[k][dim]:
-                continue
-            n = s.shape[dim]
-            shape = (n * (n + 1) // 2,)
-            for key, arena in (("factor_matrices", self.factor_arena), ("inv_factor_matrices", self.inv_arena)):
-                mine = arena.view(fi, shape)
-                src = sh[key].get(slot, sh[key].get(str(slot))) if key in sh else None
-                if src is not None and src.data_ptr() != mine.data_ptr():
-                    mine.copy_(src)
-                sh.setdefault(key, {})[slot] = mine
-                sh[key].pop(str(slot), None)
-            slot += 1
-            fi += 1
-        block[SHAMPOO] = sh
-        for key, arena in ((ADAGRAD, self.adagrad_arena), (FILTERED_GRAD, self.filtered_arena), (MOMENTUM_BUFFER, self.momentum_arena)):
-            if arena is None:
-                continue
-            mine = arena.view(k, s.shape)
-            src = block.get(key)
-            if src is not None and src.data_ptr() != mine.data_ptr():
-                mine.copy_(src)
-            block[key] = mine
-        st[s.block_key] = block
-    for p in self.params:
-        if STEP in optimizer.state[p]:
-            loaded_steps.append(int(optimizer.state[p][STEP]))
+    for param, block_key, path, mine in self._slots:
+        node = optimizer.state[param].setdefault(block_key, {})
+        for key in path[:-1]:
+            nxt = node.get(key, node.get(str(key))) if isinstance(node, dict) else None
+            if nxt is None:
+                nxt = {}
+                node[key] = nxt
+            node = nxt
+        last = path[-1]
+        src = node.get(last, node.get(str(last)))
+        if src is not None and src.data_ptr() != mine.data_ptr():
+            mine.copy_(src.to(device=mine.device, dtype=mine.dtype).reshape(mine.shape))
+        node.pop(str(last), None)
+        node[last] = mine
+    loaded_steps = [int(optimizer.state[p][STEP]) for p in self.params if STEP in optimizer.state[p]]
     if loaded_steps:
         assert len(set(loaded_steps)) == 1, f"parameters of one group disagree on step: {sorted(set(loaded_steps))}"
         self.step_tensor.fill_(loaded_steps[0])

@@ -29,8 +29,9 @@ def test_library_loads_and_exports_every_declared_symbol():
 def test_struct_layouts_match_the_header():
     import ctypes
 
-    # sa_block_desc: 2*int32, int64, 4 pointers, 2+2 pointers, 2*int32 -> 88 bytes on LP64
-    assert ctypes.sizeof(native.BlockDesc) == 88
+    # sa_block_desc: 2*int32, int64, 4 pointers, 2+2 pointers, 2*int32, 2+1 pointers -> 112 bytes on LP64
+    assert ctypes.sizeof(native.BlockDesc) == 112
+    assert native.BlockDesc.eigenvectors.offset == 88 and native.BlockDesc.corrected_eigenvalues.offset == 104
     assert native.BlockDesc.ld.offset == 8 and native.BlockDesc.factor.offset == 48
     assert native.BlockDesc.root.offset == 80
     assert ctypes.sizeof(native.StepScalars) == 52
