@@ -14,6 +14,7 @@ from __future__ import annotations
 
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -39,13 +40,31 @@ WORKLOADS = {
         + [(50257, 768)],
         max_preconditioner_dim=1024, grad_std=0.02, lr=1e-3, betas=(0.9, 0.999), epsilon=1e-12,
         graft_beta2=0.999, graft_eps=1e-8,
+        # the ragged 81 x 768 tail block of the embedding gives an order-768 factor that is rank
+        # deficient (and makes the reference raise) until it has seen ten gradients
+        start_preconditioning_step=11, distinct_gradients=12,
     ),
     # BASELINE config 1
     "cfg1": dict(
         shapes=[(512, 512), (512,)], max_preconditioner_dim=512, grad_std=1.0, lr=1e-3, betas=(0.9, 0.999),
         epsilon=1e-12, graft_beta2=0.999, graft_eps=1e-8,
     ),
+    # BASELINE config 4: the same Llama layer, eigenvalue-corrected Shampoo (SOAP), QR refresh every 10 steps
+    "llama3_8b_layer_soap": dict(
+        shapes=[(4096, 4096), (1024, 4096), (1024, 4096), (4096, 4096), (14336, 4096), (14336, 4096),
+                (4096, 14336), (4096,), (4096,)],
+        max_preconditioner_dim=1024, grad_std=1e-2, low_rank=(32, 1e-3), lr=1e-3, betas=(0.9, 0.999), epsilon=1e-12,
+        preconditioner="soap_qr", precondition_frequency=10, start_preconditioning_step=10, grafting=None,
+    ),
+    # BASELINE config 5: 4096-blocks, eigendecomposition root inverse every 50 steps
+    "large_block_eigh": dict(
+        shapes=[(4096, 4096)] * 8 + [(8192, 4096)] * 4,
+        max_preconditioner_dim=4096, spectrum=(1e-6, 1.0), lr=1e-3, betas=(0.9, 0.999), epsilon=1e-12,
+        preconditioner="eigh", precondition_frequency=50, start_preconditioning_step=50,
+        graft_beta2=0.999, graft_eps=1e-8, distinct_gradients=2,
+    ),
 }
+DOMINANT_PHASE = {"newton": "newton_gemm", "soap_qr": "precondition_gemm", "eigh": "jacobi"}
 # Deviations from the configs as literally stated, needed for the REFERENCE to run at all
 # (both verified against the real reference, see tests/golden/cfg1_as_stated.json):
 #  * 1-D blocks (bias / norm vectors) are left to grafting (inverse_exponent_override={1: {0: 0.0}}):
@@ -66,14 +85,23 @@ def build(workload: dict, device):
     params = [
         torch.nn.Parameter(0.02 * torch.randn(*s, device=device, generator=gen)) for s in workload["shapes"]
     ]
+    kind = workload.get("preconditioner", "newton")
+    if kind == "newton":
+        pc = oa.RootInvShampooPreconditionerConfig(
+            amortized_computation_config=oa.CoupledNewtonConfig(), inverse_exponent_override={1: {0: 0.0}})
+    elif kind == "eigh":
+        pc = oa.RootInvShampooPreconditionerConfig(amortized_computation_config=oa.EigenConfig())
+    else:
+        pc = oa.DefaultSOAPConfig
+    graft = None
+    if workload.get("grafting", "adam") == "adam":
+        graft = oa.AdamPreconditionerConfig(beta2=workload["graft_beta2"], epsilon=workload["graft_eps"])
     opt = oa.DistributedShampoo(
         params, lr=workload["lr"], betas=workload["betas"], epsilon=workload["epsilon"],
-        max_preconditioner_dim=workload["max_preconditioner_dim"], precondition_frequency=1,
-        start_preconditioning_step=START_PRECONDITIONING_STEP,
-        preconditioner_config=oa.RootInvShampooPreconditionerConfig(
-            amortized_computation_config=oa.CoupledNewtonConfig(), inverse_exponent_override={1: {0: 0.0}}
-        ),
-        grafting_config=oa.AdamPreconditionerConfig(beta2=workload["graft_beta2"], epsilon=workload["graft_eps"]),
+        max_preconditioner_dim=workload["max_preconditioner_dim"],
+        precondition_frequency=workload.get("precondition_frequency", 1),
+        start_preconditioning_step=workload.get("start_preconditioning_step", START_PRECONDITIONING_STEP),
+        preconditioner_config=pc, grafting_config=graft,
     )
     return params, opt
 
@@ -82,7 +110,25 @@ def make_grads(workload: dict, params, step: int, device):
     import torch
 
     gen = torch.Generator(device=device).manual_seed(1000 + step)
-    return [workload["grad_std"] * torch.randn(p.shape, device=device, generator=gen) for p in params]
+    out = []
+    for p in params:
+        if "spectrum" in workload and p.dim() == 2:
+            # G = U diag(s) V^T with Haar U, V (QR of Gaussians) and log-uniform singular values
+            lo, hi = workload["spectrum"]
+            m, n = p.shape
+            u, _ = torch.linalg.qr(torch.randn(m, n, device=device, generator=gen))
+            w, _ = torch.linalg.qr(torch.randn(n, n, device=device, generator=gen))
+            sv = torch.exp(torch.empty(n, device=device).uniform_(math.log(lo), math.log(hi), generator=gen))
+            out.append(((u * sv) @ w.T).contiguous())
+            continue
+        g = workload.get("grad_std", 1.0) * torch.randn(p.shape, device=device, generator=gen)
+        if "low_rank" in workload and p.dim() == 2:
+            r, scale = workload["low_rank"]
+            a = torch.randn(p.shape[0], r, device=device, generator=gen)
+            c = torch.randn(r, p.shape[1], device=device, generator=gen)
+            g.add_(a @ c, alpha=scale / r)
+        out.append(g)
+    return out
 
 
 def cpu_baseline(workload: dict, name: str, budget_s: float = 25.0) -> dict:
@@ -147,8 +193,8 @@ def cpu_baseline(workload: dict, name: str, budget_s: float = 25.0) -> dict:
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=6)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=None, help="default: 6, or one precondition_frequency period")
+    ap.add_argument("--warmup", type=int, default=None, help="default: 3, or start_preconditioning_step")
     ap.add_argument("--workload", default="llama3_8b_layer", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--symmetric-newton", action="store_true",
@@ -160,8 +206,6 @@ def main() -> None:
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build targets one MI355X; --gpus must be 1 (no collectives, no sharding).")
-    if args.warmup < START_PRECONDITIONING_STEP:
-        sys.exit(f"bench.py: --warmup must be >= {START_PRECONDITIONING_STEP} so that timed steps are full Shampoo steps.")
 
     import torch
 
@@ -170,17 +214,26 @@ def main() -> None:
     assert torch.cuda.is_available(), "bench.py needs an MI355X"
     device = torch.device("cuda:0")
     workload = WORKLOADS[args.workload]
+    start = workload.get("start_preconditioning_step", START_PRECONDITIONING_STEP)
+    freq = workload.get("precondition_frequency", 1)
+    if args.steps is None:
+        args.steps = 6 if freq == 1 else freq  # one full amortisation period
+    if args.warmup is None:
+        args.warmup = max(3, start + 1) if freq == 1 else start  # the first refresh is part of the warm-up
+    if args.warmup < start:
+        sys.exit(f"bench.py: --warmup must be >= {start} so that timed steps are full Shampoo steps.")
     lib = native.load()
     lib.sa_set_symmetric_newton(1 if args.symmetric_newton else 0)
     params, opt = build(workload, device)
     n_params = sum(p.numel() for p in params)
 
     total = args.warmup + args.steps
-    grads = [make_grads(workload, params, s, device) for s in range(1, total + 1)]
+    n_sets = min(total, workload.get("distinct_gradients", 8))  # pre-generated gradient sets, cycled
+    grads = [make_grads(workload, params, s, device) for s in range(1, n_sets + 1)]
     torch.cuda.synchronize()
 
     def one_step(i: int) -> None:
-        for p, g in zip(params, grads[i]):
+        for p, g in zip(params, grads[i % n_sets]):
             p.grad = g
         opt.step()
 
@@ -195,7 +248,7 @@ def main() -> None:
         del src, dst
 
     lib.sa_set_profiling(1)
-    phases = ("newton_gemm", "syrk", "precondition_gemm", "grafting", "apply")
+    phases = ("newton_gemm", "syrk", "precondition_gemm", "grafting", "apply", "jacobi", "qr_refresh", "eigenbasis_rotation")
     acc = {ph: [0.0, 0.0, 0] for ph in phases}  # ms, work, launches
     executed = 0.0
     iters = []
@@ -216,10 +269,14 @@ def main() -> None:
     lib.sa_set_profiling(0)
     ms_per_step = 1e3 * elapsed / args.steps
 
-    ng_ms, ng_flops, ng_launches = acc["newton_gemm"]
+    kind = workload.get("preconditioner", "newton")
+    dominant = DOMINANT_PHASE[kind]
+    ng_ms, ng_flops, ng_launches = acc[dominant]
     achieved = ng_flops / (ng_ms * 1e-3) / 1e12 if ng_ms > 0 else 0.0
     roofline = {
-        "kernel": "grouped_gemm_kernel (coupled-Newton X*Mp, Mp^2, Mp^4, Mp^4*M)",
+        "kernel": {"newton_gemm": "grouped_gemm_kernel (coupled-Newton X*Mp, Mp^2, Mp^4, Mp^4*M)",
+                   "precondition_gemm": "grouped_gemm_kernel (eigenbasis rotations Q_L^T G Q_R, Q_L P Q_R^T)",
+                   "jacobi": "jacobi_cols_kernel + jacobi_rows_kernel + jacobi_pivot_kernel (block Jacobi sweeps)"}[dominant],
         "bound": "mfma",
         "achieved": achieved,
         "peak": PEAK_FP32_MFMA_TFLOPS,
@@ -236,7 +293,7 @@ def main() -> None:
         "launches": ng_launches,
     }
     detail = {}
-    for ph in ("syrk", "precondition_gemm"):
+    for ph in ("syrk", "precondition_gemm", "jacobi", "qr_refresh", "eigenbasis_rotation"):
         ms, work, n = acc[ph]
         if ms > 0:
             detail[ph] = {"ms_per_step": ms / args.steps, "TFLOP/s": work / (ms * 1e-3) / 1e12,
@@ -246,7 +303,7 @@ def main() -> None:
         if ms > 0:
             detail[ph] = {"ms_per_step": ms / args.steps, "GB/s": work / (ms * 1e-3) / 1e9,
                           "frac_of_hbm_peak": work / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS}
-    detail["newton_gemm"] = {"ms_per_step": ng_ms / args.steps}
+    detail[dominant] = dict(detail.get(dominant, {}), ms_per_step=ng_ms / args.steps)
     flat = [x for row in iters for x in row if x > 0]
     detail["newton_iterations_mean"] = sum(flat) / max(len(flat), 1)
     detail["newton_iterations_max"] = max(flat) if flat else 0
@@ -268,17 +325,17 @@ def main() -> None:
             "workload": args.workload,
             "parameters": n_params,
             "max_preconditioner_dim": workload["max_preconditioner_dim"],
-            "precondition_frequency": 1,
-            "start_preconditioning_step": START_PRECONDITIONING_STEP,
-            "root_inverse": "coupled_newton",
-            "grafting": "adam",
-            "inverse_exponent_override": "{1: {0: 0.0}}",
-            "grad_std": workload["grad_std"],
+            "precondition_frequency": freq,
+            "start_preconditioning_step": start,
+            "preconditioner": {"newton": "root inverse, coupled Newton", "eigh": "root inverse, eigendecomposition",
+                               "soap_qr": "eigenvalue-corrected (SOAP), QR refresh"}[kind],
+            "grafting": workload.get("grafting", "adam"),
+            "inverse_exponent_override": "{1: {0: 0.0}}" if kind == "newton" else "{}",
         },
         "roofline": roofline,
         "phases": detail,
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and kind == "newton":
         out["cpu_baseline"] = cpu_baseline(workload, args.workload)
     print(json.dumps(out))
 
