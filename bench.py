@@ -197,9 +197,10 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=None, help="default: 3, or start_preconditioning_step")
     ap.add_argument("--workload", default="llama3_8b_layer", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--symmetric-newton", action="store_true",
-                    help="compute only the upper triangle of every coupled-Newton product and mirror it (not the "
-                         "reference's arithmetic on ill-conditioned factors; off by default)")
+    ap.add_argument("--symmetric-newton", type=int, default=2, choices=(0, 1, 2),
+                    help="coupled-Newton products: 0 = full GEMMs (the reference's arithmetic), 1 = upper triangle "
+                         "mirrored, 2 (library default) = per factor, mirrored only while the factor's previous solve "
+                         "converged within 14 iterations (condition number <~ 1e4)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB copy kernel (sa::copy_kernel) so that rocprofv3 --pmc FETCH_SIZE / "
                          "WRITE_SIZE readings can be scaled against a kernel of known traffic")
@@ -223,7 +224,7 @@ def main() -> None:
     if args.warmup < start:
         sys.exit(f"bench.py: --warmup must be >= {start} so that timed steps are full Shampoo steps.")
     lib = native.load()
-    lib.sa_set_symmetric_newton(1 if args.symmetric_newton else 0)
+    lib.sa_set_symmetric_newton(args.symmetric_newton)
     params, opt = build(workload, device)
     n_params = sum(p.numel() for p in params)
 
@@ -283,9 +284,10 @@ def main() -> None:
         "unit": "TFLOP/s",
         "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
         "traffic": None,
-        # `achieved` bills the full-GEMM algorithmic flops (2 d^3 per product); `executed_frac` is what the
-        # matrix cores really sustained (they differ only with --symmetric-newton and through tile padding).
-        "symmetric_products": bool(args.symmetric_newton),
+        # `achieved` bills the algorithmic flops of the products issued (2 d^3 for a full product,
+        # d^2 (d + 1) for a symmetric one); `executed_frac` adds the padding and the mirrored halves of
+        # diagonal tiles, i.e. what the matrix cores really sustained.
+        "symmetric_products_policy": args.symmetric_newton,
         "executed_TFLOP/s": executed / (ng_ms * 1e-3) / 1e12 if ng_ms > 0 else 0.0,
         "executed_frac": executed / (ng_ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS if ng_ms > 0 else 0.0,
         "avg_launch_ms": ng_ms / max(ng_launches, 1),

@@ -199,12 +199,18 @@ int32_t sa_phase_launches(const char* phase);
 double sa_phase_executed_flops(const char* phase); /* flops actually issued by "newton_gemm" (symmetric products are halved) */
 
 /* Coupled Newton products are symmetric in exact arithmetic (every operand is a polynomial in the
- * factor).  When enabled only the tiles on or above the diagonal of each product are computed and
- * mirrored (1.9x fewer MFMA flops at d = 2048).  Off by default: every product is a full GEMM like the
- * reference's `@` (matrix_functions.py:426-427).  Measured: identical results (1e-6) on well conditioned
- * factors, but on factors with condition number > 1e5 the mirrored iteration deviates ~10x more from
- * exact arithmetic than the reference does.  Process-wide switch. */
-int32_t sa_set_symmetric_newton(int32_t enabled); /* kernel launches the phase issued in that call */
+ * factor).  A symmetric product computes only the tiles on or above the diagonal and mirrors them
+ * (1.9x fewer MFMA flops at d = 2048); the reference's `@` (matrix_functions.py:426-427) is a full GEMM.
+ * Both variants deviate from exact arithmetic by about 3e-9 x condition number (the symmetric one by about
+ * twice as much), so they agree to < 1e-4 while the factor's condition number is below 1e4, which shows
+ * as a solve of at most 14 iterations.  Policy, process wide:
+ *   0  every product is a full GEMM, the reference's arithmetic;
+ *   1  every product is symmetric;
+ *   2  (default) per factor: symmetric only if the factor's previous solve converged within 14 iterations;
+ *      a symmetric solve that then needs more than 17 iterations or does not converge is repeated with
+ *      full products, so failure semantics are those of policy 0.
+ * No counterpart in the reference. */
+int32_t sa_set_symmetric_newton(int32_t policy);
 
 #ifdef __cplusplus
 }

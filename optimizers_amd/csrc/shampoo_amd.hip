@@ -154,7 +154,13 @@ struct Phase {
   int launches = 0;
 };
 bool g_profiling = false;
-bool g_symmetric_newton = false;
+// Symmetric-product policy of the Newton GEMMs: 0 = always full products (the reference's arithmetic),
+// 1 = always upper-triangle tiles mirrored, 2 = per factor, symmetric only when the factor's previous solve
+// converged within SYM_MAX_PREVIOUS_ITERATIONS (condition number <~ 1e4, where the two variants agree to
+// < 1e-4; measured deviation grows like 3e-9 x condition number for both).
+int g_symmetric_newton = 2;
+constexpr int SYM_MAX_PREVIOUS_ITERATIONS = 14;
+constexpr int SYM_REDO_ITERATIONS = 17;  // a symmetric solve that needed more is repeated with full products
 std::map<std::string, Phase> g_phases;
 
 struct Span {
@@ -220,7 +226,9 @@ struct sa_plan {
   Table<ChunkRef> t_chunks;
   Table<int> t_active_blocks;
   GemmTable syrk0, syrk1, g1_store, g1_norm, g2_norm, g2g_norm;
-  GemmTable nt_a[2], nt_pow[8], nt_m[2];  // Newton: X/M_p^2 launch per parity, power chain, M update per parity
+  // Newton, [0] full products / [1] symmetric products: X*M_p with M_p^2 per parity, power chain, M update per parity
+  GemmTable nt_a[2][2], nt_pow[2][8], nt_m[2][2];
+  std::vector<int> newton_history;  // per factor: iterations of its last converged solve, 0 = none
   Table<SymFactor> t_sym;
   Table<NormJob> t_normjobs;
   Table<int> t_ids;
@@ -543,7 +551,7 @@ double sa_phase_executed_flops(const char* phase) {
   return it == g_phases.end() ? -1.0 : it->second.executed;
 }
 int32_t sa_set_symmetric_newton(int32_t enabled) {
-  g_symmetric_newton = enabled != 0;
+  g_symmetric_newton = enabled < 0 ? 0 : (enabled > 2 ? 2 : enabled);
   return SA_OK;
 }
 int32_t sa_phase_launches(const char* phase) {
@@ -633,10 +641,11 @@ int32_t sa_plan_create(const sa_block_desc* blocks, int32_t n_blocks, sa_plan** 
 void sa_plan_destroy(sa_plan* p) {
   if (!p) return;
   p->t_blocks.destroy(); p->t_chunks.destroy(); p->t_active_blocks.destroy();
-  for (GemmTable* g : {&p->syrk0, &p->syrk1, &p->g1_store, &p->g1_norm, &p->g2_norm, &p->g2g_norm, &p->nt_a[0],
-                       &p->nt_a[1], &p->nt_m[0], &p->nt_m[1]})
+  for (GemmTable* g : {&p->syrk0, &p->syrk1, &p->g1_store, &p->g1_norm, &p->g2_norm, &p->g2g_norm, &p->nt_a[0][0],
+                       &p->nt_a[0][1], &p->nt_m[0][0], &p->nt_m[0][1], &p->nt_a[1][0], &p->nt_a[1][1], &p->nt_m[1][0],
+                       &p->nt_m[1][1]})
     g->t.destroy();
-  for (auto& g : p->nt_pow) g.t.destroy();
+  for (auto& row : p->nt_pow) for (auto& g : row) g.t.destroy();
   p->t_sym.destroy(); p->t_normjobs.destroy(); p->t_ids.destroy();
   p->t_jacobi.destroy(); p->t_sched.destroy(); p->t_eiginit.destroy(); p->t_eigfinal.destroy(); p->eig_gemm.t.destroy();
   for (GemmTable* g : {&p->ec_stat1, &p->ec_stat2, &p->ec_stat_l, &p->ec_stat_r, &p->ec_p1, &p->ec_p1d, &p->ec_p2, &p->ec_p2d,
@@ -822,8 +831,9 @@ int32_t sa_plan_read_preconditioned(sa_plan* p, int32_t block, float* out, void*
 // Batched coupled inverse Newton
 // --------------------------------------------------------------------------------------------
 
-static int newton_batch(sa_plan* p, const std::vector<int>& ids, int root, float eps, float bc2, int max_iter, float tol,
-                        hipStream_t s, double* flops_acc, int* launches_acc) {
+// `symmetric[i]` selects the product variant of ids[i].
+static int newton_batch(sa_plan* p, const std::vector<int>& ids, const std::vector<char>& symmetric, int root, float eps,
+                        float bc2, int max_iter, float tol, hipStream_t s, double* flops_acc, int* launches_acc) {
   const int n = (int)ids.size();
   if (n == 0) return SA_OK;
   // torch.linalg.matrix_power(M_p, root): squarings (and one extra product for root 3)
@@ -839,7 +849,6 @@ static int newton_batch(sa_plan* p, const std::vector<int>& ids, int root, float
     }
   }
   if (std::max(squarings - 1, 0) + (cube ? 1 : 0) > 4) return fail(SA_ERR_UNSUPPORTED, "root too large for the power chain");
-  const bool sym = g_symmetric_newton;
   const float alpha = (float)(-1.0 / root);          // M.mul(alpha)
   const float one_minus_alpha = (float)(1.0 - (-1.0 / root));  // .add_(I, alpha = 1 - alpha)
 
@@ -870,8 +879,10 @@ static int newton_batch(sa_plan* p, const std::vector<int>& ids, int root, float
   HIPCHECK(hipGetLastError());
 
   // ---- GEMM tables -------------------------------------------------------------------------
-  for (int par = 0; par < 2; ++par) { p->nt_a[par].clear(); p->nt_m[par].clear(); }
-  for (int k = 0; k < 8; ++k) p->nt_pow[k].clear();
+  for (int v = 0; v < 2; ++v) {
+    for (int par = 0; par < 2; ++par) { p->nt_a[v][par].clear(); p->nt_m[v][par].clear(); }
+    for (int k = 0; k < 8; ++k) p->nt_pow[v][k].clear();
+  }
   auto prob = [&](const Factor& f, const float* A, const float* B, float* C) {
     GemmProblem q{};
     q.A = A; q.B = B; q.C = C;
@@ -884,6 +895,8 @@ static int newton_batch(sa_plan* p, const std::vector<int>& ids, int root, float
   };
   for (int i = 0; i < n; ++i) {
     const Factor& f = p->factors[ids[i]];
+    const bool sym = symmetric[i] != 0;
+    const int v = sym ? 1 : 0;
     // buffer that finally holds M_p^root (depends only on the chain length)
     const float* power = nullptr;
     for (int par = 0; par < 2; ++par) {
@@ -896,31 +909,33 @@ static int newton_batch(sa_plan* p, const std::vector<int>& ids, int root, float
       float* S1 = newton_buf(p, NB_S1, f);
       float* S2 = newton_buf(p, NB_S2, f);
       // launch A: X <- X M_p, and the first squaring if the root needs one
-      p->nt_a[par].add(prob(f, X, Mp, Xn), sym);
-      if (squarings >= 1) p->nt_a[par].add(prob(f, Mp, Mp, S1), sym);
+      p->nt_a[v][par].add(prob(f, X, Mp, Xn), sym);
+      if (squarings >= 1) p->nt_a[v][par].add(prob(f, Mp, Mp, S1), sym);
       // remaining chain reads only S1/S2/Mp of this parity; build it for parity-specific Mp when cube
       const float* cur = (squarings >= 1) ? S1 : Mp;
       int slot = par * 4;  // nt_pow[0..3] parity 0, [4..7] parity 1
       float* pong[2] = {S2, S1};
       int which = 0;
       for (int q = 1; q < squarings; ++q) {
-        p->nt_pow[slot++].add(prob(f, cur, cur, pong[which]), sym);
+        p->nt_pow[v][slot++].add(prob(f, cur, cur, pong[which]), sym);
         cur = pong[which];
         which ^= 1;
       }
       if (cube) {
-        p->nt_pow[slot++].add(prob(f, cur, Mp, pong[which]), sym);
+        p->nt_pow[v][slot++].add(prob(f, cur, Mp, pong[which]), sym);
         cur = pong[which];
       }
       power = cur;
       GemmProblem m = prob(f, power, M, Mn);
       m.C2 = Mpn;
       m.err_bits = p->d_err + ids[i];
-      p->nt_m[par].add(m, sym);
+      p->nt_m[v][par].add(m, sym);
     }
   }
-  for (int par = 0; par < 2; ++par) { SACHECK(p->nt_a[par].commit(s)); SACHECK(p->nt_m[par].commit(s)); }
-  for (int k = 0; k < 8; ++k) SACHECK(p->nt_pow[k].commit(s));
+  for (int v = 0; v < 2; ++v) {
+    for (int par = 0; par < 2; ++par) { SACHECK(p->nt_a[v][par].commit(s)); SACHECK(p->nt_m[v][par].commit(s)); }
+    for (int k = 0; k < 8; ++k) SACHECK(p->nt_pow[v][k].commit(s));
+  }
 
   NewtonCtl ctl{p->d_err, p->d_active, p->d_iters, p->d_final_parity, p->d_final_err};
   int parity = 0;
@@ -942,25 +957,29 @@ static int newton_batch(sa_plan* p, const std::vector<int>& ids, int root, float
       if (h_active[ids[i]]) {
         const Factor& f = p->factors[ids[i]];
         const double d = f.d, t = f.dpad / BM;
-        flops += 2.0 * d * d * d * gemms_per_iter;
+        const bool sym = symmetric[i] != 0;
+        flops += (sym ? d * d * (d + 1.0) : 2.0 * d * d * d) * gemms_per_iter;
         executed += 2.0 * BM * BN * (double)f.dpad * (sym ? t * (t + 1) / 2 : t * t) * gemms_per_iter;
         ++live;
       }
     if (!live) break;
     {
-      int nl = 2;
-      for (int k = 0; k < 4; ++k) nl += p->nt_pow[parity * 4 + k].total_tiles ? 1 : 0;
+      int nl = 0;
+      for (int v = 0; v < 2; ++v) {
+        nl += (p->nt_a[v][parity].total_tiles ? 1 : 0) + (p->nt_m[v][parity].total_tiles ? 1 : 0);
+        for (int k = 0; k < 4; ++k) nl += p->nt_pow[v][parity * 4 + k].total_tiles ? 1 : 0;
+      }
       Span span("newton_gemm", s, flops, nl, false);
       if (g_profiling) g_phases["newton_gemm"].executed += executed;
-      if (sym) {
-        SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, true>(p->nt_a[parity], unit, s)));
-        for (int k = 0; k < 4; ++k) SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, true>(p->nt_pow[parity * 4 + k], unit, s)));
-        SACHECK((launch_gemm<A_MK, B_KN, EPI_NEWTON_M, false, true>(p->nt_m[parity], msc, s)));
-      } else {
-        SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, false>(p->nt_a[parity], unit, s)));
-        for (int k = 0; k < 4; ++k) SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, false>(p->nt_pow[parity * 4 + k], unit, s)));
-        SACHECK((launch_gemm<A_MK, B_KN, EPI_NEWTON_M, false, false>(p->nt_m[parity], msc, s)));
+      // the two variants touch disjoint factors, so their launches of one stage are independent
+      SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, true>(p->nt_a[1][parity], unit, s)));
+      SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, false>(p->nt_a[0][parity], unit, s)));
+      for (int k = 0; k < 4; ++k) {
+        SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, true>(p->nt_pow[1][parity * 4 + k], unit, s)));
+        SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, false>(p->nt_pow[0][parity * 4 + k], unit, s)));
       }
+      SACHECK((launch_gemm<A_MK, B_KN, EPI_NEWTON_M, false, true>(p->nt_m[1][parity], msc, s)));
+      SACHECK((launch_gemm<A_MK, B_KN, EPI_NEWTON_M, false, false>(p->nt_m[0][parity], msc, s)));
       *flops_acc += flops;
       *launches_acc += nl;
     }
@@ -1088,28 +1107,54 @@ int32_t sa_compute_root_inverses_newton(sa_plan* p, float bias_correction2, floa
   SACHECK(root_inverse_prologue(p, bias_correction2, epsilon, iterations_out, status_out, s, &todo));
   if (todo.empty()) return SA_OK;
 
-  // iterate, one batch per distinct root
-  std::vector<int> ones(F, 0);
-  for (int i : todo) ones[i] = 1;
-  HIPCHECK(hipMemcpyAsync(p->d_active, ones.data(), F * sizeof(int), hipMemcpyHostToDevice, s));
-  HIPCHECK(hipStreamSynchronize(s));
-  std::map<int, std::vector<int>> by_root;
-  for (int i : todo) by_root[p->factors[i].root].push_back(i);
+  // iterate, one batch per distinct root; product variant per factor from the policy and the factor's history
+  if ((int)p->newton_history.size() != F) p->newton_history.assign(F, 0);
+  std::vector<char> sym(F, 0);
+  for (int i : todo) {
+    const int h = p->newton_history[i];
+    sym[i] = g_symmetric_newton == 1 || (g_symmetric_newton == 2 && h > 0 && h <= SYM_MAX_PREVIOUS_ITERATIONS);
+  }
+  std::vector<int> iters(F, 0), par(F, 0);
+  std::vector<float> errs(F, 0.0f);
   double flops = 0.0;
   int launches = 0;
-  for (auto& kv : by_root)
-    SACHECK(newton_batch(p, kv.second, kv.first, epsilon, bias_correction2, max_iterations, tolerance, s, &flops, &launches));
-
-  // iteration counts, final errors, parities
-  std::vector<int> iters(F), par(F);
-  std::vector<float> errs(F);
-  HIPCHECK(hipMemcpyAsync(p->h_pinned, p->d_iters, F * sizeof(int), hipMemcpyDeviceToHost, s));
-  HIPCHECK(hipMemcpyAsync(p->h_pinned + F, p->d_final_parity, F * sizeof(int), hipMemcpyDeviceToHost, s));
-  HIPCHECK(hipMemcpyAsync(p->h_pinned + 2 * F, p->d_final_err, F * sizeof(float), hipMemcpyDeviceToHost, s));
-  HIPCHECK(hipStreamSynchronize(s));
-  std::memcpy(iters.data(), p->h_pinned, F * sizeof(int));
-  std::memcpy(par.data(), p->h_pinned + F, F * sizeof(int));
-  std::memcpy(errs.data(), p->h_pinned + 2 * F, F * sizeof(float));
+  auto solve = [&](const std::vector<int>& subset) -> int {
+    std::vector<int> ones(F, 0);
+    for (int i : subset) ones[i] = 1;
+    HIPCHECK(hipMemsetAsync(p->d_err, 0, F * sizeof(int), s));
+    HIPCHECK(hipMemsetAsync(p->d_iters, 0, F * sizeof(int), s));
+    HIPCHECK(hipMemsetAsync(p->d_final_parity, 0, F * sizeof(int), s));
+    HIPCHECK(hipMemcpyAsync(p->d_active, ones.data(), F * sizeof(int), hipMemcpyHostToDevice, s));
+    HIPCHECK(hipStreamSynchronize(s));
+    std::map<int, std::vector<int>> by_root;
+    for (int i : subset) by_root[p->factors[i].root].push_back(i);
+    for (auto& kv : by_root) {
+      std::vector<char> variant(kv.second.size());
+      for (size_t k = 0; k < kv.second.size(); ++k) variant[k] = sym[kv.second[k]];
+      SACHECK(newton_batch(p, kv.second, variant, kv.first, epsilon, bias_correction2, max_iterations, tolerance, s, &flops,
+                           &launches));
+    }
+    // iteration counts, final errors, parities
+    HIPCHECK(hipMemcpyAsync(p->h_pinned, p->d_iters, F * sizeof(int), hipMemcpyDeviceToHost, s));
+    HIPCHECK(hipMemcpyAsync(p->h_pinned + F, p->d_final_parity, F * sizeof(int), hipMemcpyDeviceToHost, s));
+    HIPCHECK(hipMemcpyAsync(p->h_pinned + 2 * F, p->d_final_err, F * sizeof(float), hipMemcpyDeviceToHost, s));
+    HIPCHECK(hipStreamSynchronize(s));
+    for (int i : subset) {
+      iters[i] = p->h_pinned[i];
+      par[i] = p->h_pinned[F + i];
+      std::memcpy(&errs[i], p->h_pinned + 2 * F + i, sizeof(float));
+    }
+    return SA_OK;
+  };
+  SACHECK(solve(todo));
+  if (g_symmetric_newton == 2) {
+    // a factor whose conditioning worsened since its last solve gets the reference's full products after all
+    std::vector<int> redo;
+    for (int i : todo)
+      if (sym[i] && (iters[i] > SYM_REDO_ITERATIONS || !(errs[i] <= tolerance))) { redo.push_back(i); sym[i] = 0; }
+    if (!redo.empty()) SACHECK(solve(redo));
+  }
+  for (int i : todo) p->newton_history[i] = (errs[i] <= tolerance) ? iters[i] : 0;
 
   std::vector<const float*> X(todo.size());
   for (size_t i = 0; i < todo.size(); ++i) X[i] = newton_buf(p, par[todo[i]] ? NB_X1 : NB_X0, p->factors[todo[i]]);
