@@ -42,6 +42,17 @@ struct BlockDev {
 
 struct ChunkRef { int block; int start; };
 
+// 16-byte streaming (non-temporal) accesses: data touched once per step should not evict reusable lines
+typedef float vfloat4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 nt_load4(const float* p) {
+  const vfloat4 v = __builtin_nontemporal_load(reinterpret_cast<const vfloat4*>(p));
+  return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void nt_store4(const float4& x, float* p) {
+  vfloat4 v = {x.x, x.y, x.z, x.w};
+  __builtin_nontemporal_store(v, reinterpret_cast<vfloat4*>(p));
+}
+
 __device__ __forceinline__ float block_sum(float v, float* red) {
   v = wave_sum(v);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -125,8 +136,55 @@ __global__ __launch_bounds__(EW_THREADS) void grafting_kernel(const BlockDev* __
   const bool b3 = B.ghat_tmp != nullptr;
   const bool contig = (B.ld == B.cols);
   float gsum = 0.f, hsum = 0.f;
+  constexpr int NIT = EW_CHUNK / (EW_THREADS * 4);
+  // Whole, vectorisable chunk (the common case): every load is issued before the first use, so each
+  // thread keeps up to 16 x 16 bytes in flight; streamed data bypasses the caches it would only pollute.
+  const bool whole = (cr.start + EW_CHUNK <= n_el) && (B.vec != 0);
+  if (whole) {
+    long long gi[NIT];
+    float4 g[NIT], m[NIT], v[NIT], w[NIT], mo[NIT];
 #pragma unroll
-  for (int it = 0; it < EW_CHUNK / (EW_THREADS * 4); ++it) {
+    for (int it = 0; it < NIT; ++it) {
+      const int e = cr.start + (it * EW_THREADS + threadIdx.x) * 4;
+      gi[it] = contig ? (long long)e : (long long)(e / B.cols) * B.ld + (e % B.cols);
+      g[it] = nt_load4(B.grad + gi[it]);
+    }
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int e = cr.start + (it * EW_THREADS + threadIdx.x) * 4;
+      m[it] = has_m ? nt_load4(B.filtered_grad + e) : make_float4(0, 0, 0, 0);
+      v[it] = has_v ? nt_load4(B.adagrad + e) : make_float4(0, 0, 0, 0);
+      if (MODE == 1) {
+        w[it] = nt_load4(B.param + gi[it]);
+        mo[it] = has_mom ? nt_load4(B.momentum + e) : make_float4(0, 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int e = cr.start + (it * EW_THREADS + threadIdx.x) * 4;
+      float4 t = make_float4(0, 0, 0, 0);
+      PreOut o0 = pre_element(g[it].x, m[it].x, v[it].x, t.x, s, has_m, has_v, b3);
+      PreOut o1 = pre_element(g[it].y, m[it].y, v[it].y, t.y, s, has_m, has_v, b3);
+      PreOut o2 = pre_element(g[it].z, m[it].z, v[it].z, t.z, s, has_m, has_v, b3);
+      PreOut o3 = pre_element(g[it].w, m[it].w, v[it].w, t.w, s, has_m, has_v, b3);
+      if (has_m) nt_store4(m[it], B.filtered_grad + e);
+      if (has_v) nt_store4(v[it], B.adagrad + e);
+      if (b3) *reinterpret_cast<float4*>(B.ghat_tmp + e) = t;
+      if (MODE == 0) {
+        gsum += (o0.graft * o0.graft + o1.graft * o1.graft) + (o2.graft * o2.graft + o3.graft * o3.graft);
+        hsum += (o0.ghat * o0.ghat + o1.ghat * o1.ghat) + (o2.ghat * o2.ghat + o3.ghat * o3.ghat);
+      } else {
+        apply_element(o0.graft, w[it].x, mo[it].x, s, 1.0f, has_mom);
+        apply_element(o1.graft, w[it].y, mo[it].y, s, 1.0f, has_mom);
+        apply_element(o2.graft, w[it].z, mo[it].z, s, 1.0f, has_mom);
+        apply_element(o3.graft, w[it].w, mo[it].w, s, 1.0f, has_mom);
+        *reinterpret_cast<float4*>(B.param + gi[it]) = w[it];
+        if (has_mom) nt_store4(mo[it], B.momentum + e);
+      }
+    }
+  } else
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
     const int e = cr.start + (it * EW_THREADS + threadIdx.x) * 4;
     if (e >= n_el) continue;
     const long long gi = contig ? (long long)e : (long long)(e / B.cols) * B.ld + (e % B.cols);
@@ -238,8 +296,33 @@ __global__ __launch_bounds__(EW_THREADS) void apply_kernel(const BlockDev* __res
     const float pn = sqrtf(norms[n_blocks + cr.block]) + 1e-16f;
     scale = gn / pn;
   }
+  constexpr int NIT = EW_CHUNK / (EW_THREADS * 4);
+  const bool whole = (cr.start + EW_CHUNK <= n_el) && (B.vec != 0) && (B.p_vec != 0);
+  if (whole) {
+    long long wi[NIT];
+    float4 p[NIT], w[NIT], mo[NIT];
 #pragma unroll
-  for (int it = 0; it < EW_CHUNK / (EW_THREADS * 4); ++it) {
+    for (int it = 0; it < NIT; ++it) {
+      const int e = cr.start + (it * EW_THREADS + threadIdx.x) * 4;
+      wi[it] = contig ? (long long)e : (long long)(e / B.cols) * B.ld + (e % B.cols);
+      const long long pi = p_contig ? (long long)e : (long long)(e / B.cols) * B.p_ld + (e % B.cols);
+      p[it] = nt_load4(B.p_src + pi);
+      w[it] = nt_load4(B.param + wi[it]);
+      mo[it] = has_mom ? nt_load4(B.momentum + e) : make_float4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int e = cr.start + (it * EW_THREADS + threadIdx.x) * 4;
+      apply_element(p[it].x / p_div, w[it].x, mo[it].x, s, scale, has_mom);
+      apply_element(p[it].y / p_div, w[it].y, mo[it].y, s, scale, has_mom);
+      apply_element(p[it].z / p_div, w[it].z, mo[it].z, s, scale, has_mom);
+      apply_element(p[it].w / p_div, w[it].w, mo[it].w, s, scale, has_mom);
+      *reinterpret_cast<float4*>(B.param + wi[it]) = w[it];
+      if (has_mom) nt_store4(mo[it], B.momentum + e);
+    }
+  } else
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
     const int e = cr.start + (it * EW_THREADS + threadIdx.x) * 4;
     if (e >= n_el) continue;
     const long long wi = contig ? (long long)e : (long long)(e / B.cols) * B.ld + (e % B.cols);
