@@ -177,11 +177,31 @@ __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(
   {
     int t = logical - P.tile_begin;
     if (TRI) {
-      // upper-triangular tile enumeration, row by row
-      tm = 0;
-      int rowlen = P.tiles_n;
-      while (t >= rowlen) { t -= rowlen; ++tm; --rowlen; }
-      tn = tm + t;
+      // Upper-triangular tile enumeration in super-rows of GROUP_ROWS tile rows.  Inside a super-row the
+      // tiles are walked column by column (first the little triangle at the diagonal, then full columns
+      // of GROUP_ROWS tiles), so concurrently running workgroups share A row panels and B column panels.
+      const int T = P.tiles_n;
+      int r0 = 0;
+      for (;;) {
+        const int gsz = min(GROUP_ROWS, T - r0);
+        const int tri = gsz * (gsz + 1) / 2;
+        const int cnt = tri + (T - r0 - gsz) * gsz;
+        if (t < cnt) {
+          if (t < tri) {
+            int c = 0;
+            while (t > c) { t -= c + 1; ++c; }  // column c of the triangle holds c + 1 tiles
+            tm = r0 + t;
+            tn = r0 + c;
+          } else {
+            t -= tri;
+            tm = r0 + t % gsz;
+            tn = r0 + gsz + t / gsz;
+          }
+          break;
+        }
+        t -= cnt;
+        r0 += gsz;
+      }
     } else {
       const int per_group = GROUP_ROWS * P.tiles_n;
       const int g = t / per_group, r = t - g * per_group;
