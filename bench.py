@@ -64,6 +64,11 @@ WORKLOADS = {
         graft_beta2=0.999, graft_eps=1e-8, distinct_gradients=2,
     ),
 }
+# HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (two
+# runs, each scaled by what the counter reads for sa::copy_kernel's 1 GiB copy: 2.000 and 1.000); the
+# commands and per-kernel figures are in profiles/grouped_gemm_newton_llama3_8b_layer.md.  Keyed by
+# (workload, symmetric-product policy); None where no counter run was made.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {("llama3_8b_layer", 2): 13.8e9, ("llama3_8b_layer", 0): 9.02e9}
 DOMINANT_PHASE = {"newton": "newton_gemm", "soap_qr": "precondition_gemm", "eigh": "jacobi"}
 # Deviations from the configs as literally stated, needed for the REFERENCE to run at all
 # (both verified against the real reference, see tests/golden/cfg1_as_stated.json):
@@ -283,7 +288,7 @@ def main() -> None:
         "peak": PEAK_FP32_MFMA_TFLOPS,
         "unit": "TFLOP/s",
         "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
-        "traffic": None,
+        "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get((args.workload, args.symmetric_newton)),
         # `achieved` bills the algorithmic flops of the products issued (2 d^3 for a full product,
         # d^2 (d + 1) for a symmetric one); `executed_frac` adds the padding and the mirrored halves of
         # diagonal tiles, i.e. what the matrix cores really sustained.
