@@ -206,6 +206,8 @@ def main() -> None:
                     help="coupled-Newton products: 0 = full GEMMs (the reference's arithmetic), 1 = upper triangle "
                          "mirrored, 2 (library default) = per factor, mirrored only while the factor's previous solve "
                          "converged within 14 iterations (condition number <~ 1e4)")
+    ap.add_argument("--eigh-solver", type=int, default=0, choices=(0, 1, 2),
+                    help="EigenConfig root inverse: 0 = by order (library default), 1 = block Jacobi, 2 = tridiagonalisation")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB copy kernel (sa::copy_kernel) so that rocprofv3 --pmc FETCH_SIZE / "
                          "WRITE_SIZE readings can be scaled against a kernel of known traffic")
@@ -230,6 +232,7 @@ def main() -> None:
         sys.exit(f"bench.py: --warmup must be >= {start} so that timed steps are full Shampoo steps.")
     lib = native.load()
     lib.sa_set_symmetric_newton(args.symmetric_newton)
+    lib.sa_set_eigh_solver(args.eigh_solver)
     params, opt = build(workload, device)
     n_params = sum(p.numel() for p in params)
 
@@ -254,7 +257,8 @@ def main() -> None:
         del src, dst
 
     lib.sa_set_profiling(1)
-    phases = ("newton_gemm", "syrk", "precondition_gemm", "grafting", "apply", "jacobi", "qr_refresh", "eigenbasis_rotation")
+    phases = ("newton_gemm", "syrk", "precondition_gemm", "grafting", "apply", "jacobi", "qr_refresh", "eigenbasis_rotation",
+              "tridiagonalize", "form_q", "tridiagonal_ql")
     acc = {ph: [0.0, 0.0, 0] for ph in phases}  # ms, work, launches
     executed = 0.0
     iters = []
@@ -277,17 +281,22 @@ def main() -> None:
 
     kind = workload.get("preconditioner", "newton")
     dominant = DOMINANT_PHASE[kind]
+    if kind == "eigh":  # whichever of the roofline-bound phases took longest
+        dominant = max(("jacobi", "tridiagonalize", "precondition_gemm"), key=lambda ph: acc[ph][0])
     ng_ms, ng_flops, ng_launches = acc[dominant]
-    achieved = ng_flops / (ng_ms * 1e-3) / 1e12 if ng_ms > 0 else 0.0
+    hbm_bound = dominant == "tridiagonalize"
+    achieved = ng_flops / (ng_ms * 1e-3) / (1e9 if hbm_bound else 1e12) if ng_ms > 0 else 0.0
+    peak = PEAK_HBM_GBS if hbm_bound else PEAK_FP32_MFMA_TFLOPS
     roofline = {
         "kernel": {"newton_gemm": "grouped_gemm_kernel (coupled-Newton X*Mp, Mp^2, Mp^4, Mp^4*M)",
-                   "precondition_gemm": "grouped_gemm_kernel (eigenbasis rotations Q_L^T G Q_R, Q_L P Q_R^T)",
-                   "jacobi": "jacobi_cols_kernel + jacobi_rows_kernel + jacobi_pivot_kernel (block Jacobi sweeps)"}[dominant],
-        "bound": "mfma",
+                   "precondition_gemm": "grouped_gemm_kernel (preconditioning products / eigenbasis rotations)",
+                   "jacobi": "jacobi_cols_kernel + jacobi_rows_kernel + jacobi_pivot_kernel (block Jacobi sweeps)",
+                   "tridiagonalize": "trd_symv_kernel (trailing matrix times Householder vector) + trd_column_kernel"}[dominant],
+        "bound": "hbm" if hbm_bound else "mfma",
         "achieved": achieved,
-        "peak": PEAK_FP32_MFMA_TFLOPS,
-        "unit": "TFLOP/s",
-        "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
+        "peak": peak,
+        "unit": "GB/s" if hbm_bound else "TFLOP/s",
+        "frac": achieved / peak,
         "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get((args.workload, args.symmetric_newton)),
         # `achieved` bills the algorithmic flops of the products issued (2 d^3 for a full product,
         # d^2 (d + 1) for a symmetric one); `executed_frac` adds the padding and the mirrored halves of
@@ -300,12 +309,14 @@ def main() -> None:
         "launches": ng_launches,
     }
     detail = {}
-    for ph in ("syrk", "precondition_gemm", "jacobi", "qr_refresh", "eigenbasis_rotation"):
+    for ph in ("syrk", "precondition_gemm", "jacobi", "qr_refresh", "eigenbasis_rotation", "form_q"):
         ms, work, n = acc[ph]
         if ms > 0:
             detail[ph] = {"ms_per_step": ms / args.steps, "TFLOP/s": work / (ms * 1e-3) / 1e12,
                           "frac_of_fp32_mfma_peak": work / (ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS}
-    for ph in ("grafting", "apply"):
+    if acc["tridiagonal_ql"][0] > 0:
+        detail["tridiagonal_ql"] = {"ms_per_step": acc["tridiagonal_ql"][0] / args.steps}
+    for ph in ("grafting", "apply", "tridiagonalize"):
         ms, work, n = acc[ph]
         if ms > 0:
             detail[ph] = {"ms_per_step": ms / args.steps, "GB/s": work / (ms * 1e-3) / 1e9,

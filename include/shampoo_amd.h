@@ -212,6 +212,14 @@ double sa_phase_executed_flops(const char* phase); /* flops actually issued by "
  * No counterpart in the reference. */
 int32_t sa_set_symmetric_newton(int32_t policy);
 
+/* Solver behind sa_compute_root_inverses_eigh (stands in for torch.linalg.eigh, matrix_functions.py:233-366):
+ *   0  (default) by order: two-sided block Jacobi below 512, Householder tridiagonalisation + implicit QL
+ *      with batched rotation application from 512 up to 8192;
+ *   1  block Jacobi for every factor;
+ *   2  tridiagonalisation for every factor whose padded order is at least 256.
+ * Process wide.  No counterpart in the reference. */
+int32_t sa_set_eigh_solver(int32_t solver);
+
 #ifdef __cplusplus
 }
 #endif

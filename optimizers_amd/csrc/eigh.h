@@ -253,10 +253,11 @@ __global__ __launch_bounds__(256) void jacobi_rows_kernel(const JacobiFactor* __
 }
 
 // Eigenvalue post-processing of the reference's eigh root inverse, one workgroup per factor:
-// lambda = diag(A); if min(lambda) < eps: lambda <- (lambda - min) + eps (matrix_functions.py:256-264,
+// lambda as left by the solver; if min(lambda) < eps: lambda <- (lambda - min) + eps (matrix_functions.py:256-264,
 // two rounded additions); w = lambda^exponent.  Padded entries get weight 0.
 struct EigFinal {
-  const float* A;      // diagonalised matrix, dpad x dpad
+  const float* lambda_in;  // eigenvalue i at lambda_in[i * lambda_stride] (the diagonal of the diagonalised matrix, or a vector)
+  long long lambda_stride;
   const float* V;      // eigenvectors (columns)
   float* Vs;           // V with column c scaled by w[c]
   float* lambda_out;   // dpad floats
@@ -265,6 +266,7 @@ struct EigFinal {
   float exponent;      // -1 / root
   int row_begin;       // first global 8-row slab of this factor (eig_scale_cols_kernel)
   int enabled;
+  int scale_cols;      // eigenvectors are the columns of V: produce Vs (otherwise the caller scales rows)
 };
 
 // perturb_before != 0: epsilon was already added to the diagonal before the decomposition and the
@@ -276,7 +278,7 @@ __global__ __launch_bounds__(256) void eig_weights_kernel(const EigFinal* __rest
   if (!J.enabled) return;
   const int d = J.d, dpad = J.dpad;
   float m = 3.4028234663852886e38f;
-  for (int i = threadIdx.x; i < d; i += 256) m = fminf(m, J.A[(long long)i * dpad + i]);
+  for (int i = threadIdx.x; i < d; i += 256) m = fminf(m, J.lambda_in[i * J.lambda_stride]);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) m = fminf(m, __shfl_xor(m, o, 64));
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -288,7 +290,7 @@ __global__ __launch_bounds__(256) void eig_weights_kernel(const EigFinal* __rest
   for (int i = threadIdx.x; i < dpad; i += 256) {
     float lam = 0.0f, wgt = 0.0f;
     if (i < d) {
-      lam = J.A[(long long)i * dpad + i];
+      lam = J.lambda_in[i * J.lambda_stride];
       if (shift) {
         if (first != 0.0f) lam = lam + first;
         if (eps != 0.0f) lam = lam + eps;
@@ -308,7 +310,7 @@ __global__ __launch_bounds__(256) void eig_scale_cols_kernel(const EigFinal* __r
     if (jobs[mid].row_begin <= (int)blockIdx.x) lo = mid; else hi = mid - 1;
   }
   const EigFinal& J = jobs[lo];
-  if (!J.enabled) return;
+  if (!J.enabled || !J.scale_cols) return;
   const int dpad = J.dpad;
   const int r0 = (blockIdx.x - J.row_begin) * 8;
   for (int e = threadIdx.x * 4; e < 8 * dpad; e += 256 * 4) {

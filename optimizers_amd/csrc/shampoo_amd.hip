@@ -17,6 +17,7 @@
 #include "elementwise.h"
 #include "gemm.h"
 #include "qr.h"
+#include "tridiag.h"
 
 using namespace sa;
 
@@ -138,6 +139,16 @@ int launch_gemm(const GemmTable& g, GemmScalars sc, hipStream_t s) {
   HIPCHECK(hipGetLastError());
   return SA_OK;
 }
+template <int AL, int BL, int EPI, bool EDGE>
+int launch_gemm_raw(const GemmProblem* dev, int n, int total_tiles, GemmScalars sc, hipStream_t s) {
+  if (total_tiles == 0) return SA_OK;
+  const int per = (total_tiles + NUM_XCD - 1) / NUM_XCD;
+  hipLaunchKernelGGL((grouped_gemm_kernel<AL, BL, EPI, EDGE, false>), dim3(per * NUM_XCD), dim3(GEMM_THREADS), 0, s, dev, n,
+                     total_tiles, sc);
+  HIPCHECK(hipGetLastError());
+  return SA_OK;
+}
+
 template <int AL, int BL, int EPI>
 int launch_gemm_auto(const GemmTable& g, GemmScalars sc, hipStream_t s) {
   return g.aligned ? launch_gemm<AL, BL, EPI, false>(g, sc, s) : launch_gemm<AL, BL, EPI, true>(g, sc, s);
@@ -159,6 +170,8 @@ bool g_profiling = false;
 // converged within SYM_MAX_PREVIOUS_ITERATIONS (condition number <~ 1e4, where the two variants agree to
 // < 1e-4; measured deviation grows like 3e-9 x condition number for both).
 int g_symmetric_newton = 2;
+// eigh solver: 0 = by order (block Jacobi below TRD_MIN_DIM), 1 = always block Jacobi, 2 = tridiagonalisation wherever it fits
+int g_eigh_solver = 0;
 constexpr int SYM_MAX_PREVIOUS_ITERATIONS = 14;
 constexpr int SYM_REDO_ITERATIONS = 17;  // a symmetric solve that needed more is repeated with full products
 std::map<std::string, Phase> g_phases;
@@ -241,6 +254,12 @@ struct sa_plan {
   GemmTable ec_p1, ec_p1d, ec_p2, ec_p2d, ec_p3, ec_p3n, ec_p4, ec_p4n;  // eigenvalue-corrected preconditioning
   GemmTable qr_g[6], qr_aq, qr_b;
   Table<QrPanel> t_qrpanel;
+  Table<TrdJob> t_trd;
+  hipStream_t trd_stream = nullptr;  // applies QL rotations concurrently with the next chase
+  hipEvent_t trd_ev[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+  Table<GemmProblem> t_trd_gemm;
+  Table<RowScale> t_rowscale;
+  GemmTable eig_gemm_t;
   Table<Copy2D> t_copy;
   Table<NormPair> t_normpair;
   Table<SortJob> t_sort;
@@ -550,6 +569,11 @@ double sa_phase_executed_flops(const char* phase) {
   auto it = g_phases.find(phase ? phase : "");
   return it == g_phases.end() ? -1.0 : it->second.executed;
 }
+int32_t sa_set_eigh_solver(int32_t solver) {
+  g_eigh_solver = solver < 0 ? 0 : (solver > 2 ? 2 : solver);
+  return SA_OK;
+}
+
 int32_t sa_set_symmetric_newton(int32_t enabled) {
   g_symmetric_newton = enabled < 0 ? 0 : (enabled > 2 ? 2 : enabled);
   return SA_OK;
@@ -648,6 +672,9 @@ void sa_plan_destroy(sa_plan* p) {
   for (auto& row : p->nt_pow) for (auto& g : row) g.t.destroy();
   p->t_sym.destroy(); p->t_normjobs.destroy(); p->t_ids.destroy();
   p->t_jacobi.destroy(); p->t_sched.destroy(); p->t_eiginit.destroy(); p->t_eigfinal.destroy(); p->eig_gemm.t.destroy();
+  if (p->trd_stream) { (void)hipStreamSynchronize(p->trd_stream); (void)hipStreamDestroy(p->trd_stream); }
+  for (hipEvent_t e : p->trd_ev) if (e) (void)hipEventDestroy(e);
+  p->t_trd.destroy(); p->t_trd_gemm.destroy(); p->t_rowscale.destroy(); p->eig_gemm_t.t.destroy();
   for (GemmTable* g : {&p->ec_stat1, &p->ec_stat2, &p->ec_stat_l, &p->ec_stat_r, &p->ec_p1, &p->ec_p1d, &p->ec_p2, &p->ec_p2d,
                        &p->ec_p3, &p->ec_p3n, &p->ec_p4, &p->ec_p4n, &p->qr_aq, &p->qr_b})
     g->t.destroy();
@@ -1169,6 +1196,227 @@ int32_t sa_compute_root_inverses_newton(sa_plan* p, float bias_correction2, floa
 }
 
 // --------------------------------------------------------------------------------------------
+// Batched eigendecomposition through tridiagonalisation (orders >= TRD_MIN_DIM)
+// --------------------------------------------------------------------------------------------
+
+constexpr int TRD_MIN_DIM = 512;
+constexpr int TQL_MAX_ITER = 30;  // QL sweeps allowed per factor: TQL_MAX_ITER x order, as in LAPACK's steqr
+
+// layout of the small arrays inside a factor's M1 array (floats)
+inline long long trd_p_offset(const Factor&) { return 0; }                                   // P1, P2: 2 x dpad x 64
+inline long long trd_vec_offset(const Factor& f, int k) { return 2LL * f.dpad * TRD_PW + (long long)k * f.dpad; }
+inline long long trd_diag_offset(const Factor& f) { return trd_vec_offset(f, 2); }           // vbuf, ybuf, diag, off, tau
+inline long long trd_tmat_offset(const Factor& f) { return trd_vec_offset(f, 9); }           // dpad x 32 (after two fp64 vectors)
+inline long long trd_int_offset(const Factor& f) { return trd_tmat_offset(f) + (long long)f.dpad * TRD_NB; }
+
+static int trd_side_stream(sa_plan* p) {
+  if (p->trd_stream) return SA_OK;
+  HIPCHECK(hipStreamCreateWithFlags(&p->trd_stream, hipStreamNonBlocking));  // default priority
+  for (hipEvent_t& e : p->trd_ev) HIPCHECK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+  return SA_OK;
+}
+
+// Eigendecomposition of the dense matrices in the M0 arrays of `ids` (all of one order).  On return the rows of
+// the X0 array are the eigenvectors and trd_diag_offset() of the M1 array holds the eigenvalues.  X0 must hold
+// the identity on entry.  Uses X1 (Householder vectors), Mp1 (V T), S1, M1 and Mp0 as scratch.
+static int eigh_tridiagonal(sa_plan* p, const std::vector<int>& ids, hipStream_t s, int32_t* sweeps_out, int* not_converged) {
+  const int n = (int)ids.size();
+  if (n == 0) return SA_OK;
+  const int d = p->factors[ids[0]].d, dpad = p->factors[ids[0]].dpad;
+  const long long ld = dpad;
+  const int panels = (d - 1 + TRD_NB - 1) / TRD_NB;
+
+  SACHECK(p->t_trd.begin(n));
+  for (int k = 0; k < n; ++k) {
+    const Factor& f = p->factors[ids[k]];
+    TrdJob& J = p->t_trd.host[k];
+    std::memset(&J, 0, sizeof(J));
+    float* m1 = newton_buf(p, NB_M1, f);
+    J.A = newton_buf(p, NB_M0, f);
+    J.Y = newton_buf(p, NB_X0, f);
+    J.Vall = newton_buf(p, NB_X1, f);
+    J.P1 = m1 + trd_p_offset(f);
+    J.P2 = J.P1 + (long long)dpad * TRD_PW;
+    J.vbuf = m1 + trd_vec_offset(f, 0);
+    J.ybuf = m1 + trd_vec_offset(f, 1);
+    J.diag = m1 + trd_vec_offset(f, 2);
+    J.off = m1 + trd_vec_offset(f, 3);
+    J.tau = m1 + trd_vec_offset(f, 4);
+    J.qd = reinterpret_cast<double*>(m1 + trd_vec_offset(f, 5));
+    J.qe = reinterpret_cast<double*>(m1 + trd_vec_offset(f, 7));
+    J.Tmat = m1 + trd_tmat_offset(f);
+    J.hdr = reinterpret_cast<int*>(m1 + trd_int_offset(f));
+    J.state = J.hdr + 2 * TQL_HDR;
+    J.rot = reinterpret_cast<float2*>(newton_buf(p, NB_MP0, f));
+    J.d = d; J.dpad = dpad;
+    HIPCHECK(hipMemsetAsync(J.Vall, 0, sizeof(float) * ld * ld, s));
+    HIPCHECK(hipMemsetAsync(J.vbuf, 0, sizeof(float) * 5 * ld, s));
+  }
+  SACHECK(p->t_trd.upload(s));
+  const TrdJob* jobs = p->t_trd.dev;
+
+  // GEMM problem tables: [trailing update per panel | V T for every panel | G = (V T)^T Y per panel | Y -= V G per panel]
+  std::vector<GemmProblem> probs;
+  std::vector<int> trail_off(panels), trail_tiles(panels, 0), g1_off(panels), g1_tiles(panels, 0), g2_off(panels),
+      g2_tiles(panels, 0);
+  auto push = [&](const float* A, long long lda, const float* B, long long ldb, float* C, long long ldc, int M, int N, int K,
+                  int* tiles) {
+    GemmProblem q{};
+    q.A = A; q.lda = lda; q.a_vec = vec_ok(A, lda);
+    q.B = B; q.ldb = ldb; q.b_vec = vec_ok(B, ldb);
+    q.C = C; q.ldc = ldc; q.M = M; q.N = N; q.K = K;
+    q.tiles_m = (M + BM - 1) / BM;
+    q.tiles_n = (N + BN - 1) / BN;
+    q.tile_begin = *tiles;
+    *tiles += q.tiles_m * q.tiles_n;
+    probs.push_back(q);
+  };
+  for (int b = 0; b < panels; ++b) {
+    const int q0 = std::min(b * TRD_NB + TRD_NB, d - 1);  // first row / column after the panel
+    trail_off[b] = (int)probs.size();
+    if (d - q0 > 0)
+      for (int k = 0; k < n; ++k) {
+        const TrdJob& J = p->t_trd.host[k];
+        push(J.P1 + (long long)q0 * TRD_PW, TRD_PW, J.P2 + (long long)q0 * TRD_PW, TRD_PW, J.A + q0 * ld + q0, ld, d - q0, d - q0,
+             TRD_PW, &trail_tiles[b]);
+      }
+  }
+  const int vt_off = (int)probs.size();
+  int vt_tiles = 0;
+  for (int b = 0; b < panels; ++b)
+    for (int k = 0; k < n; ++k) {
+      const Factor& f = p->factors[ids[k]];
+      const TrdJob& J = p->t_trd.host[k];
+      const int p0 = b * TRD_NB;
+      float* VT = newton_buf(p, NB_MP1, f);
+      push(J.Vall + p0 * ld + p0, ld, J.Tmat + (long long)b * TRD_NB * TRD_NB, TRD_NB, VT + p0 * ld + p0, ld, d - p0, TRD_NB, TRD_NB,
+           &vt_tiles);
+    }
+  const int vt_count = (int)probs.size() - vt_off;
+  for (int b = 0; b < panels; ++b) {
+    const int p0 = b * TRD_NB;
+    g1_off[b] = (int)probs.size();
+    for (int k = 0; k < n; ++k) {
+      const Factor& f = p->factors[ids[k]];
+      const TrdJob& J = p->t_trd.host[k];
+      push(newton_buf(p, NB_MP1, f) + p0 * ld + p0, ld, J.Y + p0 * ld, ld, newton_buf(p, NB_S1, f), ld, TRD_NB, d, d - p0,
+           &g1_tiles[b]);
+    }
+    g2_off[b] = (int)probs.size();
+    for (int k = 0; k < n; ++k) {
+      const Factor& f = p->factors[ids[k]];
+      const TrdJob& J = p->t_trd.host[k];
+      push(J.Vall + p0 * ld + p0, ld, newton_buf(p, NB_S1, f), ld, J.Y + p0 * ld, ld, d - p0, d, TRD_NB, &g2_tiles[b]);
+    }
+  }
+  SACHECK(p->t_trd_gemm.begin(probs.size()));
+  std::memcpy(p->t_trd_gemm.host, probs.data(), probs.size() * sizeof(GemmProblem));
+  SACHECK(p->t_trd_gemm.upload(s));
+  const GemmProblem* gp = p->t_trd_gemm.dev;
+  const GemmScalars unit = unit_scalars();
+
+  // ---- 1. tridiagonalise
+  {
+    Span span("tridiagonalize", s, 4.0 / 3.0 * (double)d * d * d * n, 2 * d, true);  // bytes of the matrix-vector products
+    const size_t symv_lds = (size_t)dpad * sizeof(float);
+    for (int b = 0; b < panels; ++b) {
+      const int p0 = b * TRD_NB, kcols = std::min(TRD_NB, d - 1 - p0);
+      hipLaunchKernelGGL(trd_clear_panel_kernel, dim3(std::max(1, dpad / 32), n), dim3(256), 0, s, jobs);
+      for (int i = 0; i < kcols; ++i) {
+        const int j = p0 + i;
+        hipLaunchKernelGGL(trd_column_kernel, dim3(n), dim3(TRD_COL_THREADS), 0, s, jobs, j, p0, (i > 0 ? 1 : 0) | 2);
+        hipLaunchKernelGGL(trd_symv_kernel, dim3((d - j - 1 + TRD_SYMV_ROWS - 1) / TRD_SYMV_ROWS, n), dim3(256), symv_lds, s, jobs, j);
+      }
+      hipLaunchKernelGGL(trd_column_kernel, dim3(n), dim3(TRD_COL_THREADS), 0, s, jobs, p0 + kcols, p0, 1);
+      HIPCHECK(hipGetLastError());
+      SACHECK((launch_gemm_raw<A_MK, B_NK, EPI_SUB, true>(gp + trail_off[b], n, trail_tiles[b], unit, s)));
+    }
+    // last diagonal entry (a fresh, empty panel: no pending corrections)
+    hipLaunchKernelGGL(trd_column_kernel, dim3(n), dim3(TRD_COL_THREADS), 0, s, jobs, d - 1, d - 1, 2);
+    HIPCHECK(hipGetLastError());
+  }
+
+  // ---- 2. Y = Q1^T: Y <- (I - V_b T_b^T V_b^T) Y for b = 0 .. panels - 1
+  {
+    Span span("form_q", s, 4.0 * (double)d * d * d * n, 2 * panels + 2, true);
+    hipLaunchKernelGGL(trd_tfactor_kernel, dim3(panels, n), dim3(256), 0, s, jobs);
+    HIPCHECK(hipGetLastError());
+    SACHECK((launch_gemm_raw<A_MK, B_KN, EPI_STORE, true>(gp + vt_off, vt_count, vt_tiles, unit, s)));
+    for (int b = 0; b < panels; ++b) {
+      SACHECK((launch_gemm_raw<A_KM, B_KN, EPI_STORE, true>(gp + g1_off[b], n, g1_tiles[b], unit, s)));
+      SACHECK((launch_gemm_raw<A_MK, B_KN, EPI_SUB, true>(gp + g2_off[b], n, g2_tiles[b], unit, s)));
+    }
+  }
+
+  // ---- 3. implicit QL on T, rotations applied to the rows of Y chunk by chunk
+  {
+    Span span("tridiagonal_ql", s, 0.0, 0, true);
+    hipLaunchKernelGGL(tql_init_kernel, dim3(n), dim3(256), 0, s, jobs);
+    HIPCHECK(hipGetLastError());
+    const size_t ql_lds = 2 * (size_t)dpad * sizeof(double);
+    static bool attr_set = false;
+    if (!attr_set) {
+      HIPCHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(tql_sweeps_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   2 * TRD_MAX_DIM * (int)sizeof(double)));
+      attr_set = true;
+    }
+    const long long max_chunks = ((long long)TQL_MAX_ITER * d + TQL_K - 1) / TQL_K + 1;
+    int* h_state = p->h_pinned;
+    std::vector<int> state_host(8 * n);
+    bool all_done = false;
+    // The rotations of chunk c are applied on a second stream while lane 0 of every factor already chases
+    // chunk c + 1; the two log buffers alternate, guarded by events in both directions.
+    SACHECK(trd_side_stream(p));
+    hipStream_t s2 = getenv("SA_TRD_SERIAL") ? s : p->trd_stream;
+    HIPCHECK(hipEventRecord(p->trd_ev[4], s));
+    HIPCHECK(hipStreamWaitEvent(s2, p->trd_ev[4], 0));
+    long long launched = 0;
+    for (long long c = 0; c < max_chunks && !all_done; ++c) {
+      const int buf = (int)(c & 1);
+      if (c >= 2) HIPCHECK(hipStreamWaitEvent(s, p->trd_ev[2 + buf], 0));  // apply(c - 2) has released this buffer
+      hipLaunchKernelGGL(tql_sweeps_kernel, dim3(n), dim3(64), ql_lds, s, jobs, buf, TQL_MAX_ITER * d);
+      HIPCHECK(hipEventRecord(p->trd_ev[buf], s));
+      HIPCHECK(hipStreamWaitEvent(s2, p->trd_ev[buf], 0));
+      hipLaunchKernelGGL(tql_apply_kernel, dim3((d + 255) / 256, n), dim3(256), 0, s2, jobs, buf);
+      HIPCHECK(hipEventRecord(p->trd_ev[2 + buf], s2));
+      HIPCHECK(hipGetLastError());
+      ++launched;
+      if ((c & 7) == 7) {
+        for (int k = 0; k < n; ++k)
+          HIPCHECK(hipMemcpyAsync(state_host.data() + 8 * k, p->t_trd.host[k].state, 6 * sizeof(int), hipMemcpyDeviceToHost, s));
+        HIPCHECK(hipStreamSynchronize(s));
+        all_done = true;
+        for (int k = 0; k < n; ++k)
+          if (!state_host[8 * k + 2] && !state_host[8 * k + 3]) all_done = false;
+      }
+    }
+    // join: everything later on s sees the finished Y
+    if (launched >= 1) HIPCHECK(hipStreamWaitEvent(s, p->trd_ev[2 + (int)((launched - 1) & 1)], 0));
+    if (launched >= 2) HIPCHECK(hipStreamWaitEvent(s, p->trd_ev[2 + (int)((launched - 2) & 1)], 0));
+    (void)h_state;
+    for (int k = 0; k < n; ++k)
+      HIPCHECK(hipMemcpyAsync(state_host.data() + 8 * k, p->t_trd.host[k].state, 6 * sizeof(int), hipMemcpyDeviceToHost, s));
+    HIPCHECK(hipStreamSynchronize(s));
+    for (int k = 0; k < n; ++k) {
+      sweeps_out[ids[k]] = state_host[8 * k + 4];
+      not_converged[ids[k]] = (state_host[8 * k + 2] && !state_host[8 * k + 3]) ? 0 : 1;
+      if (getenv("SA_DEBUG_TRD") && state_host[8 * k + 3] && k < 2) {
+        std::vector<float> dv(2 * d);
+        HIPCHECK(hipMemcpy(dv.data(), p->t_trd.host[k].diag, d * sizeof(float), hipMemcpyDeviceToHost));
+        HIPCHECK(hipMemcpy(dv.data() + d, p->t_trd.host[k].off, d * sizeof(float), hipMemcpyDeviceToHost));
+        char name[128];
+        snprintf(name, sizeof(name), "gpurun_out/trd_fail_%d.bin", k);
+        if (FILE* fp = fopen(name, "wb")) { fwrite(dv.data(), sizeof(float), dv.size(), fp); fclose(fp); }
+      }
+      if (getenv("SA_DEBUG_TRD")) fprintf(stderr, "trd factor %d: l=%d iter=%d done=%d failed=%d sweeps=%d scale=%g\n", ids[k], state_host[8*k], state_host[8*k+1], state_host[8*k+2], state_host[8*k+3], state_host[8*k+4], *reinterpret_cast<float*>(&state_host[8*k+5]));
+    }
+    hipLaunchKernelGGL(tql_finish_kernel, dim3(n), dim3(256), 0, s, jobs);
+    HIPCHECK(hipGetLastError());
+  }
+  return SA_OK;
+}
+
+// --------------------------------------------------------------------------------------------
 // Batched eigendecomposition root inverse (block Jacobi)
 // --------------------------------------------------------------------------------------------
 
@@ -1221,96 +1469,120 @@ int32_t sa_compute_root_inverses_eigh(sa_plan* p, float bias_correction2, float 
   hipLaunchKernelGGL(eig_init_kernel, dim3(tiles), dim3(256), 0, s, p->t_eiginit.dev, n, bias_correction2, ridge);
   HIPCHECK(hipGetLastError());
 
-  // tournament schedules, one per distinct block count
-  std::map<int, size_t> sched_off;
-  std::vector<int2> sched;
-  int max_nb = 0, max_dpad = 0;
-  for (int i = 0; i < n; ++i) {
-    const int nb = p->factors[todo[i]].dpad / JB;
-    max_nb = std::max(max_nb, nb);
-    max_dpad = std::max(max_dpad, p->factors[todo[i]].dpad);
-    if (sched_off.count(nb)) continue;
-    sched_off[nb] = sched.size();
-    const int m = nb - 1;
-    for (int r = 0; r < nb - 1; ++r)
-      for (int k = 0; k < nb / 2; ++k) {
-        int a, b;
-        if (k == 0) { a = 0; b = (r % m) + 1; }
-        else { a = ((r + k) % m) + 1; b = ((r - k + m) % m) + 1; }
-        sched.push_back(make_int2(std::min(a, b), std::max(a, b)));
-      }
+  // solver per factor: block Jacobi for small orders, tridiagonalisation + QL for the rest
+  std::vector<int> jac, jac_pos;            // factor ids / positions in todo
+  std::map<int, std::vector<int>> trd_by_d; // order -> factor ids
+  for (int k = 0; k < n; ++k) {
+    const Factor& f = p->factors[todo[k]];
+    if (g_eigh_solver != 1 && (g_eigh_solver == 2 || f.d >= TRD_MIN_DIM) && f.dpad >= 256 && f.d <= TRD_MAX_DIM)
+      trd_by_d[f.d].push_back(todo[k]);
+    else { jac.push_back(todo[k]); jac_pos.push_back(k); }
   }
-  SACHECK(p->t_sched.begin(sched.size()));
-  std::memcpy(p->t_sched.host, sched.data(), sched.size() * sizeof(int2));
-  SACHECK(p->t_sched.upload(s));
-  SACHECK(p->t_jacobi.begin(n));
-  int pairs = 0;
-  for (int i = 0; i < n; ++i) {
-    const Factor& f = p->factors[todo[i]];
-    JacobiFactor& J = p->t_jacobi.host[i];
-    std::memset(&J, 0, sizeof(J));
-    J.A = newton_buf(p, NB_M0, f);
-    J.V = newton_buf(p, NB_X0, f);
-    J.U = newton_buf(p, NB_S2, f);
-    J.nb = f.dpad / JB;
-    J.sched = p->t_sched.dev + sched_off[J.nb];
-    J.rotations = p->d_iters + todo[i];
-    J.rot_mass = p->d_final_err + todo[i];
-    J.active = p->d_active + todo[i];
-    J.thr_abs = 1e-9f * fro[i];
-    J.thr_diag = 2.4e-7f * fro[i];  // 2^-22 ||A||_F: below the eigenvalue resolution of an fp32 matrix
-    J.d = f.d; J.dpad = f.dpad;
-    J.pair_begin = pairs;
-    pairs += J.nb / 2;
-  }
-  SACHECK(p->t_jacobi.upload(s));
   std::vector<int> active(F, 0);
-  for (int i : todo) active[i] = 1;
-  HIPCHECK(hipMemcpyAsync(p->d_active, active.data(), F * sizeof(int), hipMemcpyHostToDevice, s));
-  HIPCHECK(hipStreamSynchronize(s));
+  std::vector<char> via_trd(F, 0);
 
-  int live = n;
-  for (int sweep = 0; sweep < max_sweeps && live > 0; ++sweep) {
-    HIPCHECK(hipMemsetAsync(p->d_iters, 0, F * sizeof(int), s));
-    HIPCHECK(hipMemsetAsync(p->d_final_err, 0, F * sizeof(float), s));
-    double work = 0.0;
-    for (int i = 0; i < n; ++i)
-      if (active[todo[i]]) { const double d = p->factors[todo[i]].dpad; work += 3.0 * 2.0 * d * d * JP * (d / JB - 1); }
-    {
-      Span span("jacobi", s, work, 3 * (max_nb - 1), sweep == 0);
-      for (int r = 0; r < max_nb - 1; ++r) {
-        hipLaunchKernelGGL(jacobi_pivot_kernel, dim3(pairs), dim3(256), 0, s, p->t_jacobi.dev, n, r);
-        hipLaunchKernelGGL(jacobi_cols_kernel, dim3(pairs, max_dpad / 128, 2), dim3(256), 0, s, p->t_jacobi.dev, n, r);
-        hipLaunchKernelGGL(jacobi_rows_kernel, dim3(pairs, max_dpad / 128, 1), dim3(256), 0, s, p->t_jacobi.dev, n, r);
-      }
-      HIPCHECK(hipGetLastError());
+  if (!jac.empty()) {
+    const int nj = (int)jac.size();
+    // tournament schedules, one per distinct block count
+    std::map<int, size_t> sched_off;
+    std::vector<int2> sched;
+    int max_nb = 0, max_dpad = 0;
+    for (int i = 0; i < nj; ++i) {
+      const int nb = p->factors[jac[i]].dpad / JB;
+      max_nb = std::max(max_nb, nb);
+      max_dpad = std::max(max_dpad, p->factors[jac[i]].dpad);
+      if (sched_off.count(nb)) continue;
+      sched_off[nb] = sched.size();
+      const int m = nb - 1;
+      for (int r = 0; r < nb - 1; ++r)
+        for (int k = 0; k < nb / 2; ++k) {
+          int a, b;
+          if (k == 0) { a = 0; b = (r % m) + 1; }
+          else { a = ((r + k) % m) + 1; b = ((r - k + m) % m) + 1; }
+          sched.push_back(make_int2(std::min(a, b), std::max(a, b)));
+        }
     }
-    HIPCHECK(hipMemcpyAsync(p->h_pinned, p->d_iters, F * sizeof(int), hipMemcpyDeviceToHost, s));
-    HIPCHECK(hipMemcpyAsync(p->h_pinned + F, p->d_final_err, F * sizeof(float), hipMemcpyDeviceToHost, s));
-    HIPCHECK(hipStreamSynchronize(s));
-    live = 0;
-    const float* mass = reinterpret_cast<const float*>(p->h_pinned + F);
-    for (int k = 0; k < n; ++k) {
-      const int i = todo[k];
-      if (!active[i]) continue;
-      sweeps_out[i] = sweep + 1;
-      // converged when the sweep removed less than (5e-7 ||A||_F)^2 of off-diagonal mass
-      const double tol = 5e-7 * (double)fro[k];
-      if (p->h_pinned[i] == 0 || (double)mass[i] < tol * tol) active[i] = 0; else ++live;
+    SACHECK(p->t_sched.begin(sched.size()));
+    std::memcpy(p->t_sched.host, sched.data(), sched.size() * sizeof(int2));
+    SACHECK(p->t_sched.upload(s));
+    SACHECK(p->t_jacobi.begin(nj));
+    int pairs = 0;
+    for (int i = 0; i < nj; ++i) {
+      const Factor& f = p->factors[jac[i]];
+      JacobiFactor& J = p->t_jacobi.host[i];
+      std::memset(&J, 0, sizeof(J));
+      J.A = newton_buf(p, NB_M0, f);
+      J.V = newton_buf(p, NB_X0, f);
+      J.U = newton_buf(p, NB_S2, f);
+      J.nb = f.dpad / JB;
+      J.sched = p->t_sched.dev + sched_off[J.nb];
+      J.rotations = p->d_iters + jac[i];
+      J.rot_mass = p->d_final_err + jac[i];
+      J.active = p->d_active + jac[i];
+      J.thr_abs = 1e-9f * fro[jac_pos[i]];
+      J.thr_diag = 2.4e-7f * fro[jac_pos[i]];  // 2^-22 ||A||_F: below the eigenvalue resolution of an fp32 matrix
+      J.d = f.d; J.dpad = f.dpad;
+      J.pair_begin = pairs;
+      pairs += J.nb / 2;
     }
+    SACHECK(p->t_jacobi.upload(s));
+    for (int i : jac) active[i] = 1;
     HIPCHECK(hipMemcpyAsync(p->d_active, active.data(), F * sizeof(int), hipMemcpyHostToDevice, s));
     HIPCHECK(hipStreamSynchronize(s));
+
+    int live = nj;
+    for (int sweep = 0; sweep < max_sweeps && live > 0; ++sweep) {
+      HIPCHECK(hipMemsetAsync(p->d_iters, 0, F * sizeof(int), s));
+      HIPCHECK(hipMemsetAsync(p->d_final_err, 0, F * sizeof(float), s));
+      double work = 0.0;
+      for (int i = 0; i < nj; ++i)
+        if (active[jac[i]]) { const double d = p->factors[jac[i]].dpad; work += 3.0 * 2.0 * d * d * JP * (d / JB - 1); }
+      {
+        Span span("jacobi", s, work, 3 * (max_nb - 1), sweep == 0);
+        for (int r = 0; r < max_nb - 1; ++r) {
+          hipLaunchKernelGGL(jacobi_pivot_kernel, dim3(pairs), dim3(256), 0, s, p->t_jacobi.dev, nj, r);
+          hipLaunchKernelGGL(jacobi_cols_kernel, dim3(pairs, max_dpad / 128, 2), dim3(256), 0, s, p->t_jacobi.dev, nj, r);
+          hipLaunchKernelGGL(jacobi_rows_kernel, dim3(pairs, max_dpad / 128, 1), dim3(256), 0, s, p->t_jacobi.dev, nj, r);
+        }
+        HIPCHECK(hipGetLastError());
+      }
+      HIPCHECK(hipMemcpyAsync(p->h_pinned, p->d_iters, F * sizeof(int), hipMemcpyDeviceToHost, s));
+      HIPCHECK(hipMemcpyAsync(p->h_pinned + F, p->d_final_err, F * sizeof(float), hipMemcpyDeviceToHost, s));
+      HIPCHECK(hipStreamSynchronize(s));
+      live = 0;
+      const float* mass = reinterpret_cast<const float*>(p->h_pinned + F);
+      for (int k = 0; k < nj; ++k) {
+        const int i = jac[k];
+        if (!active[i]) continue;
+        sweeps_out[i] = sweep + 1;
+        // converged when the sweep removed less than (5e-7 ||A||_F)^2 of off-diagonal mass
+        const double tol = 5e-7 * (double)fro[jac_pos[k]];
+        if (p->h_pinned[i] == 0 || (double)mass[i] < tol * tol) active[i] = 0; else ++live;
+      }
+      HIPCHECK(hipMemcpyAsync(p->d_active, active.data(), F * sizeof(int), hipMemcpyHostToDevice, s));
+      HIPCHECK(hipStreamSynchronize(s));
+    }
+  }
+  for (auto& kv : trd_by_d) {
+    SACHECK(eigh_tridiagonal(p, kv.second, s, sweeps_out, active.data()));
+    for (int i : kv.second) via_trd[i] = 1;
   }
 
   // X = V diag(f(lambda)) V^T
   SACHECK(p->t_eigfinal.begin(n));
+  SACHECK(p->t_rowscale.begin(n));
   p->eig_gemm.clear();
-  int slabs = 0;
+  p->eig_gemm_t.clear();
+  int slabs = 0, slabs_t = 0, n_t = 0;
   for (int i = 0; i < n; ++i) {
     const Factor& f = p->factors[todo[i]];
     EigFinal& J = p->t_eigfinal.host[i];
     std::memset(&J, 0, sizeof(J));
-    J.A = newton_buf(p, NB_M0, f);
+    const bool t = via_trd[todo[i]] != 0;
+    // Jacobi leaves the eigenvalues on the diagonal of A and the eigenvectors in the columns of V;
+    // the tridiagonal path leaves them in a vector (start of the Mp1 array) and in the rows of V
+    J.lambda_in = t ? newton_buf(p, NB_M1, f) + trd_diag_offset(f) : newton_buf(p, NB_M0, f);
+    J.lambda_stride = t ? 1 : (long long)f.dpad + 1;
     J.V = newton_buf(p, NB_X0, f);
     J.Vs = newton_buf(p, NB_S1, f);
     J.lambda_out = newton_buf(p, NB_MP0, f);
@@ -1319,20 +1591,33 @@ int32_t sa_compute_root_inverses_eigh(sa_plan* p, float bias_correction2, float 
     J.exponent = -1.0f / roots[todo[i]];
     J.row_begin = slabs;
     J.enabled = 1;
-    slabs += f.dpad / 8;
+    J.scale_cols = t ? 0 : 1;
     GemmProblem q{};
-    q.A = J.Vs; q.B = J.V; q.C = newton_buf(p, NB_X1, f);
+    q.A = t ? J.V : J.Vs; q.B = t ? J.Vs : J.V; q.C = newton_buf(p, NB_X1, f);
     q.lda = q.ldb = q.ldc = f.dpad;
     q.M = q.N = q.K = f.dpad;
     q.a_vec = q.b_vec = 1;
-    p->eig_gemm.add(q, false);
+    if (t) {
+      RowScale& R = p->t_rowscale.host[n_t++];
+      R.Y = J.V; R.Ys = J.Vs; R.w = J.weight_out; R.dpad = f.dpad; R.row_begin = slabs_t;
+      slabs_t += f.dpad / 8;
+      p->eig_gemm_t.add(q, false);
+    } else {
+      p->eig_gemm.add(q, false);
+    }
+    slabs += f.dpad / 8;
   }
+  p->t_rowscale.n = n_t;
   SACHECK(p->t_eigfinal.upload(s));
+  SACHECK(p->t_rowscale.upload(s));
   SACHECK(p->eig_gemm.commit(s));
+  SACHECK(p->eig_gemm_t.commit(s));
   hipLaunchKernelGGL(eig_weights_kernel, dim3(n), dim3(256), 0, s, p->t_eigfinal.dev, epsilon, perturb_before_computation ? 1 : 0);
   hipLaunchKernelGGL(eig_scale_cols_kernel, dim3(slabs), dim3(256), 0, s, p->t_eigfinal.dev, n);
+  if (n_t) hipLaunchKernelGGL(eig_scale_rows_kernel, dim3(slabs_t), dim3(256), 0, s, p->t_rowscale.dev, n_t);
   HIPCHECK(hipGetLastError());
-  SACHECK((launch_gemm<A_MK, B_NK, EPI_STORE, false, false>(p->eig_gemm, unit_scalars(), s)));
+  SACHECK((launch_gemm<A_MK, B_NK, EPI_STORE, false, false>(p->eig_gemm, unit_scalars(), s)));    // (V w) V^T
+  SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, false, false>(p->eig_gemm_t, unit_scalars(), s)));  // Y^T (w Y)
 
   std::vector<const float*> X(n);
   for (int i = 0; i < n; ++i) X[i] = newton_buf(p, NB_X1, p->factors[todo[i]]);

@@ -1,0 +1,543 @@
+// Batched symmetric eigendecomposition through tridiagonalisation, for factors too large for the
+// block-Jacobi solver to be competitive.
+//
+//   1. A = Q1 T Q1^T: blocked Householder tridiagonalisation (LAPACK sytrd/latrd recurrences).  Per column
+//      one single-workgroup kernel per factor (pending panel corrections, Householder vector, the w vector
+//      of the previous column) and one symmetric matrix-vector product over the trailing matrix, which is
+//      the HBM-bound part ((4/3) d^3 bytes per factor); per 32-column panel one rank-64 trailing update
+//      A -= [V W] [W V]^T on the grouped MFMA GEMM.
+//   2. Y = Q1^T by compact-WY block reflectors (grouped GEMMs).
+//   3. T = Z diag(lambda) Z^T by implicit QL iteration with Wilkinson shifts.  One lane per factor runs the
+//      sequential bulge chase and logs the rotations of up to TQL_K sweeps; a second kernel applies that
+//      chunk of sweeps to the rows of Y as a register-resident systolic pipeline (one thread per column of
+//      Y, one carried row per sweep), so Y is read and written once per chunk instead of once per sweep.
+// On exit row i of Y is the eigenvector of eigenvalue diag[i] (not sorted).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "gemm.h"
+
+namespace sa {
+
+typedef float vfloat4_t __attribute__((ext_vector_type(4)));
+typedef float vfloat2_t __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(1))) vfloat2_t global_float2;
+
+
+
+constexpr int TRD_NB = 32;               // panel width
+constexpr int TRD_PW = 2 * TRD_NB;       // row length of the [V | W] and [W | V] panel buffers
+constexpr int TRD_COL_THREADS = 1024;
+constexpr int TRD_ROWS_PER_THREAD = 8;   // d <= 8192
+constexpr int TRD_MAX_DIM = TRD_COL_THREADS * TRD_ROWS_PER_THREAD;
+constexpr int TRD_SYMV_ROWS = 16;
+constexpr int TQL_K = 32;                // sweeps per chunk
+constexpr int TQL_STEPS = 64;            // pipeline steps whose coefficients are staged in LDS at a time
+constexpr int TQL_HDR = 4 + 2 * TQL_K;   // ints per chunk header: nsweeps, top, bot, -, l[K], m[K]
+
+struct TrdJob {
+  float* A;       // dpad x dpad, symmetric, both triangles kept current
+  float* Y;       // dpad x dpad
+  float* Vall;    // dpad x dpad, column j = Householder vector of column j (explicit unit entry, zeros above)
+  float* P1;      // dpad x 64: [V | W] of the current panel
+  float* P2;      // dpad x 64: [W | V]
+  float* vbuf;    // dpad: current Householder vector, zero at and above the diagonal
+  float* ybuf;    // dpad: trailing matrix times vbuf
+  float* diag;    // dpad
+  float* off;     // dpad: off[j] couples j and j + 1
+  float* tau;     // dpad
+  double* qd;     // dpad: diagonal of the (unit-scaled) tridiagonal matrix during the QL iteration
+  double* qe;     // dpad: its off-diagonal
+  float* Tmat;    // (dpad / 32) x 32 x 32 triangular factors of the block reflectors
+  float2* rot;    // 2 x TQL_K x dpad rotation log (c, s)
+  int* hdr;       // 2 x TQL_HDR
+  int* state;     // l, iterations of the current eigenvalue, done, failed, total sweeps, bits of the scale
+  int d, dpad;
+};
+
+__device__ __forceinline__ float block_sum_1024(float v, float* red) {
+  v = wave_sum(v);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float t = 0.f;
+#pragma unroll
+  for (int k = 0; k < TRD_COL_THREADS / 64; ++k) t += red[k];
+  return t;
+}
+
+// P1 and P2 are adjacent: 2 * dpad * 64 floats
+__global__ __launch_bounds__(256) void trd_clear_panel_kernel(const TrdJob* __restrict__ jobs) {
+  const TrdJob& J = jobs[blockIdx.y];
+  const long long n4 = (long long)J.dpad * TRD_PW * 2 / 4;
+  float4* dst = reinterpret_cast<float4*>(J.P1);
+  for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < n4; e += (long long)gridDim.x * 256)
+    dst[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
+// sum over q of V[r][q] * cw[q] + W[r][q] * cv[q] for one row of the [V | W] buffer
+__device__ __forceinline__ float panel_row_dot(const float* __restrict__ row, const float* cv, const float* cw) {
+  float acc = 0.f;
+#pragma unroll
+  for (int q4 = 0; q4 < TRD_NB / 4; ++q4) {
+    const float4 v = *reinterpret_cast<const float4*>(row + 4 * q4);
+    const float4 w = *reinterpret_cast<const float4*>(row + TRD_NB + 4 * q4);
+    acc += v.x * cw[4 * q4] + v.y * cw[4 * q4 + 1] + v.z * cw[4 * q4 + 2] + v.w * cw[4 * q4 + 3];
+    acc += w.x * cv[4 * q4] + w.y * cv[4 * q4 + 1] + w.z * cv[4 * q4 + 2] + w.w * cv[4 * q4 + 3];
+  }
+  return acc;
+}
+
+// flags bit 0: finish w of column j - 1 (needs ybuf of that column); bit 1: start column j.
+// Panel columns are p0 .. p0 + 31; i = j - p0 columns of the panel are already in P1 / P2.
+__global__ __launch_bounds__(TRD_COL_THREADS) void trd_column_kernel(const TrdJob* __restrict__ jobs, int j, int p0,
+                                                                    int flags) {
+  __shared__ float part1[32][33];
+  __shared__ float part2[32][33];
+  __shared__ float t1[TRD_NB], t2[TRD_NB], rowV[TRD_NB], rowW[TRD_NB];
+  __shared__ float red[TRD_COL_THREADS / 64];
+  __shared__ float bc[2];
+  const TrdJob& J = jobs[blockIdx.x];
+  const int d = J.d;
+  if (j >= d) return;
+  const int tid = threadIdx.x;
+  const long long ld = J.dpad;
+  float* __restrict__ P1 = J.P1;
+  float* __restrict__ P2 = J.P2;
+
+  if (flags & 1) {
+    const int jp = j - 1, ip = jp - p0;
+    const float tau = J.tau[jp];
+    {  // t1 = W^T v, t2 = V^T v over the first ip panel columns
+      const int q = tid & 31, g = tid >> 5;
+      float a1 = 0.f, a2 = 0.f;
+      if (q < ip)
+        for (int r = jp + 1 + g; r < d; r += 32) {
+          const float vr = J.vbuf[r];
+          a1 += P1[(long long)r * TRD_PW + TRD_NB + q] * vr;
+          a2 += P1[(long long)r * TRD_PW + q] * vr;
+        }
+      part1[g][q] = a1;
+      part2[g][q] = a2;
+    }
+    __syncthreads();
+    if (tid < TRD_NB) {
+      float s1 = 0.f, s2 = 0.f;
+      for (int k = 0; k < 32; ++k) { s1 += part1[k][tid]; s2 += part2[k][tid]; }
+      t1[tid] = s1;
+      t2[tid] = s2;
+    }
+    __syncthreads();
+    float wreg[TRD_ROWS_PER_THREAD];
+    float dot = 0.f;
+#pragma unroll
+    for (int k = 0; k < TRD_ROWS_PER_THREAD; ++k) {
+      const int r = jp + 1 + tid + k * TRD_COL_THREADS;
+      float w = 0.f;
+      if (r < d) {
+        // w = tau (y - V (W^T v) - W (V^T v))
+        w = tau * (J.ybuf[r] - panel_row_dot(P1 + (long long)r * TRD_PW, t2, t1));
+        dot += w * J.vbuf[r];
+      }
+      wreg[k] = w;
+    }
+    const float alpha = -0.5f * tau * block_sum_1024(dot, red);
+#pragma unroll
+    for (int k = 0; k < TRD_ROWS_PER_THREAD; ++k) {
+      const int r = jp + 1 + tid + k * TRD_COL_THREADS;
+      if (r < d) {
+        const float w = wreg[k] + alpha * J.vbuf[r];
+        P1[(long long)r * TRD_PW + TRD_NB + ip] = w;
+        P2[(long long)r * TRD_PW + ip] = w;
+      }
+    }
+    __threadfence_block();
+    __syncthreads();
+  }
+
+  if (flags & 2) {
+    const int i = j - p0;
+    if (tid < TRD_NB) {
+      rowV[tid] = (tid < i) ? P1[(long long)j * TRD_PW + tid] : 0.f;
+      rowW[tid] = (tid < i) ? P1[(long long)j * TRD_PW + TRD_NB + tid] : 0.f;
+    }
+    __syncthreads();
+    float areg[TRD_ROWS_PER_THREAD];
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < TRD_ROWS_PER_THREAD; ++k) {
+      const int r = j + tid + k * TRD_COL_THREADS;
+      float a = 0.f;
+      if (r < d) {
+        // column j of the matrix as it stands after the i reflectors of this panel (row j is the same by symmetry)
+        a = J.A[(long long)j * ld + r];
+        if (i > 0) a -= panel_row_dot(P1 + (long long)r * TRD_PW, rowV, rowW);
+        if (r > j + 1) ss += a * a;
+      }
+      areg[k] = a;
+    }
+    const float sigma2 = block_sum_1024(ss, red);
+    if (tid == 0) bc[0] = areg[0];
+    if (tid == 1) bc[1] = areg[0];
+    __syncthreads();
+    const float ajj = bc[0];
+    const float alpha0 = (j + 1 < d) ? bc[1] : 0.f;
+    float tau = 0.f, beta = alpha0, scale = 0.f;
+    if (sigma2 != 0.f) {  // LAPACK slarfg
+      beta = -copysignf(sqrtf(alpha0 * alpha0 + sigma2), alpha0);
+      tau = (beta - alpha0) / beta;
+      scale = 1.0f / (alpha0 - beta);
+    }
+    if (tid == 0) {
+      J.diag[j] = ajj;
+      if (j + 1 < d) { J.off[j] = beta; J.tau[j] = tau; }
+    }
+    if (tid < 4 && j - tid >= 0) J.vbuf[j - tid] = 0.f;  // the product kernel starts at a 16-byte boundary
+#pragma unroll
+    for (int k = 0; k < TRD_ROWS_PER_THREAD; ++k) {
+      const int r = j + tid + k * TRD_COL_THREADS;
+      if (r < d && r > j) {
+        const float v = (r == j + 1) ? 1.0f : areg[k] * scale;
+        J.vbuf[r] = v;
+        P1[(long long)r * TRD_PW + i] = v;
+        P2[(long long)r * TRD_PW + TRD_NB + i] = v;
+        J.Vall[(long long)r * ld + j] = v;
+      }
+    }
+  }
+}
+
+// ybuf[r] = sum_c A[r][c] vbuf[c] over r, c in (j, d).  Dynamic LDS: dpad floats.
+__global__ __launch_bounds__(256) void trd_symv_kernel(const TrdJob* __restrict__ jobs, int j) {
+  extern __shared__ float vs[];
+  const TrdJob& J = jobs[blockIdx.y];
+  const int d = J.d;
+  const int r0 = j + 1 + blockIdx.x * TRD_SYMV_ROWS;
+  if (r0 >= d) return;
+  const int c0 = (j + 1) & ~3, cend = (d + 3) & ~3;
+  for (int c = c0 + threadIdx.x * 4; c < cend; c += 1024)
+    *reinterpret_cast<float4*>(vs + (c - c0)) = *reinterpret_cast<const float4*>(J.vbuf + c);
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const long long ld = J.dpad;
+  const int rbase = r0 + wave * 4;
+  const float* __restrict__ rows[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) rows[k] = J.A + (long long)min(rbase + k, d - 1) * ld;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int c = c0 + lane * 4; c < cend; c += 256) {
+    const float4 v = *reinterpret_cast<const float4*>(vs + (c - c0));
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const vfloat4_t a = __builtin_nontemporal_load(reinterpret_cast<const vfloat4_t*>(rows[k] + c));
+      acc[k] += (a.x * v.x + a.y * v.y) + (a.z * v.z + a.w * v.w);
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const float t = wave_sum(acc[k]);
+    if (lane == 0 && rbase + k < d) J.ybuf[rbase + k] = t;
+  }
+}
+
+// Triangular factor T of the block reflector of panel blockIdx.x (LAPACK slarft, forward, columnwise):
+// H_p0 ... H_p0+k-1 = I - V T V^T.  grid (panels, factors).
+__global__ __launch_bounds__(256) void trd_tfactor_kernel(const TrdJob* __restrict__ jobs) {
+  __shared__ float Vs[64][TRD_NB + 1];
+  __shared__ float S[TRD_NB][TRD_NB + 1];
+  __shared__ float Tm[TRD_NB][TRD_NB + 1];
+  __shared__ float taus[TRD_NB];
+  const TrdJob& J = jobs[blockIdx.y];
+  const int d = J.d, p0 = blockIdx.x * TRD_NB;
+  if (p0 >= d - 1) return;
+  const int kcols = min(TRD_NB, d - 1 - p0);
+  const int tid = threadIdx.x;
+  const long long ld = J.dpad;
+  const int i = tid >> 3, k0 = (tid & 7) * 4;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int rb = p0 + 1; rb < d; rb += 64) {
+    for (int e = tid; e < 64 * TRD_NB; e += 256) {
+      const int rr = e >> 5, c = e & 31, r = rb + rr;
+      Vs[rr][c] = (r < d) ? J.Vall[(long long)r * ld + p0 + c] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int rr = 0; rr < 64; ++rr) {
+      const float vi = Vs[rr][i];
+#pragma unroll
+      for (int m = 0; m < 4; ++m) acc[m] += vi * Vs[rr][k0 + m];
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int m = 0; m < 4; ++m) S[i][k0 + m] = acc[m];
+  if (tid < TRD_NB) taus[tid] = (tid < kcols) ? J.tau[p0 + tid] : 0.f;
+  for (int e = tid; e < TRD_NB * TRD_NB; e += 256) Tm[e >> 5][e & 31] = 0.f;
+  __syncthreads();
+  for (int c = 0; c < TRD_NB; ++c) {
+    if (tid < c) {
+      float a = 0.f;
+      for (int m = tid; m < c; ++m) a += Tm[tid][m] * S[m][c];
+      Tm[tid][c] = -taus[c] * a;
+    }
+    if (tid == c) Tm[c][c] = taus[c];
+    __syncthreads();
+  }
+  float* out = J.Tmat + (long long)blockIdx.x * TRD_NB * TRD_NB;
+  for (int e = tid; e < TRD_NB * TRD_NB; e += 256) out[e] = Tm[e >> 5][e & 31];
+}
+
+// Scale T to unit maximum entry and reset the QL state.  One workgroup per factor.
+__global__ __launch_bounds__(256) void tql_init_kernel(const TrdJob* __restrict__ jobs) {
+  __shared__ float red[4];
+  const TrdJob& J = jobs[blockIdx.x];
+  const int d = J.d;
+  float m = 0.f;
+  for (int i = threadIdx.x; i < d; i += 256) {
+    m = fmaxf(m, fabsf(J.diag[i]));
+    if (i < d - 1) m = fmaxf(m, fabsf(J.off[i]));
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+  __syncthreads();
+  const float tn = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  const double inv = (tn > 0.f) ? 1.0 / (double)tn : 1.0;
+  for (int i = threadIdx.x; i < d; i += 256) {
+    J.qd[i] = (double)J.diag[i] * inv;
+    J.qe[i] = (i < d - 1) ? (double)J.off[i] * inv : 0.0;
+  }
+  if (threadIdx.x == 0) {
+    J.state[0] = 0; J.state[1] = 0; J.state[2] = 0; J.state[3] = 0; J.state[4] = 0;
+    J.state[5] = __float_as_int((tn > 0.f) ? tn : 1.0f);
+    J.hdr[0] = 0;
+    J.hdr[TQL_HDR] = 0;
+  }
+}
+
+__global__ __launch_bounds__(256) void tql_finish_kernel(const TrdJob* __restrict__ jobs) {
+  const TrdJob& J = jobs[blockIdx.x];
+  const float tn = __int_as_float(J.state[5]);
+  for (int i = threadIdx.x; i < J.d; i += 256) J.diag[i] = (float)(J.qd[i] * (double)tn);
+}
+
+// Up to TQL_K implicit QL sweeps (EISPACK tql2 recurrences) per factor; lane 0 chases, all 64 lanes search
+// for the negligible off-diagonal entry.  The recurrences on the tridiagonal entries run in fp64 (same issue
+// rate as fp32 on this GPU): in fp32 the rounding of the O(1) entries at the far end of an unreduced block
+// leaves a noise floor of ~1e-7 on the small entries at the deflating end, which both stalls convergence and
+// costs absolute accuracy on small eigenvalues.  The logged rotations are fp32.  Dynamic LDS: 2 * dpad doubles.
+__global__ __launch_bounds__(64) void tql_sweeps_kernel(const TrdJob* __restrict__ jobs, int buf, int max_sweeps) {
+  extern __shared__ double lds64[];
+  __shared__ int ctl[4];  // l, iter, sweeps, failed
+  const TrdJob& J = jobs[blockIdx.x];
+  const int n = J.d, dpad = J.dpad, lane = threadIdx.x;
+  int* __restrict__ st = J.state;
+  int* __restrict__ hdr = J.hdr + buf * TQL_HDR;
+  float2* __restrict__ rot = J.rot + (long long)buf * TQL_K * dpad;
+  if (st[2] || st[3]) {
+    if (lane == 0) hdr[0] = 0;
+    return;
+  }
+  double* dd = lds64;
+  double* ee = lds64 + dpad;
+  for (int i = lane; i < n; i += 64) { dd[i] = J.qd[i]; ee[i] = J.qe[i]; }
+  if (lane == 0) { ctl[0] = st[0]; ctl[1] = st[1]; ctl[2] = 0; ctl[3] = 0; }
+  __syncthreads();
+  const double eps = 1.1920929e-7;      // fp32 resolution is all the caller can use
+  const double abs_tol = 1.4901161e-8;  // 2^-26 of the (unit) largest entry
+  int top = -1, bot = 0x7fffffff;
+  for (;;) {
+    int l = ctl[0];
+    const int sweeps = ctl[2];
+    if (l >= n || sweeps >= TQL_K || ctl[3]) break;
+    // smallest m >= l whose off-diagonal entry is negligible (ee[n - 1] = 0 ends every search)
+    int m = l;
+    for (;;) {
+      const int idx = m + lane;
+      bool small = true;
+      if (idx < n - 1) {
+        const double av = fabs(ee[idx]);
+        small = (av <= eps * (fabs(dd[idx]) + fabs(dd[idx + 1]))) || (av <= abs_tol);
+      }
+      const unsigned long long mask = __ballot(small);
+      if (mask) { m += __ffsll((long long)mask) - 1; break; }
+      m += 64;
+    }
+    m = min(m, n - 1);
+    __syncthreads();
+    if (lane == 0) {
+      if (m == l) {
+        ctl[0] = l + 1;
+        ctl[1] = 0;
+      } else if (st[4] + sweeps >= max_sweeps) {  // total sweep budget (LAPACK steqr: 30 n)
+        ctl[3] = 1;
+      } else {
+        ctl[1] += 1;
+        double g = (dd[l + 1] - dd[l]) / (2.0 * ee[l]);
+        double r = sqrt(g * g + 1.0);
+        g = dd[m] - dd[l] + ee[l] / (g + copysign(r, g));
+        double s = 1.0, c = 1.0, pp = 0.0;
+        int i = m - 1;
+        bool under = false;
+        // Operands of index i in (e_a, d_a) and of index i - 1 in (e_b, d_b); each pair is reloaded for the index
+        // two below right after its use, i.e. a full step before it is needed again.
+        double e_a = ee[i], d_a = dd[i], d_up = dd[i + 1];
+        double e_b = ee[max(i - 1, l)], d_b = dd[max(i - 1, l)];
+        global_float2* out = (global_float2*)(rot + (long long)sweeps * dpad);
+        // One step of the chase at index i with operands (e_i, d_i).  The matrix has unit scale and entries below
+        // 2^-26 count as zero, so a bulge whose square is below 1e-30 is an exact underflow for every purpose: the
+        // sweep ends there (EISPACK's recovery).  Lane 0 is the only active lane, so the test is scalar.
+        // 1 / sqrt(t): fp32 seed (relative error 2^-23) and one Newton step in fp64 (~2e-14).  Normalising the
+        // rotation in fp32 instead was measured to bring the fp32 noise floor back.
+#define TQL_STEP(e_i, d_i)                                                       \
+  {                                                                              \
+    const double f = s * e_i, b = c * e_i;                                       \
+    const double t = f * f + g * g;                                              \
+    if (__builtin_amdgcn_ballot_w64(t < 1e-30) != 0) {                           \
+      dd[i + 1] = d_up - pp;                                                     \
+      ee[m] = 0.0;                                                               \
+      under = true;                                                              \
+      break;                                                                     \
+    }                                                                            \
+    double rinv = (double)__builtin_amdgcn_rsqf((float)t);                       \
+    rinv = rinv * (1.5 - (0.5 * t) * (rinv * rinv));                             \
+    ee[i + 1] = t * rinv;                                                        \
+    s = f * rinv;                                                                \
+    c = g * rinv;                                                                \
+    g = d_up - pp;                                                               \
+    r = (d_i - g) * s + 2.0 * c * b;                                             \
+    pp = s * r;                                                                  \
+    dd[i + 1] = g + pp;                                                          \
+    g = c * r - b;                                                               \
+    out[i] = vfloat2_t{(float)c, (float)s};                                      \
+    d_up = d_i;                                                                  \
+    const int nx = max(i - 2, l);                                                \
+    e_i = ee[nx];                                                                \
+    d_i = dd[nx];                                                                \
+  }
+        while (i >= l) {
+          TQL_STEP(e_a, d_a)
+          --i;
+          if (i < l) break;
+          TQL_STEP(e_b, d_b)
+          --i;
+        }
+#undef TQL_STEP
+        const int ls = under ? i + 1 : l;
+        if (!under) {
+          dd[l] = dd[l] - pp;
+          ee[l] = g;
+          ee[m] = 0.0;
+        }
+        if (m > ls) {
+          hdr[4 + sweeps] = ls;
+          hdr[4 + TQL_K + sweeps] = m;
+          top = max(top, m);
+          bot = min(bot, ls);
+          ctl[2] = sweeps + 1;
+        }
+      }
+    }
+    __syncthreads();
+  }
+  __syncthreads();
+  for (int i = lane; i < n; i += 64) { J.qd[i] = dd[i]; J.qe[i] = ee[i]; }
+  if (lane == 0) {
+    st[0] = ctl[0];
+    st[1] = ctl[1];
+    st[2] = (ctl[0] >= n) ? 1 : 0;
+    st[3] = ctl[3];
+    st[4] += ctl[2];
+    hdr[0] = ctl[2];
+    hdr[1] = top;
+    hdr[2] = bot;
+  }
+}
+
+// Apply one chunk of logged sweeps to the rows of Y.  Sequentially a sweep rotates rows (i, i + 1) for
+// i = m - 1 down to l:  Y[i + 1] <- s Y[i] + c Y[i + 1],  Y[i] <- c Y[i] - s Y[i + 1].
+// Pipeline: at step p stage k (sweep k) works at index i = p + k on the row handed down by stage k - 1
+// (row i) and its own carried row (row i + 1); the finished row i + 1 goes to stage k + 1, row i is carried.
+// grid (ceil(d / 256), factors): one thread per column of Y.
+__global__ __launch_bounds__(256) void tql_apply_kernel(const TrdJob* __restrict__ jobs, int buf) {
+  __shared__ float2 coef[TQL_STEPS][TQL_K];
+  __shared__ int sl[TQL_K], sm[TQL_K];
+  const TrdJob& J = jobs[blockIdx.y];
+  const int* __restrict__ hdr = J.hdr + buf * TQL_HDR;
+  const int nsweeps = hdr[0];
+  if (nsweeps == 0) return;
+  const int top = hdr[1], bot = hdr[2];
+  const int dpad = J.dpad;
+  const float2* __restrict__ rot = J.rot + (long long)buf * TQL_K * dpad;
+  const int tid = threadIdx.x;
+  const int col = blockIdx.x * 256 + tid;
+  const bool valid = col < J.d;
+  float* __restrict__ Y = J.Y + (valid ? col : 0);
+  if (tid < TQL_K) {
+    sl[tid] = (tid < nsweeps) ? hdr[4 + tid] : 0x7fffffff;
+    sm[tid] = (tid < nsweeps) ? hdr[4 + TQL_K + tid] : -1;
+  }
+  float carry[TQL_K];
+#pragma unroll
+  for (int k = 0; k < TQL_K; ++k) carry[k] = 0.f;
+  carry[0] = valid ? Y[(long long)top * dpad] : 0.f;
+  const int p_last = bot - TQL_K;
+  for (int p_hi = top - 1; p_hi >= p_last; p_hi -= TQL_STEPS) {
+    __syncthreads();
+    for (int e = tid; e < TQL_STEPS * TQL_K; e += 256) {
+      const int t = e / TQL_K, k = e % TQL_K;
+      const int i = p_hi - t + k;
+      float2 cs = make_float2(1.0f, 0.0f);
+      if (i >= sl[k] && i < sm[k]) cs = rot[(long long)k * dpad + i];
+      coef[t][k] = cs;
+    }
+    __syncthreads();
+    const int steps = min(TQL_STEPS, p_hi - p_last + 1);
+    float xn = (valid && p_hi >= bot) ? Y[(long long)p_hi * dpad] : 0.f;
+    for (int t = 0; t < steps; ++t) {
+      const int p = p_hi - t;
+      float x = xn;
+      xn = (valid && t + 1 < steps && p - 1 >= bot) ? Y[(long long)(p - 1) * dpad] : 0.f;
+#pragma unroll
+      for (int k = 0; k < TQL_K; ++k) {
+        const float2 cs = coef[t][k];
+        const float f = carry[k];
+        const float up = cs.y * x + cs.x * f;
+        carry[k] = cs.x * x - cs.y * f;
+        x = up;
+      }
+      const int r = p + TQL_K;
+      if (valid && r >= bot && r <= top) Y[(long long)r * dpad] = x;
+    }
+  }
+}
+
+// Ys[r][c] = Y[r][c] * w[r]; one workgroup per 8 rows.
+struct RowScale {
+  const float* Y;
+  float* Ys;
+  const float* w;
+  int dpad;
+  int row_begin;
+};
+__global__ __launch_bounds__(256) void eig_scale_rows_kernel(const RowScale* __restrict__ jobs, int n_jobs) {
+  int lo = 0, hi = n_jobs - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (jobs[mid].row_begin <= (int)blockIdx.x) lo = mid; else hi = mid - 1;
+  }
+  const RowScale& J = jobs[lo];
+  const int dpad = J.dpad;
+  const int r0 = (blockIdx.x - J.row_begin) * 8;
+  for (int e = threadIdx.x * 4; e < 8 * dpad; e += 256 * 4) {
+    const int r = r0 + e / dpad, c = e % dpad;
+    const float4 v = *reinterpret_cast<const float4*>(J.Y + (long long)r * dpad + c);
+    const float w = J.w[r];
+    *reinterpret_cast<float4*>(J.Ys + (long long)r * dpad + c) = make_float4(v.x * w, v.y * w, v.z * w, v.w * w);
+  }
+}
+
+}  // namespace sa

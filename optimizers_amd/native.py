@@ -32,7 +32,7 @@ EXPORTS = (
     "sa_compute_root_inverses_newton", "sa_compute_root_inverses_eigh", "sa_refresh_eigenbases_qr", "sa_update_corrected_eigenvalues",
     "sa_precondition_eigenvalue_corrected", "sa_update_grafting_and_filtered_grad", "sa_precondition",
     "sa_apply_update", "sa_grafting_only_step", "sa_plan_read_norms", "sa_plan_read_preconditioned",
-    "sa_gemm_f32", "sa_copy_f32", "sa_set_profiling", "sa_phase_ms", "sa_phase_flops", "sa_phase_launches", "sa_phase_executed_flops", "sa_set_symmetric_newton",
+    "sa_gemm_f32", "sa_copy_f32", "sa_set_profiling", "sa_phase_ms", "sa_phase_flops", "sa_phase_launches", "sa_phase_executed_flops", "sa_set_symmetric_newton", "sa_set_eigh_solver",
 )
 
 
@@ -130,6 +130,7 @@ def load() -> ctypes.CDLL:
     lib.sa_phase_executed_flops.argtypes = [c_char_p]
     lib.sa_phase_executed_flops.restype = c_double
     lib.sa_set_symmetric_newton.argtypes = [c_int32]
+    lib.sa_set_eigh_solver.argtypes = [c_int32]
     lib.sa_phase_launches.argtypes = [c_char_p]
     lib.sa_phase_launches.restype = c_int32
     for name in EXPORTS:
