@@ -544,7 +544,7 @@ class _NativeGroup:
                 if self.soap:
                     pass
                 elif self.use_eigh:
-                    logger.warning(f"Jacobi eigensolver still rotating after {self.max_jacobi_sweeps} sweeps for factor matrix {name}.")
+                    logger.warning(f"Eigensolver did not converge for factor matrix {name} ({self.max_jacobi_sweeps} Jacobi sweeps, or 30 QL sweeps per eigenvalue).")
                 else:
                     logger.warning("Newton did not converge and reached maximum number of iterations!")
         # blocks whose root cannot be used by the coupled Newton iteration fail every time
