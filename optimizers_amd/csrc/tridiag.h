@@ -324,14 +324,25 @@ __global__ __launch_bounds__(256) void tql_finish_kernel(const TrdJob* __restric
   for (int i = threadIdx.x; i < J.d; i += 256) J.diag[i] = (float)(J.qd[i] * (double)tn);
 }
 
-// Up to TQL_K implicit QL sweeps (EISPACK tql2 recurrences) per factor; lane 0 chases, all 64 lanes search
-// for the negligible off-diagonal entry.  The recurrences on the tridiagonal entries run in fp64 (same issue
-// rate as fp32 on this GPU): in fp32 the rounding of the O(1) entries at the far end of an unreduced block
-// leaves a noise floor of ~1e-7 on the small entries at the deflating end, which both stalls convergence and
-// costs absolute accuracy on small eigenvalues.  The logged rotations are fp32.  Dynamic LDS: 2 * dpad doubles.
+// Implicit QL iteration (EISPACK tql2 recurrences) on the tridiagonal matrix of one factor per wavefront, up to
+// TQL_K sweeps per launch, the rotations logged for tql_apply_kernel.
+//
+// A single chase is a chain of ~12 dependent operations per rotation, i.e. latency bound, so sweeps are
+// pipelined across the lanes of the wavefront: a batch of p <= TQL_P sweeps with fixed shifts (the eigenvalues
+// of the leading p x p block of the unreduced block, found by bisection, one per lane; the Wilkinson shift when
+// p = 1) runs with lane j working TQL_LAG indices behind lane j - 1.  Lane j reads the entries lane j - 1 left
+// behind at least two steps earlier (LDS operations of one wavefront execute in order), which is exactly the
+// sequential order of the sweeps, so the batch equals p consecutive shifted QL steps.
+//
+// The recurrences run in fp64 (same issue rate as fp32 on this GPU): in fp32 the rounding of the O(1) entries at
+// the far end of an unreduced block leaves a noise floor of ~1e-7 on the small entries at the deflating end,
+// which both stalls convergence and costs absolute accuracy on small eigenvalues.  The logged rotations are fp32.
+// Dynamic LDS: 2 * dpad doubles.
+constexpr int TQL_P = 16;
+constexpr int TQL_LAG = 4;  // even: all lanes use the same operand register set in a given step
+
 __global__ __launch_bounds__(64) void tql_sweeps_kernel(const TrdJob* __restrict__ jobs, int buf, int max_sweeps) {
   extern __shared__ double lds64[];
-  __shared__ int ctl[4];  // l, iter, sweeps, failed
   const TrdJob& J = jobs[blockIdx.x];
   const int n = J.d, dpad = J.dpad, lane = threadIdx.x;
   int* __restrict__ st = J.state;
@@ -344,15 +355,16 @@ __global__ __launch_bounds__(64) void tql_sweeps_kernel(const TrdJob* __restrict
   double* dd = lds64;
   double* ee = lds64 + dpad;
   for (int i = lane; i < n; i += 64) { dd[i] = J.qd[i]; ee[i] = J.qe[i]; }
-  if (lane == 0) { ctl[0] = st[0]; ctl[1] = st[1]; ctl[2] = 0; ctl[3] = 0; }
+  int l = st[0];
+  const int done_before = st[4];
+  int sweeps = 0;
+  bool failed = false;
+  int top = -1, bot = 0x7fffffff;
   __syncthreads();
   const double eps = 1.1920929e-7;      // fp32 resolution is all the caller can use
   const double abs_tol = 1.4901161e-8;  // 2^-26 of the (unit) largest entry
-  int top = -1, bot = 0x7fffffff;
-  for (;;) {
-    int l = ctl[0];
-    const int sweeps = ctl[2];
-    if (l >= n || sweeps >= TQL_K || ctl[3]) break;
+  // every control variable below is computed identically by all lanes (uniform)
+  while (l < n) {
     // smallest m >= l whose off-diagonal entry is negligible (ee[n - 1] = 0 ends every search)
     int m = l;
     for (;;) {
@@ -367,91 +379,133 @@ __global__ __launch_bounds__(64) void tql_sweeps_kernel(const TrdJob* __restrict
       m += 64;
     }
     m = min(m, n - 1);
-    __syncthreads();
-    if (lane == 0) {
-      if (m == l) {
-        ctl[0] = l + 1;
-        ctl[1] = 0;
-      } else if (st[4] + sweeps >= max_sweeps) {  // total sweep budget (LAPACK steqr: 30 n)
-        ctl[3] = 1;
-      } else {
-        ctl[1] += 1;
-        double g = (dd[l + 1] - dd[l]) / (2.0 * ee[l]);
-        double r = sqrt(g * g + 1.0);
-        g = dd[m] - dd[l] + ee[l] / (g + copysign(r, g));
-        double s = 1.0, c = 1.0, pp = 0.0;
-        int i = m - 1;
-        bool under = false;
-        // Operands of index i in (e_a, d_a) and of index i - 1 in (e_b, d_b); each pair is reloaded for the index
-        // two below right after its use, i.e. a full step before it is needed again.
-        double e_a = ee[i], d_a = dd[i], d_up = dd[i + 1];
-        double e_b = ee[max(i - 1, l)], d_b = dd[max(i - 1, l)];
-        global_float2* out = (global_float2*)(rot + (long long)sweeps * dpad);
-        // One step of the chase at index i with operands (e_i, d_i).  The matrix has unit scale and entries below
-        // 2^-26 count as zero, so a bulge whose square is below 1e-30 is an exact underflow for every purpose: the
-        // sweep ends there (EISPACK's recovery).  Lane 0 is the only active lane, so the test is scalar.
-        // 1 / sqrt(t): fp32 seed (relative error 2^-23) and one Newton step in fp64 (~2e-14).  Normalising the
-        // rotation in fp32 instead was measured to bring the fp32 noise floor back.
-#define TQL_STEP(e_i, d_i)                                                       \
-  {                                                                              \
-    const double f = s * e_i, b = c * e_i;                                       \
-    const double t = f * f + g * g;                                              \
-    if (__builtin_amdgcn_ballot_w64(t < 1e-30) != 0) {                           \
-      dd[i + 1] = d_up - pp;                                                     \
-      ee[m] = 0.0;                                                               \
-      under = true;                                                              \
-      break;                                                                     \
-    }                                                                            \
-    double rinv = (double)__builtin_amdgcn_rsqf((float)t);                       \
-    rinv = rinv * (1.5 - (0.5 * t) * (rinv * rinv));                             \
-    ee[i + 1] = t * rinv;                                                        \
-    s = f * rinv;                                                                \
-    c = g * rinv;                                                                \
-    g = d_up - pp;                                                               \
-    r = (d_i - g) * s + 2.0 * c * b;                                             \
-    pp = s * r;                                                                  \
-    dd[i + 1] = g + pp;                                                          \
-    g = c * r - b;                                                               \
-    out[i] = vfloat2_t{(float)c, (float)s};                                      \
-    d_up = d_i;                                                                  \
-    const int nx = max(i - 2, l);                                                \
-    e_i = ee[nx];                                                                \
-    d_i = dd[nx];                                                                \
-  }
-        while (i >= l) {
-          TQL_STEP(e_a, d_a)
-          --i;
-          if (i < l) break;
-          TQL_STEP(e_b, d_b)
-          --i;
-        }
-#undef TQL_STEP
-        const int ls = under ? i + 1 : l;
-        if (!under) {
-          dd[l] = dd[l] - pp;
-          ee[l] = g;
-          ee[m] = 0.0;
-        }
-        if (m > ls) {
-          hdr[4 + sweeps] = ls;
-          hdr[4 + TQL_K + sweeps] = m;
-          top = max(top, m);
-          bot = min(bot, ls);
-          ctl[2] = sweeps + 1;
+    if (m == l) { ++l; continue; }
+    const int p = min(TQL_P, max(1, (m - l + 1) / 2));
+    if (sweeps + p > TQL_K) break;
+    if (done_before + sweeps + p > max_sweeps) { failed = true; break; }  // total budget (LAPACK steqr: 30 n)
+    if (lane == 0) ee[m] = 0.0;
+
+    // ---- shifts
+    double sigma;
+    if (p == 1) {
+      const double dl = dd[l], el = ee[l];
+      const double gw = (dd[l + 1] - dl) / (2.0 * el);
+      const double rw = sqrt(gw * gw + 1.0);
+      sigma = dl - el / (gw + copysign(rw, gw));
+    } else {
+      // lane j: j-th eigenvalue of the leading p x p block, fp32 bisection on Sturm counts
+      float db[TQL_P], e2[TQL_P];
+      float lo = 3.0e38f, hi = -3.0e38f;
+#pragma unroll
+      for (int k = 0; k < TQL_P; ++k) {
+        const bool in = k < p;
+        db[k] = in ? (float)dd[l + k] : 0.f;
+        const float ek = (in && k < p - 1) ? (float)ee[l + k] : 0.f;
+        e2[k] = ek * ek;
+      }
+#pragma unroll
+      for (int k = 0; k < TQL_P; ++k) {
+        if (k < p) {
+          const float rad = sqrtf(e2[k]) + (k > 0 ? sqrtf(e2[k - 1]) : 0.f);
+          lo = fminf(lo, db[k] - rad);
+          hi = fmaxf(hi, db[k] + rad);
         }
       }
+      for (int it = 0; it < 24; ++it) {
+        const float mid = 0.5f * (lo + hi);
+        int cnt = 0;
+        float q = 1.0f;
+#pragma unroll
+        for (int k = 0; k < TQL_P; ++k) {
+          if (k < p) {
+            q = db[k] - mid - (k > 0 ? e2[k - 1] * __builtin_amdgcn_rcpf(q) : 0.f);
+            if (q == 0.f) q = -1e-30f;
+            cnt += (q < 0.f) ? 1 : 0;
+          }
+        }
+        if (cnt > lane) hi = mid; else lo = mid;
+      }
+      sigma = (double)(0.5f * (lo + hi));
     }
-    __syncthreads();
+
+    // ---- pipelined batch of p sweeps over [l, m]
+    double s = 1.0, c = 1.0, pp = 0.0, g = 0.0, d_up = 0.0, r;
+    double e_a = 0.0, d_a = 0.0, e_b = 0.0, d_b = 0.0;
+    bool dead = false;
+    int abort_i = l - 1;
+    const int last_k = m - l - 1;
+    const int n_iter = last_k + 1 + TQL_LAG * (p - 1);
+    global_float2* out = (global_float2*)(rot + (long long)(sweeps + min(lane, p - 1)) * dpad);
+    // One step of lane `lane` at pipeline time tau: index i = m - 1 - (tau - TQL_LAG * lane), operands (e_i, d_i)
+    // of that index; they are reloaded for the index two below right after their use.  The matrix has unit scale
+    // and entries below 2^-26 count as zero, so a bulge whose square is below 1e-30 is an exact underflow for
+    // every purpose: that sweep ends there (EISPACK's recovery).  1 / sqrt(t): fp32 seed and one Newton step in
+    // fp64 (~2e-14); normalising the rotation in fp32 instead was measured to bring the fp32 noise floor back.
+#define TQL_STEP(tau_, e_i, d_i)                                                  \
+  {                                                                               \
+    const int k = (tau_) - TQL_LAG * lane;                                        \
+    const int i = m - 1 - k;                                                      \
+    if (lane < p && k == 0) {                                                     \
+      g = dd[m] - sigma;                                                          \
+      d_up = dd[m];                                                               \
+      e_a = ee[m - 1];                                                            \
+      d_a = dd[m - 1];                                                            \
+      e_b = ee[max(m - 2, l)];                                                    \
+      d_b = dd[max(m - 2, l)];                                                    \
+    }                                                                             \
+    if (lane < p && k >= 0 && k <= last_k && !dead) {                             \
+      const double f = s * e_i, b = c * e_i;                                      \
+      const double t = f * f + g * g;                                             \
+      if (t < 1e-30) {                                                            \
+        dd[i + 1] = d_up - pp;                                                    \
+        dead = true;                                                              \
+        abort_i = i;                                                              \
+      } else {                                                                    \
+        double rinv = (double)__builtin_amdgcn_rsqf((float)t);                    \
+        rinv = rinv * (1.5 - (0.5 * t) * (rinv * rinv));                          \
+        if (k != 0) ee[i + 1] = t * rinv;                                         \
+        s = f * rinv;                                                             \
+        c = g * rinv;                                                             \
+        g = d_up - pp;                                                            \
+        r = (d_i - g) * s + 2.0 * c * b;                                          \
+        pp = s * r;                                                               \
+        dd[i + 1] = g + pp;                                                       \
+        g = c * r - b;                                                            \
+        out[i] = vfloat2_t{(float)c, (float)s};                                   \
+        d_up = d_i;                                                               \
+        if (k == last_k) {                                                        \
+          dd[l] = d_i - pp;                                                       \
+          ee[l] = g;                                                              \
+        }                                                                         \
+        const int nx = max(i - 2, l);                                             \
+        e_i = ee[nx];                                                             \
+        d_i = dd[nx];                                                             \
+      }                                                                           \
+    }                                                                             \
+    __builtin_amdgcn_wave_barrier();                                              \
+    asm volatile("" ::: "memory");                                                \
+  }
+    for (int tau = 0; tau < n_iter; tau += 2) {
+      TQL_STEP(tau, e_a, d_a)
+      TQL_STEP(tau + 1, e_b, d_b)
+    }
+#undef TQL_STEP
+    if (lane < p) {
+      hdr[4 + sweeps + lane] = dead ? abort_i + 1 : l;
+      hdr[4 + TQL_K + sweeps + lane] = m;
+    }
+    top = max(top, m);
+    bot = min(bot, l);
+    sweeps += p;
   }
   __syncthreads();
   for (int i = lane; i < n; i += 64) { J.qd[i] = dd[i]; J.qe[i] = ee[i]; }
   if (lane == 0) {
-    st[0] = ctl[0];
-    st[1] = ctl[1];
-    st[2] = (ctl[0] >= n) ? 1 : 0;
-    st[3] = ctl[3];
-    st[4] += ctl[2];
-    hdr[0] = ctl[2];
+    st[0] = l;
+    st[2] = (l >= n) ? 1 : 0;
+    st[3] = failed ? 1 : 0;
+    st[4] = done_before + sweeps;
+    hdr[0] = sweeps;
     hdr[1] = top;
     hdr[2] = bot;
   }
