@@ -338,7 +338,7 @@ __global__ __launch_bounds__(256) void tql_finish_kernel(const TrdJob* __restric
 // the far end of an unreduced block leaves a noise floor of ~1e-7 on the small entries at the deflating end,
 // which both stalls convergence and costs absolute accuracy on small eigenvalues.  The logged rotations are fp32.
 // Dynamic LDS: 2 * dpad doubles.
-constexpr int TQL_P = 16;
+constexpr int TQL_P = 8;
 constexpr int TQL_LAG = 4;  // even: all lanes use the same operand register set in a given step
 
 __global__ __launch_bounds__(64) void tql_sweeps_kernel(const TrdJob* __restrict__ jobs, int buf, int max_sweeps) {
@@ -393,39 +393,42 @@ __global__ __launch_bounds__(64) void tql_sweeps_kernel(const TrdJob* __restrict
       const double rw = sqrt(gw * gw + 1.0);
       sigma = dl - el / (gw + copysign(rw, gw));
     } else {
-      // lane j: j-th eigenvalue of the leading p x p block, fp32 bisection on Sturm counts
-      float db[TQL_P], e2[TQL_P];
-      float lo = 3.0e38f, hi = -3.0e38f;
+      // lane j: j-th eigenvalue of the leading p x p block by bisection on Sturm counts.  fp64 with a refined
+      // fp32 reciprocal: the block is graded, and a shift is only useful if it resolves the small eigenvalues.
+      double db[TQL_P], e2[TQL_P];
+      double lo = 1.0e300, hi = -1.0e300;
 #pragma unroll
       for (int k = 0; k < TQL_P; ++k) {
         const bool in = k < p;
-        db[k] = in ? (float)dd[l + k] : 0.f;
-        const float ek = (in && k < p - 1) ? (float)ee[l + k] : 0.f;
+        db[k] = in ? dd[l + k] : 0.0;
+        const double ek = (in && k < p - 1) ? ee[l + k] : 0.0;
         e2[k] = ek * ek;
       }
 #pragma unroll
       for (int k = 0; k < TQL_P; ++k) {
         if (k < p) {
-          const float rad = sqrtf(e2[k]) + (k > 0 ? sqrtf(e2[k - 1]) : 0.f);
-          lo = fminf(lo, db[k] - rad);
-          hi = fmaxf(hi, db[k] + rad);
+          const double rad = sqrt(e2[k]) + (k > 0 ? sqrt(e2[k - 1]) : 0.0);
+          lo = fmin(lo, db[k] - rad);
+          hi = fmax(hi, db[k] + rad);
         }
       }
-      for (int it = 0; it < 24; ++it) {
-        const float mid = 0.5f * (lo + hi);
+      for (int it = 0; it < 44; ++it) {
+        const double mid = 0.5 * (lo + hi);
         int cnt = 0;
-        float q = 1.0f;
+        double q = 1.0;
 #pragma unroll
         for (int k = 0; k < TQL_P; ++k) {
           if (k < p) {
-            q = db[k] - mid - (k > 0 ? e2[k - 1] * __builtin_amdgcn_rcpf(q) : 0.f);
-            if (q == 0.f) q = -1e-30f;
-            cnt += (q < 0.f) ? 1 : 0;
+            double qi = (double)__builtin_amdgcn_rcpf((float)q);
+            qi = qi * (2.0 - q * qi);
+            q = db[k] - mid - (k > 0 ? e2[k - 1] * qi : 0.0);
+            if (fabs(q) < 1e-30) q = -1e-30;
+            cnt += (q < 0.0) ? 1 : 0;
           }
         }
         if (cnt > lane) hi = mid; else lo = mid;
       }
-      sigma = (double)(0.5f * (lo + hi));
+      sigma = 0.5 * (lo + hi);
     }
 
     // ---- pipelined batch of p sweeps over [l, m]
