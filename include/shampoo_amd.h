@@ -138,6 +138,16 @@ int32_t sa_compute_root_inverses_eigh(sa_plan* plan, float bias_correction2, flo
                                       int32_t perturb_before_computation, int32_t max_sweeps,
                                       int32_t* sweeps_out, int32_t* status_out, void* stream);
 
+/* Eigenbasis refresh through a full symmetric eigendecomposition: the `EighEigendecompositionConfig` branch of
+ * matrix_eigendecomposition (matrix_functions.py:725-770, :885-900) inside the eigenvalue-corrected list's
+ * amortized computation (shampoo_preconditioner_list.py:1793-1990).  A = factor / bias_correction2 + epsilon I
+ * (pass epsilon = 0 when the config does not perturb before the computation); the eigenvectors, in ascending
+ * order of their eigenvalues, replace `eigenvectors[]` of every active block.  tolerance != 0: a factor whose
+ * stored basis Q already satisfies ||B - diag B||_F <= tolerance ||B||_F, B = Q^T A Q, keeps it
+ * (matrix_functions.py:772-797).  status / sweeps arrays as in sa_compute_root_inverses_eigh. */
+int32_t sa_refresh_eigenbases_eigh(sa_plan* plan, float bias_correction2, float epsilon, float tolerance, int32_t max_sweeps,
+                                   int32_t* sweeps_out, int32_t* status_out, void* stream);
+
 /* Eigenbasis refresh of eigenvalue-corrected Shampoo with the QR algorithm: B = Q^T A Q with
  * A = unpack(factor / bias_correction2) + epsilon I; while ||B - diag(B)||_F > tolerance ||B||_F and fewer than
  * max_iterations were done: (Q', R) = qr(B) (blocked Householder), Q <- Q Q', B <- Q^T A Q; finally the columns

@@ -321,6 +321,61 @@ __global__ __launch_bounds__(256) void eig_scale_cols_kernel(const EigFinal* __r
   }
 }
 
+// Stable ascending order of the eigenvalues of one factor (ties keep their index order, like
+// torch.linalg.eigh's ascending output up to degenerate pairs): order[k] = index of the k-th smallest.
+// One workgroup per factor.
+struct RankJob {
+  const float* lambda_in;
+  long long lambda_stride;
+  int* order;
+  int d;
+};
+__global__ __launch_bounds__(256) void eig_rank_kernel(const RankJob* __restrict__ jobs) {
+  const RankJob& J = jobs[blockIdx.x];
+  const int d = J.d;
+  for (int i = threadIdx.x; i < d; i += 256) {
+    const float x = J.lambda_in[i * J.lambda_stride];
+    int rank = 0;
+    for (int j = 0; j < d; ++j) {
+      const float y = J.lambda_in[j * J.lambda_stride];
+      rank += (y < x || (y == x && j < i)) ? 1 : 0;
+    }
+    J.order[rank] = i;
+  }
+}
+
+// dst[r][k] = src[order[k]][r]: eigenvectors held as rows become sorted columns.  32 x 32 tiles through LDS,
+// grid (ceil(d / 32), ceil(d / 32), factors).
+struct RowsToCols {
+  const float* src;
+  float* dst;
+  const int* order;
+  long long lds_, ldd;
+  int d;
+};
+__global__ __launch_bounds__(256) void rows_to_sorted_cols_kernel(const RowsToCols* __restrict__ jobs) {
+  __shared__ float tile[32][33];
+  const RowsToCols& J = jobs[blockIdx.z];
+  const int d = J.d;
+  const int k0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+  if (k0 >= d || r0 >= d) return;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  for (int kk = ty; kk < 32; kk += 8) {
+    const int k = k0 + kk, r = r0 + tx;
+    float v = 0.f;
+    if (k < d && r < d) {
+      const int row = min(max(J.order[k], 0), d - 1);  // clamp: a NaN spectrum leaves ranks undefined
+      v = J.src[row * J.lds_ + r];
+    }
+    tile[kk][tx] = v;
+  }
+  __syncthreads();
+  for (int rr = ty; rr < 32; rr += 8) {
+    const int r = r0 + rr, k = k0 + tx;
+    if (r < d && k < d) J.dst[r * J.ldd + k] = tile[tx][rr];
+  }
+}
+
 // dense <- packed / bc2 (+ eps on the diagonal), V <- I : start of an eigendecomposition.
 struct EigInit {
   const float* packed;

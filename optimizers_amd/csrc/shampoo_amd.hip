@@ -259,6 +259,8 @@ struct sa_plan {
   hipEvent_t trd_ev[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
   Table<GemmProblem> t_trd_gemm;
   Table<RowScale> t_rowscale;
+  Table<RankJob> t_rank;
+  Table<RowsToCols> t_rows2cols;
   GemmTable eig_gemm_t;
   Table<Copy2D> t_copy;
   Table<NormPair> t_normpair;
@@ -674,7 +676,7 @@ void sa_plan_destroy(sa_plan* p) {
   p->t_jacobi.destroy(); p->t_sched.destroy(); p->t_eiginit.destroy(); p->t_eigfinal.destroy(); p->eig_gemm.t.destroy();
   if (p->trd_stream) { (void)hipStreamSynchronize(p->trd_stream); (void)hipStreamDestroy(p->trd_stream); }
   for (hipEvent_t e : p->trd_ev) if (e) (void)hipEventDestroy(e);
-  p->t_trd.destroy(); p->t_trd_gemm.destroy(); p->t_rowscale.destroy(); p->eig_gemm_t.t.destroy();
+  p->t_trd.destroy(); p->t_trd_gemm.destroy(); p->t_rowscale.destroy(); p->eig_gemm_t.t.destroy(); p->t_rank.destroy(); p->t_rows2cols.destroy();
   for (GemmTable* g : {&p->ec_stat1, &p->ec_stat2, &p->ec_stat_l, &p->ec_stat_r, &p->ec_p1, &p->ec_p1d, &p->ec_p2, &p->ec_p2d,
                        &p->ec_p3, &p->ec_p3n, &p->ec_p4, &p->ec_p4n, &p->qr_aq, &p->qr_b})
     g->t.destroy();
@@ -1420,55 +1422,30 @@ static int eigh_tridiagonal(sa_plan* p, const std::vector<int>& ids, hipStream_t
 // Batched eigendecomposition root inverse (block Jacobi)
 // --------------------------------------------------------------------------------------------
 
-int32_t sa_compute_root_inverses_eigh(sa_plan* p, float bias_correction2, float epsilon, const float* roots,
-                                      int32_t perturb_before_computation, int32_t max_sweeps, int32_t* sweeps_out,
-                                      int32_t* status_out, void* stream) {
-  if (!p || !roots || !sweeps_out || !status_out) return fail(SA_ERR_INVALID, "sa_compute_root_inverses_eigh: NULL argument");
-  if (!(bias_correction2 != 0.0f) || max_sweeps < 1) return fail(SA_ERR_INVALID, "bad bias correction or max_sweeps");
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  SACHECK(ensure_tables(p, nullptr, s));
-  const int F = (int)p->factors.size();
-  if (F == 0) return SA_OK;
-  for (int i = 0; i < F; ++i)
-    if (!(roots[i] > 0.0f)) return fail(SA_ERR_INVALID, "Root " + std::to_string(roots[i]) + " should be positive!");
-  const float ridge = perturb_before_computation ? epsilon : 0.0f;
-  std::vector<int> todo;
-  SACHECK(root_inverse_prologue(p, bias_correction2, ridge, sweeps_out, status_out, s, &todo));
-  if (todo.empty()) return SA_OK;
-  const int n = (int)todo.size();
-
-  // Frobenius norms (for the absolute rotation threshold)
-  std::vector<float> fro(n);
-  {
-    std::vector<float> partials(p->norm_partials_total);
-    HIPCHECK(hipMemcpyAsync(partials.data(), p->f(p->off_norm_partial), partials.size() * sizeof(float), hipMemcpyDeviceToHost, s));
-    HIPCHECK(hipStreamSynchronize(s));
-    for (int i = 0; i < n; ++i) {
-      const Factor& f = p->factors[todo[i]];
-      double acc = 0.0;
-      for (int c = 0; c < f.norm_chunks; ++c) acc += partials[f.norm_off + c];
-      fro[i] = (float)std::sqrt(acc);
-    }
-  }
-
-  // A <- unpack(factor / bc2) + ridge I, V <- I
-  SACHECK(p->t_eiginit.begin(n));
-  int tiles = 0;
-  for (int i = 0; i < n; ++i) {
+// Frobenius norms of the ridged, bias-corrected factors from the partial sums root_inverse_prologue left
+// (the absolute rotation threshold of the Jacobi solver).
+static int factor_frobenius_norms(sa_plan* p, const std::vector<int>& todo, hipStream_t s, std::vector<float>* fro) {
+  fro->resize(todo.size());
+  std::vector<float> partials(p->norm_partials_total);
+  HIPCHECK(hipMemcpyAsync(partials.data(), p->f(p->off_norm_partial), partials.size() * sizeof(float), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipStreamSynchronize(s));
+  for (size_t i = 0; i < todo.size(); ++i) {
     const Factor& f = p->factors[todo[i]];
-    EigInit& J = p->t_eiginit.host[i];
-    std::memset(&J, 0, sizeof(J));
-    J.packed = f.factor;
-    J.A = newton_buf(p, NB_M0, f);
-    J.V = newton_buf(p, NB_X0, f);
-    J.d = f.d; J.dpad = f.dpad; J.tiles = f.dpad / 64; J.enabled = 1;
-    J.tile_begin = tiles;
-    tiles += J.tiles * J.tiles;
+    double acc = 0.0;
+    for (int c = 0; c < f.norm_chunks; ++c) acc += partials[f.norm_off + c];
+    (*fro)[i] = (float)std::sqrt(acc);
   }
-  SACHECK(p->t_eiginit.upload(s));
-  hipLaunchKernelGGL(eig_init_kernel, dim3(tiles), dim3(256), 0, s, p->t_eiginit.dev, n, bias_correction2, ridge);
-  HIPCHECK(hipGetLastError());
+  return SA_OK;
+}
 
+// Eigendecomposition of the dense matrices in the M0 arrays of the factors `todo` (X0 must hold the identity).
+// Block Jacobi for small orders: eigenvalues end up on the diagonal of M0 and eigenvectors in the columns of X0.
+// Tridiagonalisation + QL otherwise (via_trd[i] = 1): eigenvalues in a vector, eigenvectors in the rows of X0.
+// `fro[k]` is the Frobenius norm of the matrix of todo[k]; active[i] != 0 on return marks a factor that did not converge.
+static int eigh_solve(sa_plan* p, const std::vector<int>& todo, const std::vector<float>& fro, int max_sweeps, int32_t* sweeps_out,
+                      std::vector<int>& active, std::vector<char>& via_trd, hipStream_t s) {
+  const int F = (int)p->factors.size();
+  const int n = (int)todo.size();
   // solver per factor: block Jacobi for small orders, tridiagonalisation + QL for the rest
   std::vector<int> jac, jac_pos;            // factor ids / positions in todo
   std::map<int, std::vector<int>> trd_by_d; // order -> factor ids
@@ -1478,8 +1455,8 @@ int32_t sa_compute_root_inverses_eigh(sa_plan* p, float bias_correction2, float 
       trd_by_d[f.d].push_back(todo[k]);
     else { jac.push_back(todo[k]); jac_pos.push_back(k); }
   }
-  std::vector<int> active(F, 0);
-  std::vector<char> via_trd(F, 0);
+  active.assign(F, 0);
+  via_trd.assign(F, 0);
 
   if (!jac.empty()) {
     const int nj = (int)jac.size();
@@ -1568,6 +1545,51 @@ int32_t sa_compute_root_inverses_eigh(sa_plan* p, float bias_correction2, float 
     for (int i : kv.second) via_trd[i] = 1;
   }
 
+  return SA_OK;
+}
+
+int32_t sa_compute_root_inverses_eigh(sa_plan* p, float bias_correction2, float epsilon, const float* roots,
+                                      int32_t perturb_before_computation, int32_t max_sweeps, int32_t* sweeps_out,
+                                      int32_t* status_out, void* stream) {
+  if (!p || !roots || !sweeps_out || !status_out) return fail(SA_ERR_INVALID, "sa_compute_root_inverses_eigh: NULL argument");
+  if (!(bias_correction2 != 0.0f) || max_sweeps < 1) return fail(SA_ERR_INVALID, "bad bias correction or max_sweeps");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SACHECK(ensure_tables(p, nullptr, s));
+  const int F = (int)p->factors.size();
+  if (F == 0) return SA_OK;
+  for (int i = 0; i < F; ++i)
+    if (!(roots[i] > 0.0f)) return fail(SA_ERR_INVALID, "Root " + std::to_string(roots[i]) + " should be positive!");
+  const float ridge = perturb_before_computation ? epsilon : 0.0f;
+  std::vector<int> todo;
+  SACHECK(root_inverse_prologue(p, bias_correction2, ridge, sweeps_out, status_out, s, &todo));
+  if (todo.empty()) return SA_OK;
+  const int n = (int)todo.size();
+
+  std::vector<float> fro;
+  SACHECK(factor_frobenius_norms(p, todo, s, &fro));
+
+  // A <- unpack(factor / bc2) + ridge I, V <- I
+  SACHECK(p->t_eiginit.begin(n));
+  int tiles = 0;
+  for (int i = 0; i < n; ++i) {
+    const Factor& f = p->factors[todo[i]];
+    EigInit& J = p->t_eiginit.host[i];
+    std::memset(&J, 0, sizeof(J));
+    J.packed = f.factor;
+    J.A = newton_buf(p, NB_M0, f);
+    J.V = newton_buf(p, NB_X0, f);
+    J.d = f.d; J.dpad = f.dpad; J.tiles = f.dpad / 64; J.enabled = 1;
+    J.tile_begin = tiles;
+    tiles += J.tiles * J.tiles;
+  }
+  SACHECK(p->t_eiginit.upload(s));
+  hipLaunchKernelGGL(eig_init_kernel, dim3(tiles), dim3(256), 0, s, p->t_eiginit.dev, n, bias_correction2, ridge);
+  HIPCHECK(hipGetLastError());
+
+  std::vector<int> active;
+  std::vector<char> via_trd;
+  SACHECK(eigh_solve(p, todo, fro, max_sweeps, sweeps_out, active, via_trd, s));
+
   // X = V diag(f(lambda)) V^T
   SACHECK(p->t_eigfinal.begin(n));
   SACHECK(p->t_rowscale.begin(n));
@@ -1630,6 +1652,170 @@ int32_t sa_compute_root_inverses_eigh(sa_plan* p, float bias_correction2, float 
 // --------------------------------------------------------------------------------------------
 // Eigenvalue-corrected Shampoo (SOAP)
 // --------------------------------------------------------------------------------------------
+
+// Eigenbasis refresh of eigenvalue-corrected Shampoo through a full eigendecomposition
+// (EighEigendecompositionConfig, matrix_functions.py:725-770 and :885-900): eigenvectors in ascending order of
+// their eigenvalues replace the stored basis.  With tolerance != 0 a factor whose current basis already satisfies
+// ||B - diag B||_F <= tolerance ||B||_F, B = Q^T A Q, keeps it.
+int32_t sa_refresh_eigenbases_eigh(sa_plan* p, float bias_correction2, float epsilon, float tolerance, int32_t max_sweeps,
+                                   int32_t* sweeps_out, int32_t* status_out, void* stream) {
+  if (!p || !sweeps_out || !status_out) return fail(SA_ERR_INVALID, "sa_refresh_eigenbases_eigh: NULL argument");
+  if (!p->eigenvalue_corrected) return fail(SA_ERR_STATE, "plan has no eigenvector state");
+  if (!(bias_correction2 != 0.0f) || max_sweeps < 1) return fail(SA_ERR_INVALID, "bad bias correction or max_sweeps");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SACHECK(ensure_tables(p, nullptr, s));
+  const int F = (int)p->factors.size();
+  if (F == 0) return SA_OK;
+  std::vector<int> todo;
+  SACHECK(root_inverse_prologue(p, bias_correction2, epsilon, sweeps_out, status_out, s, &todo));
+  if (todo.empty()) return SA_OK;
+
+  auto init_dense = [&](const std::vector<int>& ids) -> int {  // M0 <- unpack(factor / bc2) + eps I, X0 <- I
+    SACHECK(p->t_eiginit.begin(ids.size()));
+    int tiles = 0;
+    for (size_t i = 0; i < ids.size(); ++i) {
+      const Factor& f = p->factors[ids[i]];
+      EigInit& J = p->t_eiginit.host[i];
+      std::memset(&J, 0, sizeof(J));
+      J.packed = f.factor; J.A = newton_buf(p, NB_M0, f); J.V = newton_buf(p, NB_X0, f);
+      J.d = f.d; J.dpad = f.dpad; J.tiles = f.dpad / 64; J.enabled = 1; J.tile_begin = tiles;
+      tiles += J.tiles * J.tiles;
+    }
+    SACHECK(p->t_eiginit.upload(s));
+    hipLaunchKernelGGL(eig_init_kernel, dim3(tiles), dim3(256), 0, s, p->t_eiginit.dev, (int)ids.size(), bias_correction2, epsilon);
+    HIPCHECK(hipGetLastError());
+    return SA_OK;
+  };
+  SACHECK(init_dense(todo));
+
+  std::vector<int> solve = todo;
+  if (tolerance != 0.0f) {
+    // B = Q^T (A Q) with the stored basis: X1 <- Q (padded), M1 <- A Q, S1 <- Q^T M1
+    const int n = (int)todo.size();
+    SACHECK(p->t_copy.begin(n));
+    SACHECK(p->t_normpair.begin(n));
+    p->qr_aq.clear();
+    p->qr_b.clear();
+    for (int k = 0; k < n; ++k) {
+      const Factor& f = p->factors[todo[k]];
+      Copy2D& C = p->t_copy.host[k];
+      std::memset(&C, 0, sizeof(C));
+      C.src = f.eigvec; C.lds_ = f.d; C.dst = newton_buf(p, NB_X1, f); C.ldd = f.dpad; C.rows = f.d; C.cols = f.d;
+      GemmProblem q{};
+      q.A = newton_buf(p, NB_M0, f); q.lda = f.dpad; q.a_vec = 1;
+      q.B = newton_buf(p, NB_X1, f); q.ldb = f.dpad; q.b_vec = 1;
+      q.C = newton_buf(p, NB_M1, f); q.ldc = f.dpad; q.M = q.N = q.K = f.d;
+      p->qr_aq.add(q, false);
+      GemmProblem b{};
+      b.A = newton_buf(p, NB_X1, f); b.lda = f.dpad; b.a_vec = 1;
+      b.B = newton_buf(p, NB_M1, f); b.ldb = f.dpad; b.b_vec = 1;
+      b.C = newton_buf(p, NB_S1, f); b.ldc = f.dpad; b.M = b.N = b.K = f.d;
+      p->qr_b.add(b, false);
+      NormPair& J = p->t_normpair.host[k];
+      J.B = newton_buf(p, NB_S1, f); J.ldb = f.dpad; J.d = f.d;
+      J.out_all = p->d_final_err + todo[k];
+      J.out_diag = reinterpret_cast<float*>(p->d_err) + todo[k];
+    }
+    SACHECK(p->t_copy.upload(s));
+    SACHECK(p->t_normpair.upload(s));
+    SACHECK(p->qr_aq.commit(s));
+    SACHECK(p->qr_b.commit(s));
+    hipLaunchKernelGGL(copy2d_kernel, dim3(64, n), dim3(256), 0, s, p->t_copy.dev);
+    HIPCHECK(hipGetLastError());
+    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE>(p->qr_aq, unit_scalars(), s)));
+    SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_STORE>(p->qr_b, unit_scalars(), s)));
+    hipLaunchKernelGGL(diag_off_norm_kernel, dim3(n), dim3(256), 0, s, p->t_normpair.dev);
+    HIPCHECK(hipGetLastError());
+    HIPCHECK(hipMemcpyAsync(p->h_pinned, p->d_final_err, F * sizeof(float), hipMemcpyDeviceToHost, s));
+    HIPCHECK(hipMemcpyAsync(p->h_pinned + F, p->d_err, F * sizeof(float), hipMemcpyDeviceToHost, s));
+    HIPCHECK(hipStreamSynchronize(s));
+    const float* h_all = reinterpret_cast<const float*>(p->h_pinned);
+    const float* h_diag = reinterpret_cast<const float*>(p->h_pinned + F);
+    solve.clear();
+    for (int i : todo) {
+      const float norm = std::sqrt(h_all[i]), dnorm = std::sqrt(h_diag[i]);
+      const float off = std::sqrt(norm * norm - dnorm * dnorm);
+      if (off <= tolerance * norm) status_out[i] = SA_FACTOR_OK;  // the stored basis stays
+      else solve.push_back(i);
+    }
+    HIPCHECK(hipMemsetAsync(p->d_err, 0, F * sizeof(int), s));
+    if (solve.empty()) return SA_OK;
+  }
+
+  const int n = (int)solve.size();
+  std::vector<float> fro_all, fro(n);
+  SACHECK(factor_frobenius_norms(p, todo, s, &fro_all));
+  for (int k = 0; k < n; ++k)
+    fro[k] = fro_all[std::find(todo.begin(), todo.end(), solve[k]) - todo.begin()];
+  std::vector<int> active;
+  std::vector<char> via_trd;
+  SACHECK(eigh_solve(p, solve, fro, max_sweeps, sweeps_out, active, via_trd, s));
+
+  // ascending order, sorted eigenvectors (columns) -> S1, finiteness, then into the state
+  SACHECK(p->t_rank.begin(n));
+  SACHECK(p->t_copy.begin(n));
+  SACHECK(p->t_rows2cols.begin(n));
+  SACHECK(p->t_normjobs.begin(n));
+  int n_cols = 0, n_rows = 0, chunks = 0, dmax = 0;
+  for (int k = 0; k < n; ++k) {
+    const Factor& f = p->factors[solve[k]];
+    const bool t = via_trd[solve[k]] != 0;
+    dmax = std::max(dmax, f.d);
+    RankJob& R = p->t_rank.host[k];
+    R.lambda_in = t ? newton_buf(p, NB_M1, f) + trd_diag_offset(f) : newton_buf(p, NB_M0, f);
+    R.lambda_stride = t ? 1 : (long long)f.dpad + 1;
+    R.order = reinterpret_cast<int*>(newton_buf(p, NB_MP0, f));
+    R.d = f.d;
+    if (t) {
+      RowsToCols& C = p->t_rows2cols.host[n_rows++];
+      C.src = newton_buf(p, NB_X0, f); C.lds_ = f.dpad; C.dst = newton_buf(p, NB_S1, f); C.ldd = f.dpad; C.order = R.order; C.d = f.d;
+    } else {
+      Copy2D& C = p->t_copy.host[n_cols++];
+      std::memset(&C, 0, sizeof(C));
+      C.src = newton_buf(p, NB_X0, f); C.lds_ = f.dpad; C.dst = newton_buf(p, NB_S1, f); C.ldd = f.dpad;
+      C.rows = f.d; C.cols = f.d; C.perm = R.order;
+    }
+    NormJob& J = p->t_normjobs.host[k];
+    std::memset(&J, 0, sizeof(J));
+    J.src = newton_buf(p, NB_S1, f); J.nonfinite = p->d_flags + solve[k];
+    J.d = f.d; J.dpad = f.dpad; J.dense = 1; J.chunk_begin = chunks;
+    J.n_chunks = (int)(((long long)f.d * f.d + NORM_CHUNK - 1) / NORM_CHUNK); J.enabled = 1;
+    chunks += J.n_chunks;
+  }
+  p->t_copy.n = n_cols;
+  p->t_rows2cols.n = n_rows;
+  SACHECK(p->t_rank.upload(s));
+  SACHECK(p->t_copy.upload(s));
+  SACHECK(p->t_rows2cols.upload(s));
+  SACHECK(p->t_normjobs.upload(s));
+  HIPCHECK(hipMemsetAsync(p->d_flags, 0, F * sizeof(int), s));
+  hipLaunchKernelGGL(eig_rank_kernel, dim3(n), dim3(256), 0, s, p->t_rank.dev);
+  if (n_cols) hipLaunchKernelGGL(copy2d_kernel, dim3(64, n_cols), dim3(256), 0, s, p->t_copy.dev);
+  if (n_rows) hipLaunchKernelGGL(rows_to_sorted_cols_kernel, dim3((dmax + 31) / 32, (dmax + 31) / 32, n_rows), dim3(256), 0, s, p->t_rows2cols.dev);
+  hipLaunchKernelGGL((factor_norm_kernel<true>), dim3(chunks), dim3(256), 0, s, p->t_normjobs.dev, n, 1.0f, 0.0f);
+  HIPCHECK(hipGetLastError());
+  int* h_bad = p->h_pinned + 3 * F;
+  HIPCHECK(hipMemcpyAsync(h_bad, p->d_flags, F * sizeof(int), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipStreamSynchronize(s));
+  int ok = n;
+  for (int k = 0; k < n; ++k)
+    if (k < ok && h_bad[solve[k]]) { status_out[solve[k]] = SA_FACTOR_RESULT_NONFINITE; ok = k; }
+  if (ok > 0) {
+    SACHECK(p->t_copy.begin(ok));
+    for (int k = 0; k < ok; ++k) {
+      const Factor& f = p->factors[solve[k]];
+      Copy2D& C = p->t_copy.host[k];
+      std::memset(&C, 0, sizeof(C));
+      C.src = newton_buf(p, NB_S1, f); C.lds_ = f.dpad; C.dst = f.eigvec; C.ldd = f.d; C.rows = f.d; C.cols = f.d;
+      status_out[solve[k]] = active[solve[k]] ? SA_FACTOR_NOT_CONVERGED : SA_FACTOR_OK;
+    }
+    SACHECK(p->t_copy.upload(s));
+    hipLaunchKernelGGL(copy2d_kernel, dim3(64, ok), dim3(256), 0, s, p->t_copy.dev);
+    HIPCHECK(hipGetLastError());
+    HIPCHECK(hipStreamSynchronize(s));
+  }
+  return SA_OK;
+}
 
 int32_t sa_update_corrected_eigenvalues(sa_plan* p, float beta2, float weighting_factor, void* stream) {
   if (!p) return fail(SA_ERR_INVALID, "NULL plan");

@@ -26,6 +26,7 @@ from optimizers_amd.matrix_functions_types import (
     CoupledNewtonConfig,
     EigenConfig,
     EigendecompositionConfig,
+    EighEigendecompositionConfig,
     PerturbationConfig,
     PseudoInverseConfig,
     QREigendecompositionConfig,
@@ -321,10 +322,14 @@ class _NativeGroup:
             raise NotImplementedError(f"{pc=} not supported!")
         acc = pc.amortized_computation_config
         if isinstance(pc, EigenvalueCorrectedShampooPreconditionerConfig):
-            if not isinstance(acc, QREigendecompositionConfig):
+            if not isinstance(acc, (QREigendecompositionConfig, EighEigendecompositionConfig)):
                 raise NotImplementedError(
                     f"Eigendecomposition config is not implemented! Specified eigendecomposition config is {type(acc).__name__}."
                 )
+            if not isinstance(acc.rank_deficient_stability_config, PerturbationConfig):
+                raise NotImplementedError(f"{acc.rank_deficient_stability_config=} is not supported.")
+            if isinstance(acc, EighEigendecompositionConfig) and acc.eigendecomposition_offload_device != "":
+                raise NotImplementedError("eigendecomposition_offload_device: the decomposition runs on the MI355X")
             if pc.factor_matrix_eigenvectors_dtype != torch.float32 or pc.corrected_eigenvalues_dtype != torch.float32:
                 raise NotImplementedError("eigenvectors and corrected eigenvalues are fp32 in the native step")
         elif isinstance(acc, EigenConfig):
@@ -501,7 +506,16 @@ class _NativeGroup:
         (shampoo_preconditioner_list.py:314-443)."""
         pc = self.preconditioner_config
         cfg = pc.amortized_computation_config
-        if self.soap:
+        if self.soap and isinstance(cfg, EighEigendecompositionConfig):
+            # epsilon * I is added only when the config perturbs before the computation (matrix_functions.py:869-882)
+            ridge = group[EPSILON] * float(cfg.rank_deficient_stability_config.perturb_before_computation)
+            native.check(
+                self.lib.sa_refresh_eigenbases_eigh(
+                    self.plan, bc2, ridge, cfg.tolerance, self.max_jacobi_sweeps, self.iterations, self.status, stream
+                ),
+                "sa_refresh_eigenbases_eigh",
+            )
+        elif self.soap:
             native.check(
                 self.lib.sa_refresh_eigenbases_qr(
                     self.plan, bc2, group[EPSILON], cfg.max_iterations, cfg.tolerance, self.iterations, self.status, stream

@@ -29,7 +29,7 @@ EXPORTS = (
     "sa_last_error", "sa_abi_version", "sa_plan_create", "sa_plan_destroy", "sa_plan_workspace_bytes",
     "sa_plan_bind_workspace", "sa_plan_num_factors", "sa_plan_invalidate_inverse_cache",
     "sa_plan_bind_gradients", "sa_add_l2_regularization", "sa_update_factor_matrices",
-    "sa_compute_root_inverses_newton", "sa_compute_root_inverses_eigh", "sa_refresh_eigenbases_qr", "sa_update_corrected_eigenvalues",
+    "sa_compute_root_inverses_newton", "sa_compute_root_inverses_eigh", "sa_refresh_eigenbases_qr", "sa_refresh_eigenbases_eigh", "sa_update_corrected_eigenvalues",
     "sa_precondition_eigenvalue_corrected", "sa_update_grafting_and_filtered_grad", "sa_precondition",
     "sa_apply_update", "sa_grafting_only_step", "sa_plan_read_norms", "sa_plan_read_preconditioned",
     "sa_gemm_f32", "sa_copy_f32", "sa_set_profiling", "sa_phase_ms", "sa_phase_flops", "sa_phase_launches", "sa_phase_executed_flops", "sa_set_symmetric_newton", "sa_set_eigh_solver",
@@ -110,6 +110,9 @@ def load() -> ctypes.CDLL:
     ]
     lib.sa_refresh_eigenbases_qr.argtypes = [
         c_void_p, c_float, c_float, c_int32, c_float, POINTER(c_int32), POINTER(c_int32), c_void_p,
+    ]
+    lib.sa_refresh_eigenbases_eigh.argtypes = [
+        c_void_p, c_float, c_float, c_float, c_int32, POINTER(c_int32), POINTER(c_int32), c_void_p,
     ]
     lib.sa_update_corrected_eigenvalues.argtypes = [c_void_p, c_float, c_float, c_void_p]
     lib.sa_precondition_eigenvalue_corrected.argtypes = [c_void_p, POINTER(StepScalars), c_float, c_float, c_float, c_void_p]

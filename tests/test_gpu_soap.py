@@ -67,22 +67,23 @@ def test_soap_fixture_case_matches_reference():
 
 
 # shapes whose factors all have full rank by the first refresh, so that the eigenbases are well defined
+@pytest.mark.parametrize("kind", ["soap_qr", "soap_eigh"])
 @pytest.mark.parametrize("shapes, b, graft", [([(256, 256)], 128, "adam"), ([(1024, 768)], 1024, None)])
-def test_soap_medium_blocks_match_oracle(shapes, b, graft):
+def test_soap_medium_blocks_match_oracle(shapes, b, graft, kind):
     import optimizers_amd as oa
     from oracle.shampoo_oracle import OracleConfig, ShampooOracle
 
-    print(f"case {shapes} b={b} graft={graft}", flush=True)
+    print(f"case {shapes} b={b} graft={graft} {kind}", flush=True)
     g = torch.Generator().manual_seed(17)
     init = [0.1 * torch.randn(*s, generator=g) for s in shapes]
     kw = dict(lr=1e-2, betas=(0.9, 0.99), epsilon=1e-12, max_preconditioner_dim=b, precondition_frequency=3,
               start_preconditioning_step=3)
     params = [torch.nn.Parameter(t.clone().to(DEV)) for t in init]
     opt = oa.DistributedShampoo(
-        params, preconditioner_config=oa.DefaultSOAPConfig,
+        params, preconditioner_config=oa.DefaultSOAPConfig if kind == "soap_qr" else oa.DefaultEigenvalueCorrectedShampooConfig,
         grafting_config=oa.AdamPreconditionerConfig(beta2=0.99, epsilon=1e-8) if graft else None, **kw)
     ref_p = [t.clone() for t in init]
-    ocfg = OracleConfig(preconditioner="soap_qr", grafting=graft, grafting_beta2=0.99, grafting_epsilon=1e-8, **kw)
+    ocfg = OracleConfig(preconditioner=kind, grafting=graft, grafting_beta2=0.99, grafting_epsilon=1e-8, **kw)
     ref = ShampooOracle(ref_p, ocfg)
     ref64_p = [t.clone().double() for t in init]
     ref64 = ShampooOracle(ref64_p, ocfg)
@@ -116,3 +117,30 @@ def test_soap_medium_blocks_match_oracle(shapes, b, graft):
             # leading (well separated) part of the spectrum
             lead = slice(got.shape[0] - 8, got.shape[0])
             assert rel_err(got[:, lead] @ got[:, lead].T, q[:, lead] @ q[:, lead].T) < 1e-3
+
+
+def test_eigh_refresh_tolerance_keeps_a_good_enough_basis():
+    """EighEigendecompositionConfig.tolerance (matrix_functions.py:885-897): a stored basis Q with
+    ||B - diag B||_F <= tolerance ||B||_F, B = Q^T A Q, is kept; tolerance 0 always decomposes."""
+    import optimizers_amd as oa
+
+    g = torch.Generator().manual_seed(3)
+    grad = torch.randn(64, 48, generator=g)
+    out = {}
+    for tol in (1.0, 0.0):
+        p = torch.nn.Parameter(torch.zeros(64, 48, device=DEV))
+        cfg = oa.EigenvalueCorrectedShampooPreconditionerConfig(
+            amortized_computation_config=oa.EighEigendecompositionConfig(tolerance=tol))
+        opt = oa.DistributedShampoo([p], lr=1e-2, betas=(0.9, 0.99), epsilon=1e-12, max_preconditioner_dim=64,
+                                    precondition_frequency=1, start_preconditioning_step=1, preconditioner_config=cfg)
+        p.grad = grad.to(DEV)
+        opt.step()
+        basis = opt.state[p]["block_0"]["shampoo"]["factor_matrices_eigenvectors"]
+        out[tol] = [basis[j].cpu() for j in range(2)]
+    for q in out[1.0]:  # the criterion holds trivially: the identity stays
+        assert torch.equal(q, torch.eye(q.shape[0]))
+    for q, a in zip(out[0.0], (grad @ grad.T, grad.T @ grad)):
+        assert rel_err(q.T @ q, torch.eye(q.shape[0])) < 1e-5
+        lam = torch.diagonal(q.T @ a @ q)
+        assert bool((lam[1:] >= lam[:-1] - 1e-4 * lam.abs().max()).all())  # ascending, like torch.linalg.eigh
+        assert rel_err(q @ torch.diag(lam) @ q.T, a) < 1e-4
