@@ -7,10 +7,11 @@
 //      the HBM-bound part ((4/3) d^3 bytes per factor); per 32-column panel one rank-64 trailing update
 //      A -= [V W] [W V]^T on the grouped MFMA GEMM.
 //   2. Y = Q1^T by compact-WY block reflectors (grouped GEMMs).
-//   3. T = Z diag(lambda) Z^T by implicit QL iteration with Wilkinson shifts.  One lane per factor runs the
-//      sequential bulge chase and logs the rotations of up to TQL_K sweeps; a second kernel applies that
-//      chunk of sweeps to the rows of Y as a register-resident systolic pipeline (one thread per column of
-//      Y, one carried row per sweep), so Y is read and written once per chunk instead of once per sweep.
+//   3. T = Z diag(lambda) Z^T by implicit QL iteration.  One wavefront per factor runs the bulge chases, several
+//      shifted sweeps at a time pipelined across its lanes, and logs the rotations of up to TQL_K sweeps; a
+//      second kernel applies that chunk of sweeps to the rows of Y as a register-resident systolic pipeline
+//      (one thread per column of Y, one carried row per sweep), so Y is read and written once per chunk
+//      instead of once per sweep.
 // On exit row i of Y is the eigenvector of eigenvalue diag[i] (not sorted).
 #pragma once
 
@@ -24,8 +25,6 @@ namespace sa {
 typedef float vfloat4_t __attribute__((ext_vector_type(4)));
 typedef float vfloat2_t __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(1))) vfloat2_t global_float2;
-
-
 
 constexpr int TRD_NB = 32;               // panel width
 constexpr int TRD_PW = 2 * TRD_NB;       // row length of the [V | W] and [W | V] panel buffers
@@ -53,7 +52,7 @@ struct TrdJob {
   float* Tmat;    // (dpad / 32) x 32 x 32 triangular factors of the block reflectors
   float2* rot;    // 2 x TQL_K x dpad rotation log (c, s)
   int* hdr;       // 2 x TQL_HDR
-  int* state;     // l, iterations of the current eigenvalue, done, failed, total sweeps, bits of the scale
+  int* state;     // l, -, done, failed, total sweeps, bits of the scale
   int d, dpad;
 };
 
