@@ -1369,7 +1369,7 @@ static int eigh_tridiagonal(sa_plan* p, const std::vector<int>& ids, hipStream_t
     // The rotations of chunk c are applied on a second stream while lane 0 of every factor already chases
     // chunk c + 1; the two log buffers alternate, guarded by events in both directions.
     SACHECK(trd_side_stream(p));
-    hipStream_t s2 = getenv("SA_TRD_SERIAL") ? s : p->trd_stream;
+    hipStream_t s2 = p->trd_stream;
     HIPCHECK(hipEventRecord(p->trd_ev[4], s));
     HIPCHECK(hipStreamWaitEvent(s2, p->trd_ev[4], 0));
     long long launched = 0;
@@ -1402,15 +1402,6 @@ static int eigh_tridiagonal(sa_plan* p, const std::vector<int>& ids, hipStream_t
     for (int k = 0; k < n; ++k) {
       sweeps_out[ids[k]] = state_host[8 * k + 4];
       not_converged[ids[k]] = (state_host[8 * k + 2] && !state_host[8 * k + 3]) ? 0 : 1;
-      if (getenv("SA_DEBUG_TRD") && state_host[8 * k + 3] && k < 2) {
-        std::vector<float> dv(2 * d);
-        HIPCHECK(hipMemcpy(dv.data(), p->t_trd.host[k].diag, d * sizeof(float), hipMemcpyDeviceToHost));
-        HIPCHECK(hipMemcpy(dv.data() + d, p->t_trd.host[k].off, d * sizeof(float), hipMemcpyDeviceToHost));
-        char name[128];
-        snprintf(name, sizeof(name), "gpurun_out/trd_fail_%d.bin", k);
-        if (FILE* fp = fopen(name, "wb")) { fwrite(dv.data(), sizeof(float), dv.size(), fp); fclose(fp); }
-      }
-      if (getenv("SA_DEBUG_TRD")) fprintf(stderr, "trd factor %d: l=%d iter=%d done=%d failed=%d sweeps=%d scale=%g\n", ids[k], state_host[8*k], state_host[8*k+1], state_host[8*k+2], state_host[8*k+3], state_host[8*k+4], *reinterpret_cast<float*>(&state_host[8*k+5]));
     }
     hipLaunchKernelGGL(tql_finish_kernel, dim3(n), dim3(256), 0, s, jobs);
     HIPCHECK(hipGetLastError());

@@ -138,3 +138,44 @@ def test_eigh_handles_config5_spectrum(eigh_solver):
     # and the CPU oracle (LAPACK) satisfies the same bound, i.e. both are equally close to exact arithmetic
     Xo = eigh_inverse_root(G @ G.T, 4, 1e-12).double()
     assert rel_err(qk.T @ Xo @ qk, torch.diag(lam[keep].pow(-0.25))) < 5e-3
+
+
+def test_multi_step_large_blocks_default_solver_choice():
+    """Ten steps with the reference's default config on blocks of order 768 and 640 (tridiagonalisation + QL by the
+    library's own choice) and a 1-D block (block Jacobi), against the CPU oracle in fp32 with its fp64 run as the
+    noise floor.  Gradients of full rank and epsilon = 1e-6 keep the inverse roots well posed."""
+    import optimizers_amd as oa
+    from oracle.shampoo_oracle import OracleConfig, ShampooOracle
+
+    g = torch.Generator().manual_seed(23)
+    shapes = [(768, 640), (640,)]
+    init = [0.1 * torch.randn(*s, generator=g) for s in shapes]
+    kw = dict(lr=1e-2, betas=(0.9, 0.99), epsilon=1e-6, max_preconditioner_dim=1024, precondition_frequency=2,
+              start_preconditioning_step=2)
+    params = [torch.nn.Parameter(t.clone().to(DEV)) for t in init]
+    opt = oa.DistributedShampoo(params, preconditioner_config=oa.DefaultShampooConfig,
+                                grafting_config=oa.AdamPreconditionerConfig(beta2=0.99, epsilon=1e-8), **kw)
+    ocfg = OracleConfig(preconditioner="eigh", grafting="adam", grafting_beta2=0.99, grafting_epsilon=1e-8, **kw)
+    ref_p = [t.clone() for t in init]
+    ref = ShampooOracle(ref_p, ocfg)
+    ref64_p = [t.clone().double() for t in init]
+    ref64 = ShampooOracle(ref64_p, ocfg)
+    for step in range(10):
+        grads = [torch.randn(*s, generator=g) for s in shapes]
+        for p, gr in zip(params, grads):
+            p.grad = gr.to(DEV)
+        opt.step()
+        ref.step([x.clone() for x in grads])
+        ref64.step([x.double() for x in grads])
+        for p, r, r64 in zip(params, ref_p, ref64_p):
+            assert rel_err(p.detach().cpu(), r) < 1e-3 + 2.0 * rel_err(r, r64), step
+    sweeps = opt._groups[0].last_newton_iterations
+    assert max(sweeps) > 100  # QL sweep counts: the order-768 and order-640 factors went through the tridiagonal path
+    ng = opt._groups[0]
+    for k, bi in enumerate(ng.native_index):
+        spec = ng.block_specs[bi]
+        st = opt.state[params[spec.param_index]][spec.block_key]["shampoo"]
+        if spec.order != 2:
+            continue  # the 1-D block's factor has rank <= 10: its inverse root is noise in the reference as well
+        for j, inv in enumerate(ref.state[bi]["inv"]):
+            assert rel_err(st["inv_factor_matrices"][j].cpu(), inv) < 1e-3, (k, j)
