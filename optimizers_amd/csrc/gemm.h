@@ -299,7 +299,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(
         const float v = acc[i][j][e];
         if (EPI == EPI_STORE) {
           if (!EDGE || (row < M && col < N)) C[(long long)row * ldc + col] = v;
-          if (TRI && tm != tn && (!EDGE || (row < M && col < N))) C[(long long)col * ldc + row] = v;
+          if (TRI && EDGE && tm != tn && row < M && col < N) C[(long long)col * ldc + row] = v;
         } else if (EPI == EPI_STORE_SQNORM) {
           if (!EDGE || (row < M && col < N)) {
             C[(long long)row * ldc + col] = v;
@@ -336,7 +336,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(
           float mp = __fmul_rn(v, sc.mp_scale);
           if (row == col && row < P.d) mp = __fadd_rn(mp, sc.mp_diag);
           P.C2[(long long)row * ldc + col] = mp;
-          if (TRI && tm != tn) {
+          if (TRI && EDGE && tm != tn) {
             C[(long long)col * ldc + row] = v;
             P.C2[(long long)col * ldc + row] = mp;
           }
@@ -345,6 +345,38 @@ __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(
             if (dv != dv) local_nan = true;
             local = fmaxf(local, dv);
           }
+        }
+      }
+    }
+  }
+  if (TRI && !EDGE && (EPI == EPI_STORE || EPI == EPI_NEWTON_M)) {
+    // Mirror image of an off-diagonal tile: each 32 x 32 accumulator block is transposed through the (now idle)
+    // operand buffers, one private region per wavefront, and leaves as 16-byte stores along the rows of C.
+    if (tm != tn) {
+      constexpr int TS = 36;  // 32 + 4: keeps float4 alignment
+      float* stage = ((wave < 2) ? &As[0][0] : &Bs[0][0]) + (wave & 1) * (BK * LDS_STRIDE);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q)  // stage[col][row]: the four accumulator values of a group are four consecutive rows
+            *reinterpret_cast<float4*>(stage + l32 * TS + 8 * q + 4 * h) =
+                make_float4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+          __builtin_amdgcn_wave_barrier();
+          asm volatile("" ::: "memory");
+#pragma unroll
+          for (int it = 0; it < 4; ++it) {
+            const int c = (lane >> 3) + 8 * it, r4 = (lane & 7) * 4;
+            const float4 v = *reinterpret_cast<const float4*>(stage + c * TS + r4);
+            const long long o = (long long)(n0 + wn * 64 + j * 32 + c) * ldc + (m0 + wm * 64 + i * 32 + r4);
+            *reinterpret_cast<float4*>(C + o) = v;
+            if (EPI == EPI_NEWTON_M)  // off-diagonal tile: M_p has no diagonal term here
+              *reinterpret_cast<float4*>(P.C2 + o) = make_float4(__fmul_rn(v.x, sc.mp_scale), __fmul_rn(v.y, sc.mp_scale),
+                                                                 __fmul_rn(v.z, sc.mp_scale), __fmul_rn(v.w, sc.mp_scale));
+          }
+          __builtin_amdgcn_wave_barrier();
+          asm volatile("" ::: "memory");
         }
       }
     }
