@@ -66,7 +66,7 @@ def eigh_solver(request):
 
 
 @pytest.mark.parametrize("eigh_solver", [1, 2], indirect=True)
-@pytest.mark.parametrize("m, n, eps", [(96, 200, 1e-12), (300, 520, 1e-12), (1024, 1536, 1e-12), (130, 60, 1.0)])
+@pytest.mark.parametrize("m, n, eps", [(96, 200, 1e-12), (300, 520, 1e-12), (1024, 1536, 1e-12), (130, 60, 1.0), (515, 1001, 1e-12)])
 def test_eigh_root_inverse_matches_oracle_and_fp64_truth(m, n, eps, eigh_solver):
     from oracle.shampoo_oracle import eigh_inverse_root, pack_triu
 
