@@ -77,28 +77,35 @@ __global__ __launch_bounds__(256) void trd_clear_panel_kernel(const TrdJob* __re
     dst[e] = make_float4(0.f, 0.f, 0.f, 0.f);
 }
 
-// sum over q of V[r][q] * cw[q] + W[r][q] * cv[q] for one row of the [V | W] buffer
-__device__ __forceinline__ float panel_row_dot(const float* __restrict__ row, const float* cv, const float* cw) {
-  float acc = 0.f;
-#pragma unroll
-  for (int q4 = 0; q4 < TRD_NB / 4; ++q4) {
+// Two dot products over the first 4 * nq4 panel columns of one row of the [V | W] buffer:
+//   d1 = sum_q V[r][q] t1[q] + W[r][q] t2[q]      (correction of w)
+//   d2 = sum_q V[r][q] rowW[q] + W[r][q] rowV[q]  (correction of the next column)
+__device__ __forceinline__ void panel_row_dots(const float* __restrict__ row, int nq4, const float* t1, const float* t2,
+                                               const float* rowV, const float* rowW, float& d1, float& d2) {
+  d1 = 0.f;
+  d2 = 0.f;
+  for (int q4 = 0; q4 < nq4; ++q4) {
     const float4 v = *reinterpret_cast<const float4*>(row + 4 * q4);
     const float4 w = *reinterpret_cast<const float4*>(row + TRD_NB + 4 * q4);
-    acc += v.x * cw[4 * q4] + v.y * cw[4 * q4 + 1] + v.z * cw[4 * q4 + 2] + v.w * cw[4 * q4 + 3];
-    acc += w.x * cv[4 * q4] + w.y * cv[4 * q4 + 1] + w.z * cv[4 * q4 + 2] + w.w * cv[4 * q4 + 3];
+    const int q = 4 * q4;
+    d1 += (v.x * t1[q] + v.y * t1[q + 1]) + (v.z * t1[q + 2] + v.w * t1[q + 3]);
+    d1 += (w.x * t2[q] + w.y * t2[q + 1]) + (w.z * t2[q + 2] + w.w * t2[q + 3]);
+    d2 += (v.x * rowW[q] + v.y * rowW[q + 1]) + (v.z * rowW[q + 2] + v.w * rowW[q + 3]);
+    d2 += (w.x * rowV[q] + w.y * rowV[q + 1]) + (w.z * rowV[q + 2] + w.w * rowV[q + 3]);
   }
-  return acc;
 }
 
-// flags bit 0: finish w of column j - 1 (needs ybuf of that column); bit 1: start column j.
-// Panel columns are p0 .. p0 + 31; i = j - p0 columns of the panel are already in P1 / P2.
+// One column step of the panel reduction (LAPACK slatrd), one workgroup per factor.
+// flags bit 0: finish w of column j - 1 (needs ybuf of that column); bit 1: start column j (Householder vector).
+// Panel columns are p0 .. p0 + 31.  Both parts walk the same rows r >= j of the [V | W] buffer, so one pass
+// yields the correction of w and the pending rank-2k correction of column j.
 __global__ __launch_bounds__(TRD_COL_THREADS) void trd_column_kernel(const TrdJob* __restrict__ jobs, int j, int p0,
                                                                     int flags) {
   __shared__ float part1[32][33];
   __shared__ float part2[32][33];
   __shared__ float t1[TRD_NB], t2[TRD_NB], rowV[TRD_NB], rowW[TRD_NB];
   __shared__ float red[TRD_COL_THREADS / 64];
-  __shared__ float bc[2];
+  __shared__ float bc[3];
   const TrdJob& J = jobs[blockIdx.x];
   const int d = J.d;
   if (j >= d) return;
@@ -106,22 +113,29 @@ __global__ __launch_bounds__(TRD_COL_THREADS) void trd_column_kernel(const TrdJo
   const long long ld = J.dpad;
   float* __restrict__ P1 = J.P1;
   float* __restrict__ P2 = J.P2;
+  const bool fin = (flags & 1) != 0, start = (flags & 2) != 0;
+  const int jp = j - 1;
+  const int ip = fin ? jp - p0 : j - p0;  // panel columns complete on entry
+  const int nq4 = (ip + 3) / 4;
+  const float tau_p = fin ? J.tau[jp] : 0.f;
 
-  if (flags & 1) {
-    const int jp = j - 1, ip = jp - p0;
-    const float tau = J.tau[jp];
-    {  // t1 = W^T v, t2 = V^T v over the first ip panel columns
-      const int q = tid & 31, g = tid >> 5;
-      float a1 = 0.f, a2 = 0.f;
-      if (q < ip)
-        for (int r = jp + 1 + g; r < d; r += 32) {
-          const float vr = J.vbuf[r];
-          a1 += P1[(long long)r * TRD_PW + TRD_NB + q] * vr;
-          a2 += P1[(long long)r * TRD_PW + q] * vr;
-        }
-      part1[g][q] = a1;
-      part2[g][q] = a2;
-    }
+  if (tid < TRD_NB) {
+    t1[tid] = 0.f;
+    t2[tid] = 0.f;
+    rowV[tid] = (start && tid < ip) ? P1[(long long)j * TRD_PW + tid] : 0.f;
+    rowW[tid] = (start && tid < ip) ? P1[(long long)j * TRD_PW + TRD_NB + tid] : 0.f;
+  }
+  if (fin && ip > 0) {  // t1 = W^T v, t2 = V^T v over the ip complete columns
+    const int q = tid & 31, g = tid >> 5;
+    float a1 = 0.f, a2 = 0.f;
+    if (q < ip)
+      for (int r = j + g; r < d; r += 32) {
+        const float vr = J.vbuf[r];
+        a1 += P1[(long long)r * TRD_PW + TRD_NB + q] * vr;
+        a2 += P1[(long long)r * TRD_PW + q] * vr;
+      }
+    part1[g][q] = a1;
+    part2[g][q] = a2;
     __syncthreads();
     if (tid < TRD_NB) {
       float s1 = 0.f, s2 = 0.f;
@@ -129,54 +143,59 @@ __global__ __launch_bounds__(TRD_COL_THREADS) void trd_column_kernel(const TrdJo
       t1[tid] = s1;
       t2[tid] = s2;
     }
-    __syncthreads();
-    float wreg[TRD_ROWS_PER_THREAD];
-    float dot = 0.f;
+  }
+  __syncthreads();
+
+  // ---- one pass over the rows r >= j
+  float wreg[TRD_ROWS_PER_THREAD], vreg[TRD_ROWS_PER_THREAD], areg[TRD_ROWS_PER_THREAD];
+  float dot = 0.f;
 #pragma unroll
-    for (int k = 0; k < TRD_ROWS_PER_THREAD; ++k) {
-      const int r = jp + 1 + tid + k * TRD_COL_THREADS;
-      float w = 0.f;
-      if (r < d) {
-        // w = tau (y - V (W^T v) - W (V^T v))
-        w = tau * (J.ybuf[r] - panel_row_dot(P1 + (long long)r * TRD_PW, t2, t1));
-        dot += w * J.vbuf[r];
+  for (int k = 0; k < TRD_ROWS_PER_THREAD; ++k) {
+    const int r = j + tid + k * TRD_COL_THREADS;
+    float w = 0.f, vr = 0.f, a = 0.f;
+    if (r < d) {
+      float d1, d2;
+      panel_row_dots(P1 + (long long)r * TRD_PW, nq4, t1, t2, rowV, rowW, d1, d2);
+      if (fin) {
+        vr = J.vbuf[r];
+        w = tau_p * (J.ybuf[r] - d1);  // w = tau (y - V (W^T v) - W (V^T v))
+        dot += w * vr;
       }
-      wreg[k] = w;
+      // column j as it stands after the reflectors of this panel (row j of A is the same by symmetry)
+      if (start) a = J.A[(long long)j * ld + r] - d2;
     }
-    const float alpha = -0.5f * tau * block_sum_1024(dot, red);
+    wreg[k] = w;
+    vreg[k] = vr;
+    areg[k] = a;
+  }
+  if (fin) {
+    const float alpha = -0.5f * tau_p * block_sum_1024(dot, red);
 #pragma unroll
     for (int k = 0; k < TRD_ROWS_PER_THREAD; ++k) {
-      const int r = jp + 1 + tid + k * TRD_COL_THREADS;
+      const int r = j + tid + k * TRD_COL_THREADS;
       if (r < d) {
-        const float w = wreg[k] + alpha * J.vbuf[r];
+        const float w = wreg[k] + alpha * vreg[k];
+        wreg[k] = w;
         P1[(long long)r * TRD_PW + TRD_NB + ip] = w;
         P2[(long long)r * TRD_PW + ip] = w;
       }
     }
-    __threadfence_block();
+    if (tid == 0) bc[2] = wreg[0];  // w at row j
     __syncthreads();
+    if (start) {  // the column just completed also corrects column j: V[r][ip] W[j][ip] + W[r][ip] V[j][ip]
+      const float wj = bc[2], vj = 1.0f;  // the Householder vector of column j - 1 has its unit entry at row j
+#pragma unroll
+      for (int k = 0; k < TRD_ROWS_PER_THREAD; ++k) areg[k] -= vreg[k] * wj + wreg[k] * vj;
+    }
   }
 
-  if (flags & 2) {
+  if (start) {
     const int i = j - p0;
-    if (tid < TRD_NB) {
-      rowV[tid] = (tid < i) ? P1[(long long)j * TRD_PW + tid] : 0.f;
-      rowW[tid] = (tid < i) ? P1[(long long)j * TRD_PW + TRD_NB + tid] : 0.f;
-    }
-    __syncthreads();
-    float areg[TRD_ROWS_PER_THREAD];
     float ss = 0.f;
 #pragma unroll
     for (int k = 0; k < TRD_ROWS_PER_THREAD; ++k) {
       const int r = j + tid + k * TRD_COL_THREADS;
-      float a = 0.f;
-      if (r < d) {
-        // column j of the matrix as it stands after the i reflectors of this panel (row j is the same by symmetry)
-        a = J.A[(long long)j * ld + r];
-        if (i > 0) a -= panel_row_dot(P1 + (long long)r * TRD_PW, rowV, rowW);
-        if (r > j + 1) ss += a * a;
-      }
-      areg[k] = a;
+      if (r < d && r > j + 1) ss += areg[k] * areg[k];
     }
     const float sigma2 = block_sum_1024(ss, red);
     if (tid == 0) bc[0] = areg[0];
