@@ -1241,6 +1241,7 @@ static int eigh_tridiagonal(sa_plan* p, const std::vector<int>& ids, hipStream_t
     J.P2 = J.P1 + (long long)dpad * TRD_PW;
     J.vbuf = m1 + trd_vec_offset(f, 0);
     J.ybuf = m1 + trd_vec_offset(f, 1);
+    J.part = newton_buf(p, NB_S2, f);
     J.diag = m1 + trd_vec_offset(f, 2);
     J.off = m1 + trd_vec_offset(f, 3);
     J.tau = m1 + trd_vec_offset(f, 4);
@@ -1319,15 +1320,18 @@ static int eigh_tridiagonal(sa_plan* p, const std::vector<int>& ids, hipStream_t
 
   // ---- 1. tridiagonalise
   {
-    Span span("tridiagonalize", s, 4.0 / 3.0 * (double)d * d * d * n, 2 * d, true);  // bytes of the matrix-vector products
-    const size_t symv_lds = (size_t)dpad * sizeof(float);
+    Span span("tridiagonalize", s, 2.0 / 3.0 * (double)d * d * d * n, 3 * d, true);  // bytes of the matrix-vector products (one triangle)
     for (int b = 0; b < panels; ++b) {
       const int p0 = b * TRD_NB, kcols = std::min(TRD_NB, d - 1 - p0);
       hipLaunchKernelGGL(trd_clear_panel_kernel, dim3(std::max(1, dpad / 32), n), dim3(256), 0, s, jobs);
       for (int i = 0; i < kcols; ++i) {
         const int j = p0 + i;
         hipLaunchKernelGGL(trd_column_kernel, dim3(n), dim3(TRD_COL_THREADS), 0, s, jobs, j, p0, (i > 0 ? 1 : 0) | 2);
-        hipLaunchKernelGGL(trd_symv_kernel, dim3((d - j - 1 + TRD_SYMV_ROWS - 1) / TRD_SYMV_ROWS, n), dim3(256), symv_lds, s, jobs, j);
+        {
+          const int sbase = (j + 1) & ~(TRD_SB - 1), nbk = (d - sbase + TRD_SB - 1) / TRD_SB;
+          hipLaunchKernelGGL(trd_symv_kernel, dim3((nbk + 1) / 2, n), dim3(256), (size_t)nbk * TRD_SB * sizeof(float), s, jobs, j);
+          hipLaunchKernelGGL(trd_symv_reduce_kernel, dim3(nbk, n), dim3(256), 0, s, jobs, j);
+        }
       }
       hipLaunchKernelGGL(trd_column_kernel, dim3(n), dim3(TRD_COL_THREADS), 0, s, jobs, p0 + kcols, p0, 1);
       HIPCHECK(hipGetLastError());

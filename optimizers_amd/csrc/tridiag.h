@@ -31,7 +31,6 @@ constexpr int TRD_PW = 2 * TRD_NB;       // row length of the [V | W] and [W | V
 constexpr int TRD_COL_THREADS = 1024;
 constexpr int TRD_ROWS_PER_THREAD = 8;   // d <= 8192
 constexpr int TRD_MAX_DIM = TRD_COL_THREADS * TRD_ROWS_PER_THREAD;
-constexpr int TRD_SYMV_ROWS = 16;
 constexpr int TQL_K = 32;                // sweeps per chunk
 constexpr int TQL_STEPS = 64;            // pipeline steps whose coefficients are staged in LDS at a time
 constexpr int TQL_HDR = 4 + 2 * TQL_K;   // ints per chunk header: nsweeps, top, bot, -, l[K], m[K]
@@ -44,6 +43,7 @@ struct TrdJob {
   float* P2;      // dpad x 64: [W | V]
   float* vbuf;    // dpad: current Householder vector, zero at and above the diagonal
   float* ybuf;    // dpad: trailing matrix times vbuf
+  float* part;    // (dpad / 64)^2 x 4 x 64: transposed tile contributions of the symmetric product
   float* diag;    // dpad
   float* off;     // dpad: off[j] couples j and j + 1
   float* tau;     // dpad
@@ -162,7 +162,7 @@ __global__ __launch_bounds__(TRD_COL_THREADS) void trd_column_kernel(const TrdJo
         dot += w * vr;
       }
       // column j as it stands after the reflectors of this panel (row j of A is the same by symmetry)
-      if (start) a = J.A[(long long)j * ld + r] - d2;
+      if (start) a = J.A[(long long)r * ld + j] - d2;
     }
     wreg[k] = w;
     vreg[k] = vr;
@@ -228,36 +228,113 @@ __global__ __launch_bounds__(TRD_COL_THREADS) void trd_column_kernel(const TrdJo
   }
 }
 
-// ybuf[r] = sum_c A[r][c] vbuf[c] over r, c in (j, d).  Dynamic LDS: dpad floats.
+// ybuf = (trailing matrix) x vbuf over rows and columns in (j, d), reading only the tiles on and below the
+// diagonal (and only the lower triangle of those): the matrix is symmetric, so a 64 x 64 tile T = A[I][J],
+// J < I, serves both y_I += T v_J and y_J += T^T v_I.  Row blocks start at `base`, the 64-aligned index at or below j + 1.  One workgroup owns the
+// row blocks bx and nbk - 1 - bx (nbk + 1 tiles, the same for every workgroup).  It writes the row sums of its
+// blocks to ybuf and the transposed contributions, one 64-vector per tile and wavefront, to `part`;
+// trd_symv_reduce_kernel adds those to ybuf in a fixed order.  Dynamic LDS: nbk * 64 floats.
+constexpr int TRD_SB = 64;
+
+__device__ __forceinline__ void trd_symv_row_block(const TrdJob& J, const float* __restrict__ vs, int base, int nbk, int I) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int rsub = lane >> 4, c4 = (lane & 15) * 4;
+  const long long ld = J.dpad;
+  const int row0 = I * TRD_SB + 16 * wave + rsub;  // first of this lane's four rows (stride 4), relative to base
+  float vI[4], racc[4];
+#pragma unroll
+  for (int it = 0; it < 4; ++it) { vI[it] = vs[row0 + 4 * it]; racc[it] = 0.f; }
+  const float* __restrict__ Trow = J.A + (long long)(base + row0) * ld + base + c4;
+  for (int Jb = 0; Jb <= I; ++Jb) {
+    vfloat4_t a[4];
+#pragma unroll
+    for (int it = 0; it < 4; ++it)
+      a[it] = __builtin_nontemporal_load(reinterpret_cast<const vfloat4_t*>(Trow + (long long)(4 * it) * ld + Jb * TRD_SB));
+    const float4 vj = *reinterpret_cast<const float4*>(vs + Jb * TRD_SB + c4);
+    if (Jb == I) {
+      // Diagonal tile: only its lower triangle is used, like everywhere else (the two triangles of the matrix
+      // agree to rounding only, and on the numerically zero trailing blocks of a rank-deficient factor the
+      // rounding is all there is).  Entries above the diagonal are dropped here and come back as the
+      // transposed contribution of the strictly lower ones.
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const int rl = 16 * wave + rsub + 4 * it;  // row inside the tile
+        a[it].x = (c4 + 0 <= rl) ? a[it].x : 0.f;
+        a[it].y = (c4 + 1 <= rl) ? a[it].y : 0.f;
+        a[it].z = (c4 + 2 <= rl) ? a[it].z : 0.f;
+        a[it].w = (c4 + 3 <= rl) ? a[it].w : 0.f;
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < 4; ++it) racc[it] += (a[it].x * vj.x + a[it].y * vj.y) + (a[it].z * vj.z + a[it].w * vj.w);
+    {
+      if (Jb == I) {  // strictly lower part for the transposed contribution
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          const int rl = 16 * wave + rsub + 4 * it;
+          a[it].x = (c4 + 0 < rl) ? a[it].x : 0.f;
+          a[it].y = (c4 + 1 < rl) ? a[it].y : 0.f;
+          a[it].z = (c4 + 2 < rl) ? a[it].z : 0.f;
+          a[it].w = (c4 + 3 < rl) ? a[it].w : 0.f;
+        }
+      }
+      float4 cs = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        cs.x += a[it].x * vI[it];
+        cs.y += a[it].y * vI[it];
+        cs.z += a[it].z * vI[it];
+        cs.w += a[it].w * vI[it];
+      }
+#pragma unroll
+      for (int o = 16; o <= 32; o <<= 1) {
+        cs.x += __shfl_xor(cs.x, o, 64);
+        cs.y += __shfl_xor(cs.y, o, 64);
+        cs.z += __shfl_xor(cs.z, o, 64);
+        cs.w += __shfl_xor(cs.w, o, 64);
+      }
+      if (lane < 16) *reinterpret_cast<float4*>(J.part + ((long long)(I * nbk + Jb) * 4 + wave) * TRD_SB + c4) = cs;
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < 4; ++it) {
+    float t = racc[it];
+#pragma unroll
+    for (int o = 1; o <= 8; o <<= 1) t += __shfl_xor(t, o, 64);
+    if ((lane & 15) == 0) J.ybuf[base + row0 + 4 * it] = t;
+  }
+}
+
 __global__ __launch_bounds__(256) void trd_symv_kernel(const TrdJob* __restrict__ jobs, int j) {
   extern __shared__ float vs[];
   const TrdJob& J = jobs[blockIdx.y];
   const int d = J.d;
-  const int r0 = j + 1 + blockIdx.x * TRD_SYMV_ROWS;
-  if (r0 >= d) return;
-  const int c0 = (j + 1) & ~3, cend = (d + 3) & ~3;
-  for (int c = c0 + threadIdx.x * 4; c < cend; c += 1024)
-    *reinterpret_cast<float4*>(vs + (c - c0)) = *reinterpret_cast<const float4*>(J.vbuf + c);
+  const int base = (j + 1) & ~(TRD_SB - 1);
+  const int nbk = (d - base + TRD_SB - 1) / TRD_SB;
+  if (2 * (int)blockIdx.x >= nbk) return;
+  for (int c = threadIdx.x; c < nbk * TRD_SB; c += 256) vs[c] = (base + c > j) ? J.vbuf[base + c] : 0.f;
   __syncthreads();
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const long long ld = J.dpad;
-  const int rbase = r0 + wave * 4;
-  const float* __restrict__ rows[4];
-#pragma unroll
-  for (int k = 0; k < 4; ++k) rows[k] = J.A + (long long)min(rbase + k, d - 1) * ld;
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int c = c0 + lane * 4; c < cend; c += 256) {
-    const float4 v = *reinterpret_cast<const float4*>(vs + (c - c0));
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const vfloat4_t a = __builtin_nontemporal_load(reinterpret_cast<const vfloat4_t*>(rows[k] + c));
-      acc[k] += (a.x * v.x + a.y * v.y) + (a.z * v.z + a.w * v.w);
-    }
-  }
-#pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const float t = wave_sum(acc[k]);
-    if (lane == 0 && rbase + k < d) J.ybuf[rbase + k] = t;
+  const int I0 = blockIdx.x, I1 = nbk - 1 - blockIdx.x;
+  trd_symv_row_block(J, vs, base, nbk, I0);
+  if (I1 != I0) trd_symv_row_block(J, vs, base, nbk, I1);
+}
+
+// ybuf[J block] += sum over I >= J and the four wavefronts of part[I][J]; grid (nbk, factors).
+__global__ __launch_bounds__(256) void trd_symv_reduce_kernel(const TrdJob* __restrict__ jobs, int j) {
+  __shared__ float red[4][TRD_SB];
+  const TrdJob& J = jobs[blockIdx.y];
+  const int d = J.d;
+  const int base = (j + 1) & ~(TRD_SB - 1);
+  const int nbk = (d - base + TRD_SB - 1) / TRD_SB;
+  const int Jb = blockIdx.x;
+  const int q = threadIdx.x >> 6, r = threadIdx.x & 63;
+  float acc = 0.f;
+  for (int I = Jb; I < nbk; ++I) acc += J.part[((long long)(I * nbk + Jb) * 4 + q) * TRD_SB + r];
+  red[q][r] = acc;
+  __syncthreads();
+  if (q == 0) {
+    const int row = base + Jb * TRD_SB + r;
+    if (row > j && row < d) J.ybuf[row] += (red[0][r] + red[1][r]) + (red[2][r] + red[3][r]);
   }
 }
 
@@ -479,6 +556,8 @@ __global__ __launch_bounds__(64) void tql_sweeps_kernel(const TrdJob* __restrict
       const double t = f * f + g * g;                                             \
       if (t < 1e-30) {                                                            \
         dd[i + 1] = d_up - pp;                                                    \
+        if (k != 0) ee[i + 1] = 0.0; /* the new entry there is sqrt(t) */         \
+        ee[i] = b; /* the rotations so far turned e[i] into c e[i]; the bulge s e[i] is dropped */ \
         dead = true;                                                              \
         abort_i = i;                                                              \
       } else {                                                                    \

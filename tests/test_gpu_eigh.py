@@ -179,3 +179,33 @@ def test_multi_step_large_blocks_default_solver_choice():
             continue  # the 1-D block's factor has rank <= 10: its inverse root is noise in the reference as well
         for j, inv in enumerate(ref.state[bi]["inv"]):
             assert rel_err(st["inv_factor_matrices"][j].cpu(), inv) < 1e-3, (k, j)
+
+
+@pytest.mark.parametrize("eigh_solver", [1, 2], indirect=True)
+@pytest.mark.parametrize("m, n", [(260, 200), (300, 130), (1024, 768)])
+def test_eigenvectors_diagonalise_the_factor(m, n, eigh_solver):
+    """Backward error of the decomposition itself, read through the eigenbasis refresh of eigenvalue-corrected
+    Shampoo: Q^T Q = I and Q^T A Q diagonal to fp32 accuracy for full-rank and rank-deficient (+ I) factors.
+    (A QL sweep that ends on an underflow once left a stale off-diagonal entry behind: residual 1e-3.)"""
+    import optimizers_amd as oa
+
+    g = torch.Generator().manual_seed(m + n)
+    G = torch.randn(m, n, generator=g)
+    p = torch.nn.Parameter(torch.zeros(m, n, device=DEV))
+    cfg = oa.EigenvalueCorrectedShampooPreconditionerConfig(amortized_computation_config=oa.EighEigendecompositionConfig())
+    opt = oa.DistributedShampoo([p], lr=0.01, betas=(0.0, 1.0), epsilon=1.0, max_preconditioner_dim=max(m, n),
+                                precondition_frequency=1, start_preconditioning_step=1, use_bias_correction=False,
+                                preconditioner_config=cfg)
+    p.grad = G.to(DEV)
+    opt.step()
+    basis = opt.state[p]["block_0"]["shampoo"]["factor_matrices_eigenvectors"]
+    for j, A in enumerate([G.double() @ G.double().T, G.double().T @ G.double()]):
+        d = A.shape[0]
+        A = A + torch.eye(d, dtype=torch.float64)
+        Q = basis[j].cpu().double()
+        assert float((Q.T @ Q - torch.eye(d, dtype=torch.float64)).abs().max()) < 5e-5
+        B = Q.T @ A @ Q
+        off = B - torch.diag(torch.diagonal(B))
+        assert float(torch.linalg.norm(off) / torch.linalg.norm(A)) < 1e-5, (j, eigh_solver)
+        lam = torch.diagonal(B)
+        assert bool((lam[1:] >= lam[:-1] - 1e-5 * lam.abs().max()).all())
