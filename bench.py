@@ -27,14 +27,14 @@ PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 
 WORKLOADS = {
-    # BASELINE config 3: one Llama-3-8B decoder layer, blocks <= 2048, Newton every step
+    # benchmark configuration 3: one Llama-3-8B decoder layer, blocks <= 2048, Newton every step
     "llama3_8b_layer": dict(
         shapes=[(4096, 4096), (1024, 4096), (1024, 4096), (4096, 4096), (14336, 4096), (14336, 4096),
                 (4096, 14336), (4096,), (4096,)],
         max_preconditioner_dim=2048, grad_std=1e-2, lr=1e-3, betas=(0.9, 0.999), epsilon=1e-12,
         graft_beta2=0.999, graft_eps=1e-8,
     ),
-    # BASELINE config 2: GPT-2-small parameter set, blocks <= 1024 (ragged)
+    # benchmark configuration 2: GPT-2-small parameter set, blocks <= 1024 (ragged)
     "gpt2_small": dict(
         shapes=sum(([(2304, 768), (768, 768), (3072, 768), (768, 3072), (768,), (768,)] for _ in range(12)), [])
         + [(50257, 768)],
@@ -44,19 +44,19 @@ WORKLOADS = {
         # deficient (and makes the reference raise) until it has seen ten gradients
         start_preconditioning_step=11, distinct_gradients=12,
     ),
-    # BASELINE config 1
+    # benchmark configuration 1
     "cfg1": dict(
         shapes=[(512, 512), (512,)], max_preconditioner_dim=512, grad_std=1.0, lr=1e-3, betas=(0.9, 0.999),
         epsilon=1e-12, graft_beta2=0.999, graft_eps=1e-8,
     ),
-    # BASELINE config 4: the same Llama layer, eigenvalue-corrected Shampoo (SOAP), QR refresh every 10 steps
+    # benchmark configuration 4: the same Llama layer, eigenvalue-corrected Shampoo (SOAP), QR refresh every 10 steps
     "llama3_8b_layer_soap": dict(
         shapes=[(4096, 4096), (1024, 4096), (1024, 4096), (4096, 4096), (14336, 4096), (14336, 4096),
                 (4096, 14336), (4096,), (4096,)],
         max_preconditioner_dim=1024, grad_std=1e-2, low_rank=(32, 1e-3), lr=1e-3, betas=(0.9, 0.999), epsilon=1e-12,
         preconditioner="soap_qr", precondition_frequency=10, start_preconditioning_step=10, grafting=None,
     ),
-    # BASELINE config 5: 4096-blocks, eigendecomposition root inverse every 50 steps
+    # benchmark configuration 5: 4096-blocks, eigendecomposition root inverse every 50 steps
     "large_block_eigh": dict(
         shapes=[(4096, 4096)] * 8 + [(8192, 4096)] * 4,
         max_preconditioner_dim=4096, spectrum=(1e-6, 1.0), lr=1e-3, betas=(0.9, 0.999), epsilon=1e-12,

@@ -91,7 +91,7 @@ CASES = {
         max_preconditioner_dim=16, precondition_frequency=3, start_preconditioning_step=3,
         preconditioner="soap_qr", override_1d=False, grafting=None,
     ),
-    "cfg1_override": dict(  # BASELINE config 1 with 1-D blocks left to grafting
+    "cfg1_override": dict(  # benchmark configuration 1 with 1-D blocks left to grafting
         shapes=[[512, 512], [512]], seed=0, grad_scale=1.0, steps=10, zero_init=True, torch_seed_grads=True,
         lr=1e-3, betas=[0.9, 0.999], epsilon=1e-12, weight_decay=0.0, weight_decay_type="DECOUPLED",
         max_preconditioner_dim=512, precondition_frequency=1, start_preconditioning_step=1,
@@ -208,7 +208,7 @@ def run_case(name, c):
 
 
 def cfg1_as_stated():
-    """BASELINE config 1 verbatim: what does the reference do?"""
+    """benchmark configuration 1 verbatim: what does the reference do?"""
     torch.manual_seed(0)
     w = torch.nn.Parameter(torch.zeros(512, 512))
     b = torch.nn.Parameter(torch.zeros(512))

@@ -109,7 +109,7 @@ def test_eigh_root_inverse_matches_oracle_and_fp64_truth(m, n, eps, eigh_solver)
 
 @pytest.mark.parametrize("eigh_solver", [1, 2], indirect=True)
 def test_eigh_handles_config5_spectrum(eigh_solver):
-    """Singular values log-uniform in [1e-6, 1] (BASELINE config 5): eigenvalues span 1e-12..1."""
+    """Singular values log-uniform in [1e-6, 1] (benchmark configuration 5): eigenvalues span 1e-12..1."""
     from oracle.shampoo_oracle import eigh_inverse_root
 
     g = torch.Generator().manual_seed(9)

@@ -36,7 +36,7 @@ def test_soap_fixture_case_matches_reference():
     ref64 = ShampooOracle(ref64_p, oracle_config(c))
     # The 1-D blocks and the 8-column blocks of this case own rank-deficient factors for the first steps: the
     # basis the QR refresh returns for their null space is decided by rounding, in the reference as well.  The
-    # bound is therefore 1e-3 plus twice the reference algorithm's own fp32-vs-fp64 gap (see DESIGN.md).
+    # bound is therefore 1e-3 plus twice the reference algorithm's own fp32-vs-fp64 gap.
     worst_allow = 0.0
     for s, grads in grad_stream(c):
         for p, g in zip(params, grads):

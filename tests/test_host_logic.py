@@ -108,7 +108,7 @@ def test_partition_equals_oracle_blocks(shape, b):
 
 
 def test_baseline_block_tables():
-    """Block and factor counts of the BASELINE configs."""
+    """Block and factor counts of the five benchmark configurations."""
     gpt2 = sum(([(2304, 768), (768, 768), (3072, 768), (768, 3072), (768,), (768,)] for _ in range(12)), []) + [(50257, 768)]
     blocks = [s for i, sh in enumerate(gpt2) for s in partition_parameter(i, sh, 1024)]
     assert len(blocks) == 194

@@ -71,7 +71,7 @@ def test_config1_with_override_matches_reference():
 
 
 def test_config1_as_stated_raises_like_reference():
-    """BASELINE config 1 verbatim makes the reference raise PreconditionerValueError at
+    """benchmark configuration 1 verbatim makes the reference raise PreconditionerValueError at
     step 1 on the bias block's rank-1 factor; the oracle must fail the same way."""
     with open(os.path.join(GOLDEN, "cfg1_as_stated.json")) as f:
         rec = json.load(f)
