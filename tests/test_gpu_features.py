@@ -248,3 +248,37 @@ def test_large_ragged_kronecker_update_and_precondition():
             assert rel_err(st["shampoo"]["inv_factor_matrices"][j].cpu(), f) < 1e-3
     for q, r in zip(params, ref_p):
         assert rel_err(q.detach().cpu(), r) < 1e-4
+
+
+@pytest.mark.parametrize("kind", ["newton", "eigh", "soap_qr"])
+def test_zero_dimensional_empty_and_tiny_parameters(kind):
+    """The reference's distributor fixture (shampoo_distributor_test.py:24-341): 0-D, empty, 1-D and tiny 2-D
+    parameters in one group go through the same step."""
+    import optimizers_amd as oa
+    from oracle.shampoo_oracle import OracleConfig, ShampooOracle
+
+    g = torch.Generator().manual_seed(0)
+    shapes = [(), (0, 5), (7,), (6, 4), (1, 3)]
+    init = [torch.randn(s, generator=g) for s in shapes]
+    pc = {"newton": oa.RootInvShampooPreconditionerConfig(amortized_computation_config=oa.CoupledNewtonConfig()),
+          "eigh": oa.DefaultShampooConfig, "soap_qr": oa.DefaultSOAPConfig}[kind]
+    kw = dict(lr=1e-2, betas=(0.9, 0.99), epsilon=1e-4, max_preconditioner_dim=8, precondition_frequency=1,
+              start_preconditioning_step=2)
+    params = [torch.nn.Parameter(t.clone().to(DEV)) for t in init]
+    opt = oa.DistributedShampoo(params, preconditioner_config=pc,
+                                grafting_config=oa.AdamPreconditionerConfig(beta2=0.99, epsilon=1e-8), **kw)
+    ref_p = [t.clone() for t in init]
+    ref = ShampooOracle(ref_p, OracleConfig(preconditioner=kind, grafting="adam", grafting_beta2=0.99,
+                                            grafting_epsilon=1e-8, **kw))
+    for _ in range(4):
+        grads = [torch.randn(s, generator=g) for s in shapes]
+        for p, gr in zip(params, grads):
+            p.grad = gr.to(DEV)
+        opt.step()
+        ref.step([x.clone() for x in grads])
+    assert float(params[0].detach().cpu()) != float(init[0])  # the 0-D parameter is stepped
+    assert rel_err(params[0].detach().cpu().reshape(1), ref_p[0].reshape(1)) < 1e-6
+    assert params[1].numel() == 0
+    # the 1-D block's factor has rank one with epsilon = 1e-4: loose bound, the others are well conditioned
+    for p, r, tol in zip(params[2:], ref_p[2:], (5e-3, 1e-5, 1e-5)):
+        assert rel_err(p.detach().cpu(), r) < tol
