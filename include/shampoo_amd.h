@@ -128,14 +128,21 @@ int32_t sa_compute_root_inverses_newton(sa_plan* plan, float bias_correction2, f
                                         int32_t max_iterations, float tolerance,
                                         int32_t* iterations_out, int32_t* status_out, void* stream);
 
-/* Batched symmetric eigendecomposition root inverse on every factor (two-sided block Jacobi):
- * A = unpack(factor / bias_correction2) (+ epsilon I when perturb_before_computation), (lambda, Q) = eigh(A),
- * spectrum shifted as the reference does when min(lambda) < epsilon, X = Q diag(lambda^(-1/root)) Q^T
- * (matrix_functions.py:306-366, 698-770, 179-279 via shampoo_preconditioner_list.py:314-443, 631-680).
- * roots: host array, one (possibly fractional) root per factor.  sweeps_out / status_out as for the Newton call;
- * SA_FACTOR_NOT_CONVERGED means rotations were still being applied in sweep max_sweeps. */
+/* Batched symmetric eigendecomposition root inverse on every factor (solver: see sa_set_eigh_solver):
+ * A = unpack(factor / bias_correction2), (lambda, Q) = eigh(A), X = Q diag(w) Q^T
+ * (matrix_functions.py:179-279, 306-366, 698-770 via shampoo_preconditioner_list.py:314-443, 631-680).
+ * stability selects the reference's rank_deficient_stability_config:
+ *   0  PerturbationConfig(perturb_before_computation=False): lambda <- lambda - min(lambda_min, 0) + epsilon;
+ *   1  PerturbationConfig(perturb_before_computation=True): A + epsilon I is decomposed, and the spectrum is
+ *      shifted by -lambda_min + epsilon only if lambda_min < epsilon;
+ *   2  PseudoInverseConfig(rank_rtol, rank_atol): epsilon must be 0; w = 0 where
+ *      lambda <= max(rank_atol, rtol * max(lambda_max, 0)), rtol = rank_rtol or, for rank_rtol < 0 (the
+ *      reference's None), order * 2^-23.
+ * Otherwise w = lambda^(-1/root).  roots: host array, one (possibly fractional) root per factor.
+ * sweeps_out / status_out as for the Newton call; SA_FACTOR_NOT_CONVERGED means the solver gave up
+ * (Jacobi rotations still being applied in sweep max_sweeps, or the QL sweep budget of 30 per eigenvalue). */
 int32_t sa_compute_root_inverses_eigh(sa_plan* plan, float bias_correction2, float epsilon, const float* roots,
-                                      int32_t perturb_before_computation, int32_t max_sweeps,
+                                      int32_t stability, float rank_rtol, float rank_atol, int32_t max_sweeps,
                                       int32_t* sweeps_out, int32_t* status_out, void* stream);
 
 /* Eigenbasis refresh through a full symmetric eigendecomposition: the `EighEigendecompositionConfig` branch of

@@ -269,24 +269,38 @@ struct EigFinal {
   int scale_cols;      // eigenvectors are the columns of V: produce Vs (otherwise the caller scales rows)
 };
 
-// perturb_before != 0: epsilon was already added to the diagonal before the decomposition and the
-// spectrum is shifted only if its minimum is still below epsilon; otherwise (matrix_functions.py:265-271)
-// lambda <- (lambda - min(lambda_min, 0)) + epsilon unconditionally.
-__global__ __launch_bounds__(256) void eig_weights_kernel(const EigFinal* __restrict__ jobs, float eps, int perturb_before) {
-  __shared__ float red[4];
+// stability 1: epsilon was already added to the diagonal before the decomposition and the spectrum is shifted
+// only if its minimum is still below epsilon; stability 0 (matrix_functions.py:265-271):
+// lambda <- (lambda - min(lambda_min, 0)) + epsilon unconditionally; stability 2 (PseudoInverseConfig,
+// matrix_functions.py:206-249): eigenvalues at or below max(rank_atol, rtol * max(lambda_max, 0)) get weight 0,
+// rtol = rank_rtol, or d * 2^-23 when rank_rtol < 0 (the reference's None).
+__global__ __launch_bounds__(256) void eig_weights_kernel(const EigFinal* __restrict__ jobs, float eps, int stability,
+                                                         float rank_rtol, float rank_atol) {
+  __shared__ float red[4], redmax[4];
   const EigFinal& J = jobs[blockIdx.x];
   if (!J.enabled) return;
   const int d = J.d, dpad = J.dpad;
-  float m = 3.4028234663852886e38f;
-  for (int i = threadIdx.x; i < d; i += 256) m = fminf(m, J.lambda_in[i * J.lambda_stride]);
+  float m = 3.4028234663852886e38f, mx = -3.4028234663852886e38f;
+  for (int i = threadIdx.x; i < d; i += 256) {
+    const float l = J.lambda_in[i * J.lambda_stride];
+    m = fminf(m, l);
+    mx = fmaxf(mx, l);
+  }
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) m = fminf(m, __shfl_xor(m, o, 64));
+  for (int o = 32; o > 0; o >>= 1) {
+    m = fminf(m, __shfl_xor(m, o, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+  }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  if (lane == 0) red[wave] = m;
+  if (lane == 0) { red[wave] = m; redmax[wave] = mx; }
   __syncthreads();
   const float lam_min = fminf(fminf(red[0], red[1]), fminf(red[2], red[3]));
-  const bool shift = perturb_before ? (lam_min < eps) : true;
-  const float first = perturb_before ? -lam_min : -fminf(lam_min, 0.0f);
+  const float lam_max = fmaxf(fmaxf(redmax[0], redmax[1]), fmaxf(redmax[2], redmax[3]));
+  const bool pinv = stability == 2;
+  const bool shift = pinv ? false : (stability == 1 ? (lam_min < eps) : true);
+  const float first = (stability == 1) ? -lam_min : -fminf(lam_min, 0.0f);
+  const float rtol = (rank_rtol < 0.0f) ? (float)d * 1.1920929e-7f : rank_rtol;
+  const float cutoff = fmaxf(rtol * fmaxf(lam_max, 0.0f), rank_atol);
   for (int i = threadIdx.x; i < dpad; i += 256) {
     float lam = 0.0f, wgt = 0.0f;
     if (i < d) {
@@ -295,7 +309,7 @@ __global__ __launch_bounds__(256) void eig_weights_kernel(const EigFinal* __rest
         if (first != 0.0f) lam = lam + first;
         if (eps != 0.0f) lam = lam + eps;
       }
-      wgt = powf(lam, J.exponent);
+      wgt = (pinv && lam <= cutoff) ? 0.0f : powf(lam, J.exponent);
     }
     J.lambda_out[i] = lam;
     J.weight_out[i] = wgt;

@@ -1544,7 +1544,7 @@ static int eigh_solve(sa_plan* p, const std::vector<int>& todo, const std::vecto
 }
 
 int32_t sa_compute_root_inverses_eigh(sa_plan* p, float bias_correction2, float epsilon, const float* roots,
-                                      int32_t perturb_before_computation, int32_t max_sweeps, int32_t* sweeps_out,
+                                      int32_t stability, float rank_rtol, float rank_atol, int32_t max_sweeps, int32_t* sweeps_out,
                                       int32_t* status_out, void* stream) {
   if (!p || !roots || !sweeps_out || !status_out) return fail(SA_ERR_INVALID, "sa_compute_root_inverses_eigh: NULL argument");
   if (!(bias_correction2 != 0.0f) || max_sweeps < 1) return fail(SA_ERR_INVALID, "bad bias correction or max_sweeps");
@@ -1554,7 +1554,10 @@ int32_t sa_compute_root_inverses_eigh(sa_plan* p, float bias_correction2, float 
   if (F == 0) return SA_OK;
   for (int i = 0; i < F; ++i)
     if (!(roots[i] > 0.0f)) return fail(SA_ERR_INVALID, "Root " + std::to_string(roots[i]) + " should be positive!");
-  const float ridge = perturb_before_computation ? epsilon : 0.0f;
+  if (stability < 0 || stability > 2) return fail(SA_ERR_INVALID, "stability must be 0, 1 or 2");
+  if (stability == 2 && epsilon != 0.0f)
+    return fail(SA_ERR_INVALID, "epsilon=" + std::to_string(epsilon) + " should be 0.0 when using pseudo-inverse!");
+  const float ridge = (stability == 1) ? epsilon : 0.0f;
   std::vector<int> todo;
   SACHECK(root_inverse_prologue(p, bias_correction2, ridge, sweeps_out, status_out, s, &todo));
   if (todo.empty()) return SA_OK;
@@ -1629,7 +1632,7 @@ int32_t sa_compute_root_inverses_eigh(sa_plan* p, float bias_correction2, float 
   SACHECK(p->t_rowscale.upload(s));
   SACHECK(p->eig_gemm.commit(s));
   SACHECK(p->eig_gemm_t.commit(s));
-  hipLaunchKernelGGL(eig_weights_kernel, dim3(n), dim3(256), 0, s, p->t_eigfinal.dev, epsilon, perturb_before_computation ? 1 : 0);
+  hipLaunchKernelGGL(eig_weights_kernel, dim3(n), dim3(256), 0, s, p->t_eigfinal.dev, epsilon, stability, rank_rtol, rank_atol);
   hipLaunchKernelGGL(eig_scale_cols_kernel, dim3(slabs), dim3(256), 0, s, p->t_eigfinal.dev, n);
   if (n_t) hipLaunchKernelGGL(eig_scale_rows_kernel, dim3(slabs_t), dim3(256), 0, s, p->t_rowscale.dev, n_t);
   HIPCHECK(hipGetLastError());

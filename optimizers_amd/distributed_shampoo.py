@@ -333,7 +333,7 @@ class _NativeGroup:
             if pc.factor_matrix_eigenvectors_dtype != torch.float32 or pc.corrected_eigenvalues_dtype != torch.float32:
                 raise NotImplementedError("eigenvectors and corrected eigenvalues are fp32 in the native step")
         elif isinstance(acc, EigenConfig):
-            if not isinstance(acc.rank_deficient_stability_config, PerturbationConfig):
+            if not isinstance(acc.rank_deficient_stability_config, (PerturbationConfig, PseudoInverseConfig)):
                 raise NotImplementedError(f"{acc.rank_deficient_stability_config=} is not supported.")
             if acc.eigendecomposition_offload_device != "":
                 raise NotImplementedError("eigendecomposition_offload_device: the decomposition runs on the MI355X")
@@ -524,10 +524,15 @@ class _NativeGroup:
             )
         elif self.use_eigh:
             roots = (ctypes.c_float * max(self.n_factors, 1))(*self.factor_roots)
+            stab = cfg.rank_deficient_stability_config
+            if isinstance(stab, PseudoInverseConfig):
+                # rank_rtol=None is the reference's "order * machine epsilon" (matrix_functions.py:226-229)
+                mode, rtol, atol = 2, (-1.0 if stab.rank_rtol is None else float(stab.rank_rtol)), float(stab.rank_atol)
+            else:
+                mode, rtol, atol = int(stab.perturb_before_computation), 0.0, 0.0
             native.check(
                 self.lib.sa_compute_root_inverses_eigh(
-                    self.plan, bc2, group[EPSILON], roots,
-                    int(cfg.rank_deficient_stability_config.perturb_before_computation), self.max_jacobi_sweeps,
+                    self.plan, bc2, group[EPSILON], roots, mode, rtol, atol, self.max_jacobi_sweeps,
                     self.iterations, self.status, stream,
                 ),
                 "sa_compute_root_inverses_eigh",

@@ -106,7 +106,8 @@ def load() -> ctypes.CDLL:
         c_void_p, c_float, c_float, c_int32, c_float, POINTER(c_int32), POINTER(c_int32), c_void_p,
     ]
     lib.sa_compute_root_inverses_eigh.argtypes = [
-        c_void_p, c_float, c_float, POINTER(c_float), c_int32, c_int32, POINTER(c_int32), POINTER(c_int32), c_void_p,
+        c_void_p, c_float, c_float, POINTER(c_float), c_int32, c_float, c_float, c_int32, POINTER(c_int32), POINTER(c_int32),
+        c_void_p,
     ]
     lib.sa_refresh_eigenbases_qr.argtypes = [
         c_void_p, c_float, c_float, c_int32, c_float, POINTER(c_int32), POINTER(c_int32), c_void_p,

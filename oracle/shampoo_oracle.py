@@ -197,6 +197,21 @@ def eigh_inverse_root(a: Tensor, root: float, eps: float = 0.0) -> Tensor:
     return q * lam.pow(-1.0 / root).unsqueeze(0) @ q.T
 
 
+def eigh_pseudo_inverse_root(
+    a: Tensor, root: float, rank_rtol: float | None = None, rank_atol: float = 0.0
+) -> Tensor:
+    """matrix_functions.py:206-249 (PseudoInverseConfig, epsilon = 0): eigenvalues at or
+    below max(rank_atol, rtol * relu(lambda_max)) get weight zero, rtol = rank_rtol or
+    n * machine epsilon; the others lambda^(-1/root).
+    Pinned by numpy.linalg.pinv (root 1, same cutoff) and closed forms on projectors.
+    """
+    lam, q = torch.linalg.eigh(a)
+    rtol = lam.numel() * torch.finfo(lam.dtype).eps if rank_rtol is None else rank_rtol
+    cutoff = torch.clamp(rtol * lam.max().relu(), min=rank_atol)
+    w = torch.where(lam <= cutoff, torch.zeros_like(lam), lam.pow(-1.0 / root))
+    return q * w.unsqueeze(0) @ q.T
+
+
 def qr_refresh(
     a: Tensor, q_prev: Tensor, eps: float = 0.0, max_iterations: int = 1, tolerance: float = 0.0
 ) -> tuple[Tensor, Tensor]:

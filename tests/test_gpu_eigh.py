@@ -209,3 +209,29 @@ def test_eigenvectors_diagonalise_the_factor(m, n, eigh_solver):
         assert float(torch.linalg.norm(off) / torch.linalg.norm(A)) < 1e-5, (j, eigh_solver)
         lam = torch.diagonal(B)
         assert bool((lam[1:] >= lam[:-1] - 1e-5 * lam.abs().max()).all())
+
+
+@pytest.mark.parametrize("eigh_solver", [1, 2], indirect=True)
+@pytest.mark.parametrize("m, n", [(96, 40), (600, 260)])
+def test_pseudo_inverse_root_of_rank_deficient_factors(m, n, eigh_solver):
+    """EigenConfig(rank_deficient_stability_config=PseudoInverseConfig(rank_rtol=None)), epsilon = 0: eigenvalues
+    below order x machine epsilon x lambda_max, i.e. the null space of the rank-n factor G G^T, get weight zero
+    (matrix_functions.py:206-249).  (The default rank_rtol = 0 only drops eigenvalues <= 0.)"""
+    import optimizers_amd as oa
+    from oracle.shampoo_oracle import eigh_pseudo_inverse_root, pack_triu
+
+    g = torch.Generator().manual_seed(m * n)
+    G = torch.randn(m, n, generator=g)
+    p = torch.nn.Parameter(torch.zeros(m, n, device=DEV))
+    pc = oa.RootInvShampooPreconditionerConfig(
+        amortized_computation_config=oa.EigenConfig(rank_deficient_stability_config=oa.PseudoInverseConfig(rank_rtol=None)))
+    opt = oa.DistributedShampoo([p], lr=0.01, betas=(0.0, 1.0), epsilon=0.0, max_preconditioner_dim=max(m, n),
+                                precondition_frequency=1, start_preconditioning_step=1, use_bias_correction=False,
+                                preconditioner_config=pc)
+    p.grad = G.to(DEV)
+    opt.step()
+    st = opt.state[p]["block_0"]["shampoo"]
+    for j, A64 in enumerate([G.double() @ G.double().T, G.double().T @ G.double()]):
+        got = st["inv_factor_matrices"][j].cpu()
+        want = pack_triu(eigh_pseudo_inverse_root(A64, 4, rank_rtol=A64.shape[0] * 1.1920929e-7).float())
+        assert rel_err(got, want) < 1e-3, (j, rel_err(got, want))

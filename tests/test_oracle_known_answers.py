@@ -215,3 +215,29 @@ def test_ema_factor_is_gram_ema_and_uses_raw_gradient():
         opt.step([g])
     torch.testing.assert_close(opt.state[0]["factors"][0], L, rtol=1e-5, atol=1e-7)
     torch.testing.assert_close(opt.state[0]["factors"][1], R, rtol=1e-5, atol=1e-7)
+
+
+def test_pseudo_inverse_root_matches_numpy_pinv_and_projector_closed_form():
+    """PseudoInverseConfig branch (matrix_functions.py:206-249).  Root 1 is the Moore-Penrose inverse: numpy's
+    pinv with the same relative cutoff must agree; for a scaled projector c P the root-r result is c^(-1/r) P."""
+    import numpy as np
+
+    g = torch.Generator().manual_seed(5)
+    B = torch.randn(12, 5, generator=g, dtype=torch.float64)
+    A = B @ B.T  # rank 5 of 12
+    X = O.eigh_pseudo_inverse_root(A, 1)
+    want = torch.from_numpy(np.linalg.pinv(A.numpy(), rcond=12 * torch.finfo(torch.float64).eps, hermitian=True))
+    torch.testing.assert_close(X, want, atol=1e-10, rtol=1e-8)
+    # the null space stays a null space for every root
+    lam, q = torch.linalg.eigh(A)
+    null = q[:, :7]
+    for root in (2, 4):
+        Xr = O.eigh_pseudo_inverse_root(A, root)
+        assert float((Xr @ null).abs().max()) < 1e-10
+    Q, _ = torch.linalg.qr(torch.randn(9, 3, generator=g, dtype=torch.float64))
+    P = Q @ Q.T
+    torch.testing.assert_close(O.eigh_pseudo_inverse_root(16.0 * P, 4), 0.5 * P, atol=1e-12, rtol=1e-10)
+    # absolute tolerance: everything at or below rank_atol is dropped
+    D = torch.diag(torch.tensor([4.0, 1.0, 0.25], dtype=torch.float64))
+    torch.testing.assert_close(O.eigh_pseudo_inverse_root(D, 2, rank_rtol=0.0, rank_atol=0.25),
+                               torch.diag(torch.tensor([0.5, 1.0, 0.0], dtype=torch.float64)))
