@@ -65,7 +65,9 @@ typedef struct sa_block_desc {
   int32_t root[2];        /* integer inverse root (4 for matrices, 2 for vectors by default) */
   /* eigenvalue-corrected Shampoo / SOAP (shampoo_preconditioner_list.py:942-1007): dense d x d eigenbasis of
    * each factor (row-major, columns are eigenvectors) and the second moment kept in the rotated basis
-   * (rows x cols, contiguous).  NULL for root-inverse Shampoo. */
+   * (rows x cols, contiguous).  NULL for root-inverse Shampoo.  eigenvectors[k] with factor[k] == NULL is a
+   * fixed basis: it rotates the block but has no statistics and is never refreshed (a block whose basis
+   * changes are all ignored, ignored_basis_change_dims, passes one identity matrix). */
   float* eigenvectors[2];
   float* corrected_eigenvalues;
 } sa_block_desc;

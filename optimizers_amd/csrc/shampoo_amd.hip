@@ -340,7 +340,9 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
     if (mode == 0) { B.ghat_src = B.grad; B.ghat_ld = d.ld; }
     else if (mode == 1) { B.ghat_src = d.filtered_grad; B.ghat_ld = d.cols; }
     else { B.ghat_src = ghbuf(p) + eo; B.ghat_ld = d.cols; }
-    const bool precond = p->block_factor[0][b] >= 0 || p->block_factor[1][b] >= 0;
+    // a block is preconditioned if a side has a Kronecker factor or, for eigenvalue-corrected Shampoo, a fixed basis
+    const bool precond = p->block_factor[0][b] >= 0 || p->block_factor[1][b] >= 0 ||
+                         (d.corrected_eigenvalues && (d.eigenvectors[0] || d.eigenvectors[1]));
     B.p_is_ghat = precond ? 0 : 1;
     if (precond) { B.p_src = pbuf(p) + eo; B.p_ld = d.cols; }
     else { B.p_src = B.ghat_src; B.p_ld = B.ghat_ld; }
@@ -405,12 +407,14 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
     for (int b : active) {
       const sa_block_desc& d = p->blocks[b];
       const BlockDev& B = p->t_blocks.host[b];
-      const int f0 = p->block_factor[0][b], f1 = p->block_factor[1][b];
-      if (f0 < 0 && f1 < 0) continue;
+      // eigenvectors[side] without factor[side] is a fixed basis: it rotates, but has no statistics and is never
+      // refreshed (an ignored basis change, shampoo_preconditioner_list.py:1843-1865, passes the identity)
+      const float* QL = d.eigenvectors[0];
+      const float* QR = d.eigenvectors[1];
+      const int f0 = QL ? 0 : -1, f1 = QR ? 0 : -1;
+      if (!d.corrected_eigenvalues || (f0 < 0 && f1 < 0)) continue;
       const long long eo = p->elem_off[b];
       float* part = p->f(p->off_ptile_partial) + p->ptile_begin_all[b];
-      const float* QL = f0 >= 0 ? p->factors[f0].eigvec : nullptr;
-      const float* QR = f1 >= 0 ? p->factors[f1].eigvec : nullptr;
       const float* G = p->grads[b];
       auto mk = [&](const float* A, long long lda, const float* Bm, long long ldb, float* C, float* C2, int K) {
         GemmProblem q{};
@@ -615,7 +619,10 @@ int32_t sa_plan_create(const sa_block_desc* blocks, int32_t n_blocks, sa_plan** 
     p->ptile_begin_all[b] = ptiles;
     ptiles += ((d.rows + BM - 1) / BM) * ((d.cols + BN - 1) / BN);
     for (int side = 0; side < 2; ++side) {
-      if (!d.factor[side]) continue;
+      if (!d.factor[side]) {
+        if (d.eigenvectors[side] && d.corrected_eigenvalues) p->eigenvalue_corrected = true;  // fixed basis
+        continue;
+      }
       if ((!d.inv_factor[side] && !d.eigenvectors[side]) || (d.inv_factor[side] && d.root[side] < 1)) {
         delete p;
         return fail(SA_ERR_INVALID, "sa_plan_create: factor without inverse / eigenvector storage or with root < 1");

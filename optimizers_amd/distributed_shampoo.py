@@ -165,8 +165,6 @@ class _NativeGroup:
                 sel = tuple(d not in ignored for d in range(order))
                 self.selectors.append(sel)
                 self.roots.append((1 / pc.inverse_exponent_override.get(order, 1 / 2),) * sum(sel))
-                if not any(sel):
-                    raise NotImplementedError("a block with every basis change ignored is not built natively")
             else:
                 exps = [self._inverse_exponent(pc, d, order) for d in range(order)]
                 self.selectors.append(tuple(e != 0.0 for e in exps))
@@ -220,6 +218,12 @@ class _NativeGroup:
                 shampoo_state["corrected_eigenvalues"] = self.corrected_arena.view(k, s.shape)
                 d.corrected_eigenvalues = shampoo_state["corrected_eigenvalues"].data_ptr()
                 self._slots.append((p, s.block_key, (SHAMPOO, "corrected_eigenvalues"), shampoo_state["corrected_eigenvalues"]))
+            if self.soap and not any(self.selectors[k]):
+                # every basis change ignored: the block is preconditioned in the standard basis (this is Adam /
+                # RMSprop on the block, shampoo_eigenvalue_correction_test.py:60-272); the native step rotates
+                # by one identity matrix on the smaller dim, which is exact
+                dim = min(range(s.order), key=lambda t: s.shape[t])
+                d.eigenvectors[dim] = self._identity(s.shape[dim]).data_ptr()
             slot = 0
             for dim in range(s.order):
                 if not self.selectors[k][dim]:
@@ -306,6 +310,12 @@ class _NativeGroup:
         for p in params:
             optimizer.state[p][STEP] = self.step_tensor
         self.stream: torch.cuda.Stream | None = None
+
+    def _identity(self, n: int) -> torch.Tensor:
+        cache = self.__dict__.setdefault("_identities", {})
+        if n not in cache:
+            cache[n] = torch.eye(n, device=self.device, dtype=torch.float32)
+        return cache[n]
 
     def close(self) -> None:
         if self.plan:

@@ -144,3 +144,34 @@ def test_eigh_refresh_tolerance_keeps_a_good_enough_basis():
         lam = torch.diagonal(q.T @ a @ q)
         assert bool((lam[1:] >= lam[:-1] - 1e-4 * lam.abs().max()).all())  # ascending, like torch.linalg.eigh
         assert rel_err(q @ torch.diag(lam) @ q.T, a) < 1e-4
+
+
+@pytest.mark.parametrize("weight_decay", [0.0, 0.1])
+def test_all_basis_changes_ignored_is_adam(weight_decay):
+    """shampoo_eigenvalue_correction_test.py:60-272: eigenvalue-corrected Shampoo whose basis changes are all
+    ignored preconditions in the standard basis, i.e. it is Adam (AdamW with decoupled weight decay)."""
+    import optimizers_amd as oa
+
+    g = torch.Generator().manual_seed(11)
+    shapes = [(24, 16), (16,), (5, 40)]
+    init = [torch.randn(s, generator=g) for s in shapes]
+    params = [torch.nn.Parameter(t.clone().to(DEV)) for t in init]
+    cfg = oa.EigenvalueCorrectedShampooPreconditionerConfig(ignored_basis_change_dims={1: [0], 2: [0, 1]})
+    opt = oa.DistributedShampoo(params, lr=1e-2, betas=(0.9, 0.999), epsilon=1e-8, weight_decay=weight_decay,
+                                max_preconditioner_dim=16, precondition_frequency=1, start_preconditioning_step=1,
+                                use_bias_correction=True, preconditioner_config=cfg, grafting_config=None)
+    ref_p = [torch.nn.Parameter(t.clone()) for t in init]
+    ref = (torch.optim.AdamW(ref_p, lr=1e-2, betas=(0.9, 0.999), eps=1e-8, weight_decay=weight_decay)
+           if weight_decay else torch.optim.Adam(ref_p, lr=1e-2, betas=(0.9, 0.999), eps=1e-8))
+    for _ in range(5):
+        grads = [torch.randn(s, generator=g) for s in shapes]
+        for p, r, gr in zip(params, ref_p, grads):
+            p.grad = gr.to(DEV)
+            r.grad = gr.clone()
+        opt.step()
+        ref.step()
+    for p, r in zip(params, ref_p):
+        assert rel_err(p.detach().cpu(), r.detach()) < 1e-5
+    # no Kronecker factors and no eigenbases are kept for ignored dims
+    st = opt.state[params[0]]["block_0"]["shampoo"]
+    assert len(st["factor_matrices"]) == 0 and len(st["factor_matrices_eigenvectors"]) == 0
