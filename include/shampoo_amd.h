@@ -38,6 +38,9 @@ extern "C" {
 #define SA_FACTOR_RESULT_NONFINITE 2 /* inverse root holds nan/inf        (shampoo_preconditioner_list.py:405) */
 #define SA_FACTOR_NOT_CONVERGED 3    /* max_iterations reached; result kept (matrix_functions.py:678-681) */
 #define SA_FACTOR_SKIPPED 4          /* follows a non-finite factor; not computed, state untouched */
+#define SA_FACTOR_SOLVER_FAILED 5    /* the solver gave up where the reference raises inside matrix_inverse_root
+                                        (matrix_functions.py:543, 629, 655); the stored inverse is untouched and the
+                                        caller counts the failure (shampoo_preconditioner_list.py:388-443) */
 
 /* Grafting flavours (distributed_shampoo.py:673-714). */
 #define SA_GRAFT_NONE 0
@@ -129,6 +132,19 @@ int32_t sa_update_factor_matrices(sa_plan* plan, float beta2, float weighting_fa
 int32_t sa_compute_root_inverses_newton(sa_plan* plan, float bias_correction2, float epsilon,
                                         int32_t max_iterations, float tolerance,
                                         int32_t* iterations_out, int32_t* status_out, void* stream);
+
+/* Batched coupled higher-order iteration on every factor (CoupledHigherOrderConfig; matrix_functions.py:439-661 via
+ * :682-689): A = unpack(factor / bias_correction2), A_r = A + max(rel_epsilon * |A|_inf, abs_epsilon) I,
+ * z = 1 / trace(A_r); one plain Newton step, then steps with M_p = sum_{i < order} b_i (I - M)^i until the error
+ * max|M - I| is at most `tolerance`, max_iterations is reached, or the error grows by more than 1.2 x or repeats
+ * itself below 1e-3 (the update of that step stays).  A factor whose result has |A_r X^p - I|_max > 0.1 or holds
+ * nan/inf gets SA_FACTOR_SOLVER_FAILED and keeps its stored inverse; the optimizer's epsilon plays no part, as in
+ * the reference.  Orders 2..8; roots as for the Newton call (the root's denominator must be 1).
+ * iterations_out / status_out as for the Newton call; the call synchronises the stream before it returns. */
+int32_t sa_compute_root_inverses_higher_order(sa_plan* plan, float bias_correction2, float rel_epsilon,
+                                              float abs_epsilon, int32_t max_iterations, float tolerance,
+                                              int32_t order, int32_t* iterations_out, int32_t* status_out,
+                                              void* stream);
 
 /* Batched symmetric eigendecomposition root inverse on every factor (solver: see sa_set_eigh_solver):
  * A = unpack(factor / bias_correction2), (lambda, Q) = eigh(A), X = Q diag(w) Q^T
@@ -238,6 +254,13 @@ int32_t sa_set_symmetric_newton(int32_t policy);
  *   2  tridiagonalisation for every factor whose padded order is at least 256.
  * Process wide.  No counterpart in the reference. */
 int32_t sa_set_eigh_solver(int32_t solver);
+
+/* Trace scaling (use_trace_scaling / trace_scaling_exponent, shampoo_preconditioner_list.py:366-371): when
+ * enabled, every root-inverse and eigenbasis computation of this plan works on
+ *   (factor / bias_correction2) * max(trace(factor / bias_correction2), floor) ^ (-exponent)
+ * instead of factor / bias_correction2; `floor` is the optimizer's epsilon.  The multiplier is evaluated on the
+ * device, one per factor, in front of the finiteness check of the input.  Off by default. */
+int32_t sa_plan_set_trace_scaling(sa_plan* plan, int32_t enabled, float exponent, float floor);
 
 #ifdef __cplusplus
 }

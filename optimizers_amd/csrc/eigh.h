@@ -393,6 +393,7 @@ __global__ __launch_bounds__(256) void rows_to_sorted_cols_kernel(const RowsToCo
 // dense <- packed / bc2 (+ eps on the diagonal), V <- I : start of an eigendecomposition.
 struct EigInit {
   const float* packed;
+  const float* scale;  // optional per-factor multiplier applied after the division by bc2 (trace scaling)
   float* A;
   float* V;
   int d, dpad;
@@ -419,6 +420,7 @@ __global__ __launch_bounds__(256) void eig_init_kernel(const EigInit* __restrict
     if (r < d && c < d) {
       const int rs = min(r, c), cs = max(r, c);
       v = J.packed[(long long)rs * d - ((long long)rs * (rs - 1)) / 2 + (cs - rs)] / bc2;
+      if (J.scale != nullptr) v = v * J.scale[0];
       if (r == c && eps != 0.0f) v = v + eps;
     }
     J.A[(long long)r * dpad + c] = v;

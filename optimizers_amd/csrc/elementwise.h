@@ -385,6 +385,7 @@ struct SymFactor {
   float* dense_out[3];     // dense destinations
   unsigned int* err_bits;
   const float* norm_partial;  // Newton init: per-chunk partial sums of squares
+  const float* scale;      // Newton init: optional per-factor multiplier applied after the division by bc2
   int n_norm_partial;
   int d, dpad;
   int tile_begin;          // first tile-pair id
@@ -455,6 +456,7 @@ __global__ __launch_bounds__(256) void sym_pass_kernel(const SymFactor* __restri
         v = F.packed_in[packed_off(rs, cs, d)];
         if (MODE == SYM_NEWTON_INIT) {
           v = v / bc2;
+          if (F.scale != nullptr) v = v * F.scale[0];
           if (r == c && eps != 0.0f) v = v + eps;
         }
       }
@@ -505,6 +507,7 @@ __global__ __launch_bounds__(256) void sym_pass_kernel(const SymFactor* __restri
 struct NormJob {
   const float* src;     // packed factor, or dense matrix when dense != 0
   float* partial;       // n_chunks partial sums
+  float* scale;         // optional per-factor multiplier applied after the division by bc2 (trace scaling)
   int* nonfinite;       // set to 1 when a non-finite value is seen
   int d, dpad, dense;
   int chunk_begin;      // first workgroup id of this job
@@ -554,6 +557,7 @@ __global__ __launch_bounds__(256) void factor_norm_kernel(const NormJob* __restr
       while (r + 1 < d && packed_off(r + 1, r + 1, d) <= e) ++r;
       const bool diag = (packed_off(r, r, d) == e);
       float v = J.src[e] / bc2;
+      if (J.scale != nullptr) v = v * J.scale[0];
       if (!(fabsf(v) <= 3.4028234663852886e38f)) bad = true;
       if (diag && eps != 0.0f) v = v + eps;
       acc += diag ? v * v : 2.0f * (v * v);
@@ -563,6 +567,153 @@ __global__ __launch_bounds__(256) void factor_norm_kernel(const NormJob* __restr
   if (!CHECK_ONLY) {
     const float s = block_sum(acc, red);
     if (threadIdx.x == 0) J.partial[chunk] = s;
+  }
+}
+
+// Trace scaling: scale = max(trace(factor / bc2), floor) ^ (-exponent), one workgroup per job
+// (reference: shampoo_preconditioner_list.py:366-371).
+__global__ __launch_bounds__(256) void trace_scale_kernel(const NormJob* __restrict__ jobs, float bc2, float floor,
+                                                         float exponent) {
+  __shared__ float red[4];
+  const NormJob& J = jobs[blockIdx.x];
+  if (!J.enabled || J.scale == nullptr) return;
+  const int d = J.d;
+  float acc = 0.f;
+  for (int i = threadIdx.x; i < d; i += 256) acc += J.src[packed_off(i, i, d)] / bc2;
+  const float trace = block_sum(acc, red);
+  // a NaN trace stays NaN (like torch.clamp), so the finiteness check that follows sees it
+  if (threadIdx.x == 0) J.scale[0] = powf(trace != trace ? trace : fmaxf(trace, floor), -exponent);
+}
+
+// ---- start of the coupled higher-order iteration (reference: matrix_functions.py:528-572) ---------------
+// The bias-corrected factor sits dense (dpad-strided, zero padded) in A.
+struct HoJob {
+  float* A;         // dense factor; becomes M = z (A + eps I)
+  float* Mp;        // M_p of the first (plain Newton) step: M * s + (1 - s) I
+  float* X;         // z^(1/root) I
+  float* rowsum;    // d absolute row sums
+  float* params;    // [0] z = 1 / trace(A + eps I), [1] eps = max(rel * |A|_inf, abs), [2] |A|_inf
+  int d, dpad;
+};
+
+// grid (ceil(max d / 4), jobs): one wavefront per row
+__global__ __launch_bounds__(256) void ho_rowsum_kernel(const HoJob* __restrict__ jobs) {
+  const HoJob& J = jobs[blockIdx.y];
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (row >= J.d) return;
+  const float* __restrict__ a = J.A + (long long)row * J.dpad;
+  float acc = 0.f;
+  for (int c = lane; c < J.d; c += 64) acc += fabsf(a[c]);
+  acc = wave_sum(acc);
+  if (lane == 0) J.rowsum[row] = acc;
+}
+
+// one workgroup per job
+__global__ __launch_bounds__(256) void ho_setup_kernel(const HoJob* __restrict__ jobs, float rel_eps, float abs_eps) {
+  __shared__ float red[4];
+  __shared__ float eps_sh;
+  const HoJob& J = jobs[blockIdx.x];
+  float mx = 0.f;
+  bool nan = false;
+  for (int i = threadIdx.x; i < J.d; i += 256) {
+    const float v = J.rowsum[i];
+    if (v != v) nan = true;
+    mx = fmaxf(mx, v);
+  }
+  if (nan) mx = __builtin_nanf("");
+  mx = wave_max_nan(mx);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float m = red[0];
+    for (int w = 1; w < 4; ++w) m = (m != m || red[w] != red[w]) ? __builtin_nanf("") : fmaxf(m, red[w]);
+    const float scaled = m * rel_eps;
+    eps_sh = scaled != scaled ? scaled : fmaxf(scaled, abs_eps);  // torch.clamp(min=...) keeps a NaN
+    J.params[1] = eps_sh;
+    J.params[2] = m;
+  }
+  __syncthreads();
+  const float eps = eps_sh;
+  float acc = 0.f;
+  for (int i = threadIdx.x; i < J.d; i += 256) acc += J.A[(long long)i * J.dpad + i] + eps;
+  const float trace = block_sum(acc, red);
+  if (threadIdx.x == 0) J.params[0] = 1.0f / trace;
+}
+
+// grid (ceil(max dpad^2 / 1024), jobs); ridge_only: A <- A + eps I and nothing else
+__global__ __launch_bounds__(256) void ho_start_kernel(const HoJob* __restrict__ jobs, int root, int ridge_only) {
+  const HoJob& J = jobs[blockIdx.y];
+  const long long total = (long long)J.dpad * J.dpad;
+  const long long e0 = ((long long)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (e0 >= total) return;
+  const float z = ridge_only ? 1.0f : J.params[0], eps = J.params[1];
+  const float s = -1.0f / (float)root, one_minus_s = 1.0f - (-1.0f / (float)root);
+  const float x0 = ridge_only ? 0.f : powf(z, 1.0f / (float)root);
+  const int r = (int)(e0 / J.dpad), c0 = (int)(e0 % J.dpad);  // dpad is a multiple of 4: one row per thread
+  float4 a = *reinterpret_cast<const float4*>(J.A + e0);
+  float av[4] = {a.x, a.y, a.z, a.w}, mv[4], pv[4], xv[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const bool diag = (c0 + k == r) && r < J.d;
+    float v = av[k];
+    if (diag) v = v + eps;
+    const float m = ridge_only ? v : z * v;
+    mv[k] = m;
+    float mp = __fmul_rn(m, s);
+    if (diag) mp = __fadd_rn(mp, one_minus_s);
+    pv[k] = mp;
+    xv[k] = diag ? x0 : 0.f;
+  }
+  *reinterpret_cast<float4*>(J.A + e0) = make_float4(mv[0], mv[1], mv[2], mv[3]);
+  if (!ridge_only) {
+    *reinterpret_cast<float4*>(J.Mp + e0) = make_float4(pv[0], pv[1], pv[2], pv[3]);
+    *reinterpret_cast<float4*>(J.X + e0) = make_float4(xv[0], xv[1], xv[2], xv[3]);
+  }
+}
+
+// Loop control of the higher-order iteration (matrix_functions.py:574-619), one thread per factor.  `call` counts
+// the evaluations: 0 follows the start (the first step always runs), 1 follows that step (its error becomes the
+// reference error), later calls compare the new error with the kept one: more than 1.2 x, or equal below 1e-3,
+// ends the loop with the last update in place.  flag: 0 converged, 1 iteration limit, 2 early stop.
+struct HigherOrderCtl {
+  unsigned int* err_bits;
+  int* active;
+  int* iterations;
+  int* final_parity;
+  float* final_err;
+  float* kept_err;
+  int* flag;
+};
+
+__global__ void higher_order_control_kernel(HigherOrderCtl c, const int* __restrict__ ids, int n, float tol, int max_iter,
+                                            int call, int cur_parity) {
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const int f = ids[i];
+    if (!c.active[f]) continue;
+    const float fresh = __uint_as_float(c.err_bits[f]);
+    c.err_bits[f] = 0u;
+    bool go;
+    int flag = 0;
+    if (call == 0) {
+      go = true;
+    } else {
+      float err = c.kept_err[f];
+      bool early = false;
+      if (call == 1) err = fresh;
+      else if (fresh > err * 1.2f || (fresh == err && err < 1e-3f)) early = true;
+      else err = fresh;
+      c.kept_err[f] = err;
+      go = !early && (err > tol) && (c.iterations[f] < max_iter);
+      flag = early ? 2 : ((err > tol) ? 1 : 0);
+    }
+    if (go) {
+      c.iterations[f] += 1;
+    } else {
+      c.active[f] = 0;
+      c.final_parity[f] = cur_parity;
+      c.final_err[f] = c.kept_err[f];
+      c.flag[f] = flag;
+    }
   }
 }
 

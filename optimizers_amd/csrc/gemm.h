@@ -44,13 +44,14 @@ enum Epilogue {
   EPI_SQ_EMA = 4,       // C = beta*C + alpha*acc^2        (second moment in the eigenbasis)
   EPI_DIVPOW = 5,       // C = acc / ((C2 / div)^pow_exp + eps)   (C2 has the layout of C)
   EPI_SUB = 6,          // C -= acc                         (block-reflector updates of the QR refresh)
+  EPI_HORNER = 7,       // C = alpha*acc + beta*C2 + mp_diag*I over d x d (C2 read only; Horner step of a matrix polynomial)
 };
 
 struct GemmProblem {
   const float* A;
   const float* B;
   float* C;
-  float* C2;               // EPI_NEWTON_M: M_p output.  EPI_STORE_SQNORM: per-tile partial sums
+  float* C2;               // EPI_NEWTON_M: M_p output.  EPI_STORE_SQNORM: per-tile partial sums.  EPI_HORNER: addend (read)
   unsigned int* err_bits;  // EPI_NEWTON_M: atomicMax target (bit pattern of a non-negative float)
   const int* active;       // optional: skip the problem when *active == 0
   long long lda, ldb, ldc;
@@ -64,7 +65,7 @@ struct GemmProblem {
 // Scalars shared by every problem of one launch.
 struct GemmScalars {
   float a_div, b_div;      // operand is divided by this on load (1.0f = as stored)
-  float alpha, beta;       // EPI_SYRK_EMA: C = beta*C + alpha*acc
+  float alpha, beta;       // EPI_SYRK_EMA: C = beta*C + alpha*acc.  EPI_HORNER: C = alpha*acc + beta*C2 + mp_diag*I
   float mp_scale, mp_diag; // EPI_NEWTON_M: M_p = M*mp_scale + mp_diag*I
   float div, pow_exp, eps; // EPI_DIVPOW
 };
@@ -330,6 +331,13 @@ __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(
             const long long o = (long long)row * ldc + col;
             C[o] = C[o] - v;
           }
+        } else if (EPI == EPI_HORNER) {
+          // operands are zero padded to the tile grid, so every (row, col) is in bounds and the padding stays zero
+          const long long o = (long long)row * ldc + col;
+          float r = __fmul_rn(v, sc.alpha);
+          if (sc.beta != 0.0f) r = __fadd_rn(r, __fmul_rn(P.C2[o], sc.beta));
+          if (row == col && row < P.d) r = __fadd_rn(r, sc.mp_diag);
+          C[o] = r;
         } else if (EPI == EPI_NEWTON_M) {
           // operands are zero padded to the tile grid, so every (row, col) is in bounds
           C[(long long)row * ldc + col] = v;

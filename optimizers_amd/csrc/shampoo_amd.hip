@@ -241,6 +241,8 @@ struct sa_plan {
   GemmTable syrk0, syrk1, g1_store, g1_norm, g2_norm, g2g_norm;
   // Newton, [0] full products / [1] symmetric products: X*M_p with M_p^2 per parity, power chain, M update per parity
   GemmTable nt_a[2][2], nt_pow[2][8], nt_m[2][2];
+  GemmTable nt_h[8];      // Horner products of the higher-order iteration
+  Table<HoJob> t_ho;
   std::vector<int> newton_history;  // per factor: iterations of its last converged solve, 0 = none
   Table<SymFactor> t_sym;
   Table<NormJob> t_normjobs;
@@ -277,6 +279,17 @@ struct sa_plan {
   int* d_flags = nullptr;
   int* d_nactive = nullptr;
   int* h_pinned = nullptr;  // 4 * F + 16 ints
+
+  // higher-order iteration: per factor {z, eps, |A|_inf, -}, the kept error and the termination flag
+  float* d_ho = nullptr;
+  float* d_kept_err = nullptr;
+  int* d_hoflag = nullptr;
+
+  // trace scaling of the bias-corrected factor before any root inverse / eigenbasis computation
+  float* d_scale = nullptr;  // one multiplier per factor
+  bool trace_scaling = false;
+  float trace_exponent = 0.5f, trace_floor = 0.0f;
+  const float* scale_of(int factor) const { return trace_scaling ? d_scale + factor : nullptr; }
 
   float* f(long long off) const { return reinterpret_cast<float*>(ws) + off; }
 };
@@ -575,6 +588,16 @@ double sa_phase_executed_flops(const char* phase) {
   auto it = g_phases.find(phase ? phase : "");
   return it == g_phases.end() ? -1.0 : it->second.executed;
 }
+int32_t sa_plan_set_trace_scaling(sa_plan* p, int32_t enabled, float exponent, float floor) {
+  if (!p) return fail(SA_ERR_INVALID, "sa_plan_set_trace_scaling: null plan");
+  if (enabled && !(exponent > 0.0f && exponent <= 1.0f))
+    return fail(SA_ERR_INVALID, "sa_plan_set_trace_scaling: exponent must be in (0, 1]");
+  p->trace_scaling = enabled != 0;
+  p->trace_exponent = exponent;
+  p->trace_floor = floor;
+  return SA_OK;
+}
+
 int32_t sa_set_eigh_solver(int32_t solver) {
   g_eigh_solver = solver < 0 ? 0 : (solver > 2 ? 2 : solver);
   return SA_OK;
@@ -662,7 +685,9 @@ int32_t sa_plan_create(const sa_block_desc* blocks, int32_t n_blocks, sa_plan** 
   if (dm((void**)&p->d_err, F * 4) != hipSuccess || dm((void**)&p->d_active, F * 4) != hipSuccess ||
       dm((void**)&p->d_iters, F * 4) != hipSuccess || dm((void**)&p->d_final_parity, F * 4) != hipSuccess ||
       dm((void**)&p->d_final_err, F * 4) != hipSuccess || dm((void**)&p->d_flags, F * 4) != hipSuccess ||
-      dm((void**)&p->d_nactive, 64) != hipSuccess ||
+      dm((void**)&p->d_nactive, 64) != hipSuccess || dm((void**)&p->d_scale, F * 4) != hipSuccess ||
+      dm((void**)&p->d_ho, F * 16) != hipSuccess || dm((void**)&p->d_kept_err, F * 4) != hipSuccess ||
+      dm((void**)&p->d_hoflag, F * 4) != hipSuccess ||
       hipHostMalloc((void**)&p->h_pinned, (4 * F + 16) * sizeof(int), hipHostMallocDefault) != hipSuccess) {
     sa_plan_destroy(p);
     return fail(SA_ERR_HIP, "sa_plan_create: device allocation of control arrays failed");
@@ -679,6 +704,8 @@ void sa_plan_destroy(sa_plan* p) {
                        &p->nt_m[1][1]})
     g->t.destroy();
   for (auto& row : p->nt_pow) for (auto& g : row) g.t.destroy();
+  for (auto& g : p->nt_h) g.t.destroy();
+  p->t_ho.destroy();
   p->t_sym.destroy(); p->t_normjobs.destroy(); p->t_ids.destroy();
   p->t_jacobi.destroy(); p->t_sched.destroy(); p->t_eiginit.destroy(); p->t_eigfinal.destroy(); p->eig_gemm.t.destroy();
   if (p->trd_stream) { (void)hipStreamSynchronize(p->trd_stream); (void)hipStreamDestroy(p->trd_stream); }
@@ -690,7 +717,8 @@ void sa_plan_destroy(sa_plan* p) {
   for (auto& g : p->qr_g) g.t.destroy();
   p->t_qrpanel.destroy(); p->t_copy.destroy(); p->t_normpair.destroy(); p->t_sort.destroy();
   for (void* q : {(void*)p->d_err, (void*)p->d_active, (void*)p->d_iters, (void*)p->d_final_parity,
-                  (void*)p->d_final_err, (void*)p->d_flags, (void*)p->d_nactive})
+                  (void*)p->d_final_err, (void*)p->d_flags, (void*)p->d_nactive, (void*)p->d_scale,
+                  (void*)p->d_ho, (void*)p->d_kept_err, (void*)p->d_hoflag})
     if (q) (void)hipFree(q);
   if (p->h_pinned) (void)hipHostFree(p->h_pinned);
   delete p;
@@ -899,6 +927,7 @@ static int newton_batch(sa_plan* p, const std::vector<int>& ids, const std::vect
     SymFactor& S = p->t_sym.host[i];
     std::memset(&S, 0, sizeof(S));
     S.packed_in = f.factor;
+    S.scale = p->scale_of(ids[i]);
     S.dense_out[0] = newton_buf(p, NB_M0, f);
     S.dense_out[1] = newton_buf(p, NB_MP0, f);
     S.dense_out[2] = newton_buf(p, NB_X0, f);
@@ -1056,6 +1085,7 @@ static int root_inverse_prologue(sa_plan* p, float bias_correction2, float norm_
     std::memset(&J, 0, sizeof(J));
     J.src = f.factor;
     J.partial = p->f(p->off_norm_partial) + f.norm_off;
+    J.scale = const_cast<float*>(p->scale_of((*todo)[i]));
     J.nonfinite = p->d_flags + (*todo)[i];
     J.d = f.d; J.dpad = f.dpad; J.dense = 0;
     J.chunk_begin = chunks;
@@ -1064,6 +1094,9 @@ static int root_inverse_prologue(sa_plan* p, float bias_correction2, float norm_
     chunks += f.norm_chunks;
   }
   SACHECK(p->t_normjobs.upload(s));
+  if (p->trace_scaling)
+    hipLaunchKernelGGL(trace_scale_kernel, dim3((unsigned)todo->size()), dim3(256), 0, s, p->t_normjobs.dev, bias_correction2,
+                       p->trace_floor, p->trace_exponent);
   hipLaunchKernelGGL((factor_norm_kernel<false>), dim3(chunks), dim3(256), 0, s, p->t_normjobs.dev, (int)todo->size(),
                      bias_correction2, norm_eps);
   HIPCHECK(hipGetLastError());
@@ -1079,8 +1112,10 @@ static int root_inverse_prologue(sa_plan* p, float bias_correction2, float norm_
 
 // Shared back end: finiteness of every result X (dense, dpad-strided), then pack + mirror the results that
 // precede the first non-finite one into inv_factor and the dense inverse cache.
+// With `failures_are_local` a non-finite result only marks its own factor SA_FACTOR_SOLVER_FAILED (the solver
+// raised; the previous inverse stays) and every other result is committed; n_ok then counts nothing useful.
 static int root_inverse_epilogue(sa_plan* p, const std::vector<int>& todo, const std::vector<const float*>& X,
-                                 int32_t* status_out, hipStream_t s, size_t* n_ok) {
+                                 int32_t* status_out, hipStream_t s, size_t* n_ok, bool failures_are_local = false) {
   const int F = (int)p->factors.size();
   int* h_bad = p->h_pinned + 3 * F;
   HIPCHECK(hipMemsetAsync(p->d_flags, 0, F * sizeof(int), s));
@@ -1105,15 +1140,23 @@ static int root_inverse_epilogue(sa_plan* p, const std::vector<int>& todo, const
   HIPCHECK(hipMemcpyAsync(h_bad, p->d_flags, F * sizeof(int), hipMemcpyDeviceToHost, s));
   HIPCHECK(hipStreamSynchronize(s));
   size_t ok = todo.size();
-  for (size_t i = 0; i < todo.size(); ++i)
-    if (h_bad[todo[i]]) { status_out[todo[i]] = SA_FACTOR_RESULT_NONFINITE; ok = i; break; }
+  std::vector<size_t> keep;
+  for (size_t i = 0; i < todo.size(); ++i) {
+    if (h_bad[todo[i]]) {
+      if (failures_are_local) { status_out[todo[i]] = SA_FACTOR_SOLVER_FAILED; continue; }
+      status_out[todo[i]] = SA_FACTOR_RESULT_NONFINITE; ok = i; break;
+    }
+    keep.push_back(i);
+  }
   *n_ok = ok;
+  ok = keep.size();
   if (ok > 0) {
     SACHECK(p->t_sym.begin(ok));
     int tiles = 0;
-    for (size_t i = 0; i < ok; ++i) {
+    for (size_t k = 0; k < ok; ++k) {
+      const size_t i = keep[k];
       const Factor& f = p->factors[todo[i]];
-      SymFactor& S = p->t_sym.host[i];
+      SymFactor& S = p->t_sym.host[k];
       std::memset(&S, 0, sizeof(S));
       S.dense_in = X[i];
       S.packed_out = f.inv;
@@ -1201,6 +1244,323 @@ int32_t sa_compute_root_inverses_newton(sa_plan* p, float bias_correction2, floa
     iterations_out[fi] = iters[fi];
     if (i < ok) status_out[fi] = (errs[fi] <= tolerance) ? SA_FACTOR_OK : SA_FACTOR_NOT_CONVERGED;
   }
+  return SA_OK;
+}
+
+// --------------------------------------------------------------------------------------------
+// Batched coupled higher-order iteration (reference: matrix_functions.py:439-661)
+// --------------------------------------------------------------------------------------------
+
+constexpr int HO_MAX_ORDER = 8;
+
+// Binary power chain of `base` for exponent `root` (1, 2, 3 or a power of two) into the S1 / S2 arrays of `f`;
+// stage k goes to `stages[k]`.  Returns the array that holds the power.
+struct PowerChain {
+  int squarings = 0;
+  bool cube = false;
+  int stages() const { return std::max(squarings - 1, 0) + (cube ? 1 : 0); }
+};
+static int power_chain_for(int root, PowerChain* pc) {
+  pc->squarings = 0; pc->cube = false;
+  if (root == 3) { pc->squarings = 1; pc->cube = true; return SA_OK; }
+  int r = root;
+  while (r > 1) {
+    if (r & 1) return fail(SA_ERR_UNSUPPORTED, "coupled iterations are built for roots 1, 2, 3 and powers of two; got " + std::to_string(root));
+    r >>= 1;
+    ++pc->squarings;
+  }
+  if (pc->stages() > 4) return fail(SA_ERR_UNSUPPORTED, "root too large for the power chain");
+  return SA_OK;
+}
+
+static int higher_order_batch(sa_plan* p, const std::vector<int>& ids, int root, int order, float rel_eps, float abs_eps,
+                              float bc2, int max_iter, float tol, hipStream_t s, double* flops_acc, int* launches_acc) {
+  const int n = (int)ids.size();
+  if (n == 0) return SA_OK;
+  PowerChain pc;
+  SACHECK(power_chain_for(root, &pc));
+  const int squarings = pc.squarings;
+  const bool cube = pc.cube;
+  const int horner = order - 2;  // products that build M_p from I - M
+  // b_0 = 1, b_i = b_{i-1} (1 + (i - 1) p) / (i p): exact integer products, one division per entry
+  std::vector<double> b(order, 1.0);
+  {
+    double num = 1.0, den = 1.0;
+    for (int i = 1; i < order; ++i) { num *= 1.0 + (i - 1.0) * root; den *= (double)i * root; b[i] = num / den; }
+  }
+
+  // ---- start: A dense, |A|_inf, eps, z, then M, M_p of the plain Newton step, X -------------------------
+  SACHECK(p->t_ids.begin(n));
+  std::memcpy(p->t_ids.host, ids.data(), n * sizeof(int));
+  SACHECK(p->t_ids.upload(s));
+  SACHECK(p->t_eiginit.begin(n));
+  SACHECK(p->t_ho.begin(n));
+  int tiles = 0, dmax = 0, dpadmax = 0;
+  for (int i = 0; i < n; ++i) {
+    const Factor& f = p->factors[ids[i]];
+    EigInit& J = p->t_eiginit.host[i];
+    std::memset(&J, 0, sizeof(J));
+    J.packed = f.factor; J.scale = p->scale_of(ids[i]); J.A = newton_buf(p, NB_M0, f); J.V = newton_buf(p, NB_X0, f);
+    J.d = f.d; J.dpad = f.dpad; J.tiles = f.dpad / 64; J.enabled = 1; J.tile_begin = tiles;
+    tiles += J.tiles * J.tiles;
+    HoJob& H = p->t_ho.host[i];
+    std::memset(&H, 0, sizeof(H));
+    H.A = newton_buf(p, NB_M0, f); H.Mp = newton_buf(p, NB_MP1, f); H.X = newton_buf(p, NB_X0, f);
+    H.rowsum = newton_buf(p, NB_S1, f); H.params = p->d_ho + 4 * ids[i];
+    H.d = f.d; H.dpad = f.dpad;
+    dmax = std::max(dmax, f.d); dpadmax = std::max(dpadmax, f.dpad);
+  }
+  SACHECK(p->t_eiginit.upload(s));
+  SACHECK(p->t_ho.upload(s));
+  const unsigned start_blocks = (unsigned)(((long long)dpadmax * dpadmax + 1023) / 1024);
+  hipLaunchKernelGGL(eig_init_kernel, dim3(tiles), dim3(256), 0, s, p->t_eiginit.dev, n, bc2, 0.0f);
+  hipLaunchKernelGGL(ho_rowsum_kernel, dim3((dmax + 3) / 4, n), dim3(256), 0, s, p->t_ho.dev);
+  hipLaunchKernelGGL(ho_setup_kernel, dim3(n), dim3(256), 0, s, p->t_ho.dev, rel_eps, abs_eps);
+  hipLaunchKernelGGL(ho_start_kernel, dim3(start_blocks, n), dim3(256), 0, s, p->t_ho.dev, root, 0);
+  HIPCHECK(hipGetLastError());
+
+  // ---- GEMM tables (full products) -----------------------------------------------------------------------
+  for (int par = 0; par < 2; ++par) { p->nt_a[0][par].clear(); p->nt_m[0][par].clear(); }
+  for (int k = 0; k < 8; ++k) { p->nt_pow[0][k].clear(); p->nt_h[k].clear(); }
+  auto prob = [&](const Factor& f, const float* A, const float* B, float* C) {
+    GemmProblem q{};
+    q.A = A; q.B = B; q.C = C;
+    q.lda = q.ldb = q.ldc = f.dpad;
+    q.M = q.N = q.K = f.dpad;
+    q.d = f.d;
+    q.a_vec = q.b_vec = 1;
+    q.active = p->d_active + (&f - p->factors.data());
+    return q;
+  };
+  for (int i = 0; i < n; ++i) {
+    const Factor& f = p->factors[ids[i]];
+    float* Mp0 = newton_buf(p, NB_MP0, f);
+    float* Mp1 = newton_buf(p, NB_MP1, f);
+    float* S1 = newton_buf(p, NB_S1, f);
+    float* S2 = newton_buf(p, NB_S2, f);
+    for (int par = 0; par < 2; ++par) {
+      const float* X = newton_buf(p, par ? NB_X1 : NB_X0, f);
+      float* Xn = newton_buf(p, par ? NB_X0 : NB_X1, f);
+      const float* M = newton_buf(p, par ? NB_M1 : NB_M0, f);
+      float* Mn = newton_buf(p, par ? NB_M0 : NB_M1, f);
+      // order 2: the epilogue of the last product writes the next M_p itself, alternating between the two M_p
+      // arrays; order >= 3: it writes I - M to Mp0 and the Horner products leave M_p in Mp1
+      const float* Mp = (order == 2 && par == 1) ? Mp0 : Mp1;
+      float* seed = (order == 2 && par == 1) ? Mp1 : Mp0;
+      p->nt_a[0][par].add(prob(f, X, Mp, Xn), false);
+      if (squarings >= 1) p->nt_a[0][par].add(prob(f, Mp, Mp, S1), false);
+      const float* cur = (squarings >= 1) ? S1 : Mp;
+      int slot = par * 4;
+      float* pong[2] = {S2, S1};
+      int which = 0;
+      for (int q = 1; q < squarings; ++q) {
+        p->nt_pow[0][slot++].add(prob(f, cur, cur, pong[which]), false);
+        cur = pong[which];
+        which ^= 1;
+      }
+      if (cube) {
+        p->nt_pow[0][slot++].add(prob(f, cur, Mp, pong[which]), false);
+        cur = pong[which];
+      }
+      GemmProblem m = prob(f, cur, M, Mn);
+      m.C2 = seed;
+      m.err_bits = p->d_err + ids[i];
+      p->nt_m[0][par].add(m, false);
+    }
+    const float* prev = Mp0;
+    for (int k = 0; k < horner; ++k) {
+      float* out = (k == horner - 1) ? Mp1 : ((k & 1) ? S2 : S1);
+      GemmProblem h = prob(f, prev, Mp0, out);
+      h.C2 = Mp0;  // read only
+      p->nt_h[k].add(h, false);
+      prev = out;
+    }
+  }
+  for (int par = 0; par < 2; ++par) { SACHECK(p->nt_a[0][par].commit(s)); SACHECK(p->nt_m[0][par].commit(s)); }
+  for (int k = 0; k < 8; ++k) { SACHECK(p->nt_pow[0][k].commit(s)); SACHECK(p->nt_h[k].commit(s)); }
+
+  HigherOrderCtl ctl{p->d_err, p->d_active, p->d_iters, p->d_final_parity, p->d_final_err, p->d_kept_err, p->d_hoflag};
+  int parity = 0;
+  hipLaunchKernelGGL(higher_order_control_kernel, dim3(1), dim3(256), 0, s, ctl, p->t_ids.dev, n, tol, max_iter, 0, parity);
+  HIPCHECK(hipGetLastError());
+  int* h_active = p->h_pinned;
+  const int Fall = (int)p->factors.size();
+  HIPCHECK(hipMemcpyAsync(h_active, p->d_active, Fall * sizeof(int), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipStreamSynchronize(s));
+  GemmScalars unit = unit_scalars();
+  GemmScalars msc = unit_scalars();
+  if (order == 2) { msc.mp_scale = (float)(-b[1]); msc.mp_diag = (float)(b[1] + b[0]); }
+  else { msc.mp_scale = -1.0f; msc.mp_diag = 1.0f; }
+  for (int it = 0; it <= max_iter; ++it) {
+    const int gemms = 1 + squarings + (cube ? 1 : 0) + 1 + (it >= 1 ? horner : 0);
+    double flops = 0.0;
+    int live = 0;
+    for (int i = 0; i < n; ++i)
+      if (h_active[ids[i]]) {
+        const double d = p->factors[ids[i]].d;
+        flops += 2.0 * d * d * d * gemms;
+        ++live;
+      }
+    if (!live) break;
+    {
+      int nl = (p->nt_a[0][parity].total_tiles ? 1 : 0) + (p->nt_m[0][parity].total_tiles ? 1 : 0) + (it >= 1 ? horner : 0);
+      for (int k = 0; k < 4; ++k) nl += p->nt_pow[0][parity * 4 + k].total_tiles ? 1 : 0;
+      Span span("newton_gemm", s, flops, nl, false);
+      if (g_profiling) g_phases["newton_gemm"].executed += flops;
+      if (it >= 1) {
+        for (int k = 0; k < horner; ++k) {
+          GemmScalars hs = unit_scalars();
+          // first product: b_{o-1} (I-M)^2 + b_{o-2} (I-M) + b_{o-3} I; later ones: M_p (I-M) + b_i I
+          hs.alpha = (k == 0) ? (float)b[order - 1] : 1.0f;
+          hs.beta = (k == 0) ? (float)b[order - 2] : 0.0f;
+          hs.mp_diag = (float)b[order - 3 - k];
+          SACHECK((launch_gemm<A_MK, B_KN, EPI_HORNER, false, false>(p->nt_h[k], hs, s)));
+        }
+      }
+      SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, false>(p->nt_a[0][parity], unit, s)));
+      for (int k = 0; k < 4; ++k)
+        SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, false>(p->nt_pow[0][parity * 4 + k], unit, s)));
+      SACHECK((launch_gemm<A_MK, B_KN, EPI_NEWTON_M, false, false>(p->nt_m[0][parity], msc, s)));
+      *flops_acc += flops;
+      *launches_acc += nl;
+    }
+    parity ^= 1;
+    hipLaunchKernelGGL(higher_order_control_kernel, dim3(1), dim3(256), 0, s, ctl, p->t_ids.dev, n, tol, max_iter, it + 1, parity);
+    HIPCHECK(hipGetLastError());
+    HIPCHECK(hipMemcpyAsync(h_active, p->d_active, Fall * sizeof(int), hipMemcpyDeviceToHost, s));
+    HIPCHECK(hipStreamSynchronize(s));
+  }
+  return SA_OK;
+}
+
+// |A_r X^p - I|_max of the finished factors of one root (matrix_functions.py:622-626): A_r is rebuilt in Mp0,
+// X^p goes through S1 / S2, the product lands in the M array that does not hold the final M.
+static int higher_order_residuals(sa_plan* p, const std::vector<int>& ids, const std::vector<int>& par, int root, float bc2,
+                                  hipStream_t s) {
+  const int n = (int)ids.size();
+  if (n == 0) return SA_OK;
+  PowerChain pc;
+  SACHECK(power_chain_for(root, &pc));
+  SACHECK(p->t_eiginit.begin(n));
+  SACHECK(p->t_ho.begin(n));
+  int tiles = 0, dpadmax = 0;
+  for (int i = 0; i < n; ++i) {
+    const Factor& f = p->factors[ids[i]];
+    EigInit& J = p->t_eiginit.host[i];
+    std::memset(&J, 0, sizeof(J));
+    J.packed = f.factor; J.scale = p->scale_of(ids[i]); J.A = newton_buf(p, NB_MP0, f); J.V = newton_buf(p, NB_MP1, f);
+    J.d = f.d; J.dpad = f.dpad; J.tiles = f.dpad / 64; J.enabled = 1; J.tile_begin = tiles;
+    tiles += J.tiles * J.tiles;
+    HoJob& H = p->t_ho.host[i];
+    std::memset(&H, 0, sizeof(H));
+    H.A = newton_buf(p, NB_MP0, f); H.params = p->d_ho + 4 * ids[i]; H.d = f.d; H.dpad = f.dpad;
+    dpadmax = std::max(dpadmax, f.dpad);
+  }
+  SACHECK(p->t_eiginit.upload(s));
+  SACHECK(p->t_ho.upload(s));
+  hipLaunchKernelGGL(eig_init_kernel, dim3(tiles), dim3(256), 0, s, p->t_eiginit.dev, n, bc2, 0.0f);
+  hipLaunchKernelGGL(ho_start_kernel, dim3((unsigned)(((long long)dpadmax * dpadmax + 1023) / 1024), n), dim3(256), 0, s,
+                     p->t_ho.dev, root, 1);
+  HIPCHECK(hipGetLastError());
+  for (int k = 0; k < 8; ++k) p->nt_pow[0][k].clear();
+  p->nt_m[0][0].clear();
+  for (int i = 0; i < n; ++i) {
+    const Factor& f = p->factors[ids[i]];
+    auto prob = [&](const float* A, const float* B, float* C) {
+      GemmProblem q{};
+      q.A = A; q.B = B; q.C = C;
+      q.lda = q.ldb = q.ldc = f.dpad;
+      q.M = q.N = q.K = f.dpad;
+      q.d = f.d;
+      q.a_vec = q.b_vec = 1;
+      return q;
+    };
+    const float* X = newton_buf(p, par[ids[i]] ? NB_X1 : NB_X0, f);
+    float* S1 = newton_buf(p, NB_S1, f);
+    float* S2 = newton_buf(p, NB_S2, f);
+    const float* cur = X;
+    int slot = 0;
+    float* pong[2] = {S1, S2};
+    int which = 0;
+    for (int q = 0; q < pc.squarings; ++q) {
+      p->nt_pow[0][slot++].add(prob(cur, cur, pong[which]), false);
+      cur = pong[which];
+      which ^= 1;
+    }
+    if (pc.cube) {
+      p->nt_pow[0][slot++].add(prob(cur, X, pong[which]), false);
+      cur = pong[which];
+    }
+    GemmProblem m = prob(newton_buf(p, NB_MP0, f), cur, newton_buf(p, par[ids[i]] ? NB_M0 : NB_M1, f));
+    m.C2 = newton_buf(p, NB_MP1, f);
+    m.err_bits = p->d_err + ids[i];
+    p->nt_m[0][0].add(m, false);
+  }
+  for (int k = 0; k < 8; ++k) SACHECK(p->nt_pow[0][k].commit(s));
+  SACHECK(p->nt_m[0][0].commit(s));
+  GemmScalars unit = unit_scalars();
+  for (int k = 0; k < 8; ++k) SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, false>(p->nt_pow[0][k], unit, s)));
+  SACHECK((launch_gemm<A_MK, B_KN, EPI_NEWTON_M, false, false>(p->nt_m[0][0], unit, s)));
+  return SA_OK;
+}
+
+int32_t sa_compute_root_inverses_higher_order(sa_plan* p, float bias_correction2, float rel_epsilon, float abs_epsilon,
+                                              int32_t max_iterations, float tolerance, int32_t order,
+                                              int32_t* iterations_out, int32_t* status_out, void* stream) {
+  if (!p || !iterations_out || !status_out) return fail(SA_ERR_INVALID, "sa_compute_root_inverses_higher_order: NULL argument");
+  if (!(bias_correction2 != 0.0f) || max_iterations < 0) return fail(SA_ERR_INVALID, "bad bias correction or max_iterations");
+  if (order < 2 || order > HO_MAX_ORDER)
+    return fail(SA_ERR_UNSUPPORTED, "the higher-order iteration is built for orders 2.." + std::to_string(HO_MAX_ORDER));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SACHECK(ensure_tables(p, nullptr, s));
+  const int F = (int)p->factors.size();
+  if (F == 0) return SA_OK;
+  if (g_profiling) { Phase& ph = g_phases["newton_gemm"]; ph.used = 0; ph.work = 0.0; ph.executed = 0.0; ph.launches = 0; }
+  std::vector<int> todo;
+  SACHECK(root_inverse_prologue(p, bias_correction2, 0.0f, iterations_out, status_out, s, &todo));
+  if (todo.empty()) return SA_OK;
+
+  std::vector<int> ones(F, 0);
+  for (int i : todo) ones[i] = 1;
+  HIPCHECK(hipMemsetAsync(p->d_err, 0, F * sizeof(int), s));
+  HIPCHECK(hipMemsetAsync(p->d_iters, 0, F * sizeof(int), s));
+  HIPCHECK(hipMemsetAsync(p->d_final_parity, 0, F * sizeof(int), s));
+  HIPCHECK(hipMemsetAsync(p->d_hoflag, 0, F * sizeof(int), s));
+  HIPCHECK(hipMemsetAsync(p->d_kept_err, 0, F * sizeof(float), s));
+  HIPCHECK(hipMemcpyAsync(p->d_active, ones.data(), F * sizeof(int), hipMemcpyHostToDevice, s));
+  HIPCHECK(hipStreamSynchronize(s));
+  std::map<int, std::vector<int>> by_root;
+  for (int i : todo) by_root[p->factors[i].root].push_back(i);
+  double flops = 0.0;
+  int launches = 0;
+  for (auto& kv : by_root)
+    SACHECK(higher_order_batch(p, kv.second, kv.first, order, rel_epsilon, abs_epsilon, bias_correction2, max_iterations,
+                               tolerance, s, &flops, &launches));
+  std::vector<int> iters(F, 0), par(F, 0), flag(F, 0);
+  HIPCHECK(hipMemcpyAsync(p->h_pinned, p->d_iters, F * sizeof(int), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipMemcpyAsync(p->h_pinned + F, p->d_final_parity, F * sizeof(int), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipMemcpyAsync(p->h_pinned + 2 * F, p->d_hoflag, F * sizeof(int), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipMemsetAsync(p->d_err, 0, F * sizeof(int), s));
+  HIPCHECK(hipStreamSynchronize(s));
+  for (int i : todo) { iters[i] = p->h_pinned[i]; par[i] = p->h_pinned[F + i]; flag[i] = p->h_pinned[2 * F + i]; }
+
+  // the reference's accuracy gate: |A_r X^p - I|_max above 0.1 is a solver failure
+  for (auto& kv : by_root) SACHECK(higher_order_residuals(p, kv.second, par, kv.first, bias_correction2, s));
+  HIPCHECK(hipMemcpyAsync(p->h_pinned + 3 * F, p->d_err, F * sizeof(int), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipStreamSynchronize(s));
+  std::vector<int> pass;
+  std::vector<const float*> X;
+  for (int i : todo) {
+    float residual;
+    std::memcpy(&residual, p->h_pinned + 3 * F + i, sizeof(float));
+    iterations_out[i] = iters[i];
+    if (residual > 0.1f) { status_out[i] = SA_FACTOR_SOLVER_FAILED; continue; }
+    status_out[i] = flag[i] == 1 ? SA_FACTOR_NOT_CONVERGED : SA_FACTOR_OK;
+    pass.push_back(i);
+    X.push_back(newton_buf(p, par[i] ? NB_X1 : NB_X0, p->factors[i]));
+  }
+  size_t ok = 0;
+  if (!pass.empty()) SACHECK(root_inverse_epilogue(p, pass, X, status_out, s, &ok, true));
   return SA_OK;
 }
 
@@ -1581,6 +1941,7 @@ int32_t sa_compute_root_inverses_eigh(sa_plan* p, float bias_correction2, float 
     EigInit& J = p->t_eiginit.host[i];
     std::memset(&J, 0, sizeof(J));
     J.packed = f.factor;
+    J.scale = p->scale_of(todo[i]);
     J.A = newton_buf(p, NB_M0, f);
     J.V = newton_buf(p, NB_X0, f);
     J.d = f.d; J.dpad = f.dpad; J.tiles = f.dpad / 64; J.enabled = 1;
@@ -1682,7 +2043,7 @@ int32_t sa_refresh_eigenbases_eigh(sa_plan* p, float bias_correction2, float eps
       const Factor& f = p->factors[ids[i]];
       EigInit& J = p->t_eiginit.host[i];
       std::memset(&J, 0, sizeof(J));
-      J.packed = f.factor; J.A = newton_buf(p, NB_M0, f); J.V = newton_buf(p, NB_X0, f);
+      J.packed = f.factor; J.scale = p->scale_of(ids[i]); J.A = newton_buf(p, NB_M0, f); J.V = newton_buf(p, NB_X0, f);
       J.d = f.d; J.dpad = f.dpad; J.tiles = f.dpad / 64; J.enabled = 1; J.tile_begin = tiles;
       tiles += J.tiles * J.tiles;
     }
@@ -1971,7 +2332,7 @@ int32_t sa_refresh_eigenbases_qr(sa_plan* p, float bias_correction2, float epsil
     const Factor& f = p->factors[todo[i]];
     EigInit& J = p->t_eiginit.host[i];
     std::memset(&J, 0, sizeof(J));
-    J.packed = f.factor; J.A = newton_buf(p, NB_M0, f); J.V = newton_buf(p, NB_MP0, f);
+    J.packed = f.factor; J.scale = p->scale_of(todo[i]); J.A = newton_buf(p, NB_M0, f); J.V = newton_buf(p, NB_MP0, f);
     J.d = f.d; J.dpad = f.dpad; J.tiles = f.dpad / 64; J.enabled = 1; J.tile_begin = tiles;
     tiles += J.tiles * J.tiles;
     Copy2D& C = p->t_copy.host[i];

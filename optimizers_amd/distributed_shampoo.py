@@ -23,6 +23,7 @@ import torch
 from optimizers_amd import native
 from optimizers_amd.blocking import BlockSpec, partition_parameter
 from optimizers_amd.matrix_functions_types import (
+    CoupledHigherOrderConfig,
     CoupledNewtonConfig,
     EigenConfig,
     EigendecompositionConfig,
@@ -195,6 +196,7 @@ class _NativeGroup:
         self.factor_block: list[int] = []
         self.factor_roots: list[float] = []
         self.use_eigh = isinstance(pc.amortized_computation_config, EigenConfig)
+        self.use_higher_order = isinstance(pc.amortized_computation_config, CoupledHigherOrderConfig)
         self._slots: list[tuple[torch.Tensor, str, tuple, torch.Tensor]] = []
         self.bad_root_blocks: dict[int, str] = {}
         self.failed_counter: dict[int, int] = {}
@@ -250,6 +252,10 @@ class _NativeGroup:
                 self.factor_roots.append(float(self.roots[k][slot]))
                 if self.use_eigh or self.soap:
                     d.root[dim] = max(int(round(self.roots[k][slot])), 1)  # unused by the eigh path
+                elif root.denominator != 1 and self.use_higher_order:
+                    raise NotImplementedError(
+                        f"CoupledHigherOrderConfig with a fractional root ({root}) is not built natively"
+                    )
                 elif root.denominator != 1:
                     # the reference raises inside matrix_inverse_root at every amortized step and
                     # tolerates it num_tolerated_failed_amortized_computations times
@@ -297,6 +303,11 @@ class _NativeGroup:
             )
             self.n_factors = int(self.lib.sa_plan_num_factors(self.plan))
             assert self.n_factors == len(self.factor_names)
+            if pc.use_trace_scaling:
+                native.check(
+                    self.lib.sa_plan_set_trace_scaling(self.plan, 1, pc.trace_scaling_exponent, group[EPSILON]),
+                    "sa_plan_set_trace_scaling",
+                )
         else:
             self.n_factors = 0
         self.iterations = (ctypes.c_int32 * max(self.n_factors, 1))()
@@ -347,6 +358,9 @@ class _NativeGroup:
                 raise NotImplementedError(f"{acc.rank_deficient_stability_config=} is not supported.")
             if acc.eigendecomposition_offload_device != "":
                 raise NotImplementedError("eigendecomposition_offload_device: the decomposition runs on the MI355X")
+        elif isinstance(acc, CoupledHigherOrderConfig):
+            if not 2 <= acc.order <= 8:
+                raise NotImplementedError(f"CoupledHigherOrderConfig: orders 2..8 are built, got {acc.order=}")
         elif not isinstance(acc, CoupledNewtonConfig):
             raise NotImplementedError(
                 f"Root inverse config is not implemented! Specified root inverse config is {acc=}."
@@ -355,8 +369,6 @@ class _NativeGroup:
             raise NotImplementedError("use_symmetric_packing=False: the native step keeps factors packed")
         if pc.factor_matrix_dtype != torch.float32 or getattr(pc, "inv_factor_matrix_dtype", torch.float32) != torch.float32:
             raise NotImplementedError("factor matrices are fp32 in the native step")
-        if pc.use_trace_scaling:
-            raise NotImplementedError("use_trace_scaling is not built")
         if group[ITERATE_AVERAGING_CONFIG] is not None and not isinstance(
             group[ITERATE_AVERAGING_CONFIG], ClassicMomentumConfig
         ):
@@ -547,6 +559,14 @@ class _NativeGroup:
                 ),
                 "sa_compute_root_inverses_eigh",
             )
+        elif self.use_higher_order:
+            native.check(
+                self.lib.sa_compute_root_inverses_higher_order(
+                    self.plan, bc2, cfg.rel_epsilon, cfg.abs_epsilon, cfg.max_iterations, cfg.tolerance, cfg.order,
+                    self.iterations, self.status, stream,
+                ),
+                "sa_compute_root_inverses_higher_order",
+            )
         else:
             native.check(
                 self.lib.sa_compute_root_inverses_newton(
@@ -572,10 +592,28 @@ class _NativeGroup:
             if st == native.SA_FACTOR_NOT_CONVERGED:
                 if self.soap:
                     pass
+                elif self.use_higher_order:
+                    logger.warning("Higher order method did not converge and reached maximum number of iterations!")
                 elif self.use_eigh:
                     logger.warning(f"Eigensolver did not converge for factor matrix {name} ({self.max_jacobi_sweeps} Jacobi sweeps, or 30 QL sweeps per eigenvalue).")
                 else:
                     logger.warning("Newton did not converge and reached maximum number of iterations!")
+        # a solver failure keeps the block's previous inverse and is tolerated a limited number of consecutive times
+        # (shampoo_preconditioner_list.py:388-443)
+        failed_now = {self.factor_block[i] for i in range(self.n_factors) if int(self.status[i]) == native.SA_FACTOR_SOLVER_FAILED}
+        computed_now = {self.factor_block[i] for i in range(self.n_factors) if int(self.status[i]) != native.SA_FACTOR_SKIPPED}
+        for k in computed_now - failed_now - set(self.bad_root_blocks):
+            self.failed_counter[k] = 0
+        for k in sorted(failed_now):
+            count = self.failed_counter.get(k, 0) + 1
+            self.failed_counter[k] = count
+            names = tuple(n for n, b in zip(self.factor_names, self.factor_block) if b == k)
+            logger.warning(f"Matrix computation failed for factor matrices {names}. Using previous preconditioner and continuing...")
+            if count > pc.num_tolerated_failed_amortized_computations:
+                raise ValueError(
+                    f"The number of failed amortized computations for factors {names} exceeded the allowed tolerance. "
+                    "The last seen exception was an ArithmeticError of the coupled higher-order iteration."
+                )
         # blocks whose root cannot be used by the coupled Newton iteration fail every time
         for k, message in self.bad_root_blocks.items():
             count = self.failed_counter.get(k, 0) + 1

@@ -21,6 +21,7 @@ SA_FACTOR_INPUT_NONFINITE = 1
 SA_FACTOR_RESULT_NONFINITE = 2
 SA_FACTOR_NOT_CONVERGED = 3
 SA_FACTOR_SKIPPED = 4
+SA_FACTOR_SOLVER_FAILED = 5
 SA_GRAFT_NONE = 0
 SA_GRAFT_SGD = 1
 SA_GRAFT_ADAGRAD = 2
@@ -33,6 +34,7 @@ EXPORTS = (
     "sa_precondition_eigenvalue_corrected", "sa_update_grafting_and_filtered_grad", "sa_precondition",
     "sa_apply_update", "sa_grafting_only_step", "sa_plan_read_norms", "sa_plan_read_preconditioned",
     "sa_gemm_f32", "sa_copy_f32", "sa_set_profiling", "sa_phase_ms", "sa_phase_flops", "sa_phase_launches", "sa_phase_executed_flops", "sa_set_symmetric_newton", "sa_set_eigh_solver",
+    "sa_plan_set_trace_scaling", "sa_compute_root_inverses_higher_order",
 )
 
 
@@ -105,6 +107,9 @@ def load() -> ctypes.CDLL:
     lib.sa_compute_root_inverses_newton.argtypes = [
         c_void_p, c_float, c_float, c_int32, c_float, POINTER(c_int32), POINTER(c_int32), c_void_p,
     ]
+    lib.sa_compute_root_inverses_higher_order.argtypes = [
+        c_void_p, c_float, c_float, c_float, c_int32, c_float, c_int32, POINTER(c_int32), POINTER(c_int32), c_void_p,
+    ]
     lib.sa_compute_root_inverses_eigh.argtypes = [
         c_void_p, c_float, c_float, POINTER(c_float), c_int32, c_float, c_float, c_int32, POINTER(c_int32), POINTER(c_int32),
         c_void_p,
@@ -135,6 +140,7 @@ def load() -> ctypes.CDLL:
     lib.sa_phase_executed_flops.restype = c_double
     lib.sa_set_symmetric_newton.argtypes = [c_int32]
     lib.sa_set_eigh_solver.argtypes = [c_int32]
+    lib.sa_plan_set_trace_scaling.argtypes = [c_void_p, c_int32, c_float, c_float]
     lib.sa_phase_launches.argtypes = [c_char_p]
     lib.sa_phase_launches.restype = c_int32
     for name in EXPORTS:

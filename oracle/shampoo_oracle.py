@@ -182,6 +182,97 @@ def newton_inverse_root(
     return x, m, bool(err <= tolerance), it, err
 
 
+
+class OracleArithmeticError(ArithmeticError):
+    """The failures matrix_functions.py:543-546, :629-632, :655-658 raise as ArithmeticError."""
+
+
+def higher_order_coefficients(p: int, order: int) -> list[float]:
+    """matrix_functions.py:520-526: Taylor coefficients of (1 - x)^(-1/p),
+    b_0 = 1, b_i = b_{i-1} * (1 + (i - 1) p) / (i p), kept as exact integer
+    numerator / denominator products and divided once per entry.
+    Pinned by the binomial series (-1)^i binom(-1/p, i) in the tests.
+    """
+    b = [1.0]
+    num, den = 1, 1
+    for i in range(1, order):
+        num *= 1 + (i - 1) * p
+        den *= i * p
+        b.append(num / den)
+    return b
+
+
+def higher_order_inverse_root(
+    a: Tensor,
+    root: Fraction,
+    rel_epsilon: float = 0.0,
+    abs_epsilon: float = 0.0,
+    max_iterations: int = 100,
+    tolerance: float = 1e-8,
+    order: int = 3,
+) -> tuple[Tensor, Tensor, str, int, Tensor]:
+    """preconditioner/matrix_functions.py:439-661 (coupled higher-order iteration).
+
+    A_r = A + max(rel_eps * |A|_inf, abs_eps) I; z = 1 / trace(A_r); X = z^(1/p) I, M = z A_r;
+    one unconditional Newton step; then while error > tol and it < max: M_p = sum_i b_i (I - M)^i
+    by Horner, X <- X M_p, M <- M_p^p M; stop early when the new error exceeds 1.2 x the previous
+    one or repeats it below 1e-3 (X and M keep the last update, the error does not).  Afterwards
+    |A_r X^p - I|_max > 0.1 and a non-finite X^q raise.
+    Returns (X^q, M, flag, iterations, true_error), flag in {"converged", "max_iters", "early_stop"}.
+    Pinned by: the reference's known answers matrix_functions_test.py:216-273 (orders 2..6, roots
+    2 and 2/2), its failure cases :275-287, :337-370, fp64 eigh truth, order 2 against
+    newton_inverse_root on the same start, and fixture trajectories (iteration counts, flags).
+    """
+    p, q = root.numerator, root.denominator
+    b = higher_order_coefficients(p, order)
+    d = a.shape[0]
+    s = -1 / p
+    lam_max = torch.linalg.matrix_norm(a, torch.inf)
+    if not math.isfinite(lam_max.item()):
+        raise OracleArithmeticError("Input matrix has entries close to inf, exiting root inverse")
+    eps = torch.clamp(lam_max * rel_epsilon, min=abs_epsilon)
+    eye = torch.eye(d, dtype=a.dtype, device=a.device)
+    a_r = a + eps * eye  # _matrix_perturbation with a tensor epsilon, matrix_functions.py:145-176
+    z = torch.reciprocal(torch.trace(a_r))
+    x = torch.pow(z, -s) * eye
+    m = z * a_r
+    err = torch.linalg.vector_norm(m - eye, torch.inf)
+    # one plain Newton step first (:565-572)
+    m_p = m.mul(s).add_(eye, alpha=(1 - s))
+    x = x @ m_p
+    m = torch.linalg.matrix_power(m_p, p) @ m
+    err = torch.linalg.vector_norm(m - eye, torch.inf)
+    it = 1
+    flag = None
+    while err > tolerance and it < max_iterations:
+        it += 1
+        base = eye - m
+        m_p = base.mul(b[order - 1]).add_(eye, alpha=b[order - 2])
+        for i in reversed(range(order - 2)):
+            m_p = torch.addmm(eye, m_p, base, beta=b[i])
+        x = x @ m_p
+        m = torch.linalg.matrix_power(m_p, p) @ m
+        new_err = torch.linalg.vector_norm(m - eye, torch.inf)
+        if new_err > err * 1.2 or (new_err == err and err < 1e-3):
+            flag = "early_stop"
+            break
+        err = new_err
+    if flag is None:
+        flag = "max_iters" if err > tolerance else "converged"
+    true_err = torch.linalg.vector_norm(a_r @ torch.linalg.matrix_power(x, p) - eye, torch.inf)
+    if true_err > 1e-1:
+        raise OracleArithmeticError(
+            f"Error in matrix inverse root (before powering for fractions) {true_err} exceeds threshold 1e-1, raising an exception!"
+        )
+    if q > 1:
+        x = torch.linalg.matrix_power(x, q)
+    if not torch.isfinite(x).all():
+        raise OracleArithmeticError(
+            "NaN/Inf in matrix inverse root (after powering for fractions), raising an exception!"
+        )
+    return x, m, flag, it, true_err
+
+
 def eigh_inverse_root(a: Tensor, root: float, eps: float = 0.0) -> Tensor:
     """matrix_functions.py:306-366 + :698-770 + :179-279 with the default
     PerturbationConfig(perturb_before_computation=True): ridge first, eigh,
@@ -248,8 +339,8 @@ def qr_refresh(
 class OracleConfig:
     """Hyper-parameters with the reference's names (distributed_shampoo.py:361-382).
 
-    preconditioner: "newton" | "eigh" (RootInvShampooPreconditionerConfig with
-    CoupledNewtonConfig / EigenConfig) or "soap_qr" | "soap_eigh"
+    preconditioner: "newton" | "higher_order" | "eigh" (RootInvShampooPreconditionerConfig with
+    CoupledNewtonConfig / CoupledHigherOrderConfig / EigenConfig) or "soap_qr" | "soap_eigh"
     (EigenvalueCorrectedShampooPreconditionerConfig).
     grafting: None | "adam" | "rmsprop" | "adagrad" | "sgd".
     """
@@ -267,6 +358,11 @@ class OracleConfig:
     preconditioner: str = "eigh"
     newton_max_iterations: int = 100
     newton_tolerance: float = 1e-6
+    higher_order: int = 3  # CoupledHigherOrderConfig fields (matrix_functions_types.py:217-240)
+    higher_order_rel_epsilon: float = 0.0
+    higher_order_abs_epsilon: float = 0.0
+    higher_order_max_iterations: int = 100
+    higher_order_tolerance: float = 1e-8
     qr_max_iterations: int = 1
     qr_tolerance: float = 0.0
     inverse_exponent_override: dict = field(default_factory=dict)
@@ -279,6 +375,8 @@ class OracleConfig:
     use_nesterov: bool = False
     use_symmetric_packing: bool = True
     num_tolerated_failed_amortized_computations: int = 3
+    use_trace_scaling: bool = False  # shampoo_types.py:187-188
+    trace_scaling_exponent: float = 0.5
 
 
 class ShampooOracle:
@@ -410,6 +508,9 @@ class ShampooOracle:
         last_exc: Exception | None = None
         for k, f in enumerate(st["factors"]):
             a = self._unpack(f / self.bc2_shampoo)
+            if cfg.use_trace_scaling:  # shampoo_preconditioner_list.py:366-371
+                safe_trace = torch.clamp(torch.trace(a), min=cfg.epsilon)
+                a = a * torch.pow(safe_trace, -cfg.trace_scaling_exponent)
             name = f"{self.block_ids[bi][0]}.{self.block_ids[bi][1]}.{k}"
             if not torch.isfinite(a).all():
                 raise OraclePreconditionerValueError(
@@ -433,6 +534,12 @@ class ShampooOracle:
                             )
                         res, _, _, it, _ = newton_inverse_root(
                             a, root.numerator, cfg.epsilon, cfg.newton_max_iterations, cfg.newton_tolerance
+                        )
+                        iters.append(it)
+                    elif cfg.preconditioner == "higher_order":  # matrix_functions.py:682-689: epsilon is not passed on
+                        res, _, _, it, _ = higher_order_inverse_root(
+                            a, root, cfg.higher_order_rel_epsilon, cfg.higher_order_abs_epsilon,
+                            cfg.higher_order_max_iterations, cfg.higher_order_tolerance, cfg.higher_order,
                         )
                         iters.append(it)
                     else:

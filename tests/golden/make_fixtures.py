@@ -2,7 +2,9 @@
 
 Run once, in the build container only (the reference checkout does not travel):
 
-    python tests/golden/make_fixtures.py [/root/reference]
+    python tests/golden/make_fixtures.py [/root/reference] [--only name,name,...]
+
+(`--only` rewrites just the named multi-step cases / groups and leaves the other files alone.)
 
 It imports `distributed_shampoo` from the reference checkout, runs it on CPU in
 fp32 on tiny seeded cases and stores inputs/outputs as .npz (data only, no
@@ -24,12 +26,19 @@ from unittest import mock
 import numpy as np
 import torch
 
-REF = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
+_args = [a for a in sys.argv[1:]]
+ONLY = None
+if "--only" in _args:
+    k = _args.index("--only")
+    ONLY = set(_args[k + 1].split(","))
+    del _args[k : k + 2]
+REF = _args[0] if _args else "/root/reference"
 sys.path.insert(0, REF)
 
 from distributed_shampoo import (  # noqa: E402
     AdaGradPreconditionerConfig,
     AdamPreconditionerConfig,
+    CoupledHigherOrderConfig,
     CoupledNewtonConfig,
     DefaultSOAPConfig,
     DistributedShampoo,
@@ -91,6 +100,34 @@ CASES = {
         max_preconditioner_dim=16, precondition_frequency=3, start_preconditioning_step=3,
         preconditioner="soap_qr", override_1d=False, grafting=None,
     ),
+    "trace_scaled_newton": dict(  # use_trace_scaling without grafting: the scale of the inverse roots matters
+        shapes=[[24, 20], [20]], seed=6, grad_scale=1.0, steps=8,
+        lr=1e-2, betas=[0.9, 0.99], epsilon=1e-6, weight_decay=0.0, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=16, precondition_frequency=2, start_preconditioning_step=4,
+        preconditioner="newton", override_1d=True, grafting=None,
+        use_trace_scaling=True, trace_scaling_exponent=0.5,
+    ),
+    "trace_scaled_eigh": dict(
+        shapes=[[24, 20], [20]], seed=7, grad_scale=0.5, steps=8,
+        lr=1e-2, betas=[0.9, 0.99], epsilon=1e-4, weight_decay=0.0, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=16, precondition_frequency=2, start_preconditioning_step=4,
+        preconditioner="eigh", override_1d=False, grafting="adagrad", grafting_epsilon=1e-8,
+        use_trace_scaling=True, trace_scaling_exponent=1.0,
+    ),
+    "higher_order": dict(  # CoupledHigherOrderConfig, default order 3
+        shapes=[[24, 20], [20]], seed=8, grad_scale=1.0, steps=8,
+        lr=1e-2, betas=[0.9, 0.99], epsilon=1e-12, weight_decay=0.0, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=16, precondition_frequency=2, start_preconditioning_step=4,
+        preconditioner="higher_order", override_1d=True, grafting="adam", grafting_beta2=0.99, grafting_epsilon=1e-8,
+        ho_order=3, ho_rel_epsilon=1e-6, ho_abs_epsilon=1e-10,
+    ),
+    "higher_order_o5": dict(  # order 5, 1-D blocks preconditioned too, no grafting
+        shapes=[[20, 12], [12]], seed=9, grad_scale=1.0, steps=6,
+        lr=1e-2, betas=[0.9, 0.99], epsilon=1e-12, weight_decay=0.0, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=8, precondition_frequency=1, start_preconditioning_step=3,
+        preconditioner="higher_order", override_1d=False, grafting=None,
+        ho_order=5, ho_rel_epsilon=1e-3, ho_abs_epsilon=0.0,
+    ),
     "cfg1_override": dict(  # benchmark configuration 1 with 1-D blocks left to grafting
         shapes=[[512, 512], [512]], seed=0, grad_scale=1.0, steps=10, zero_init=True, torch_seed_grads=True,
         lr=1e-3, betas=[0.9, 0.999], epsilon=1e-12, weight_decay=0.0, weight_decay_type="DECOUPLED",
@@ -101,15 +138,25 @@ CASES = {
 
 
 def build_reference(c, params):
+    trace = dict(
+        use_trace_scaling=c.get("use_trace_scaling", False), trace_scaling_exponent=c.get("trace_scaling_exponent", 0.5)
+    )
     if c["preconditioner"] == "newton":
         pc = RootInvShampooPreconditionerConfig(
             amortized_computation_config=CoupledNewtonConfig(),
-            inverse_exponent_override={1: {0: 0.0}} if c["override_1d"] else {},
+            inverse_exponent_override={1: {0: 0.0}} if c["override_1d"] else {}, **trace,
+        )
+    elif c["preconditioner"] == "higher_order":
+        pc = RootInvShampooPreconditionerConfig(
+            amortized_computation_config=CoupledHigherOrderConfig(
+                rel_epsilon=c["ho_rel_epsilon"], abs_epsilon=c["ho_abs_epsilon"], order=c["ho_order"]
+            ),
+            inverse_exponent_override={1: {0: 0.0}} if c["override_1d"] else {}, **trace,
         )
     elif c["preconditioner"] == "eigh":
         pc = RootInvShampooPreconditionerConfig(
             amortized_computation_config=EigenConfig(),
-            inverse_exponent_override={1: {0: 0.0}} if c["override_1d"] else {},
+            inverse_exponent_override={1: {0: 0.0}} if c["override_1d"] else {}, **trace,
         )
     elif c["preconditioner"] == "soap_qr":
         pc = EigenvalueCorrectedShampooPreconditionerConfig(
@@ -159,10 +206,22 @@ def run_case(name, c):
         dist_calls.append(0)
         return real_mir(*a, **k)
 
+    # the higher-order iteration evaluates torch.linalg.vector_norm once at the start, once per iteration and
+    # once for the final residual
+    real_vn = torch.linalg.vector_norm
+
+    def counting_vn(*a, **k):
+        if dist_calls:
+            dist_calls[-1] += 1
+        return real_vn(*a, **k)
+
+    higher = c["preconditioner"] == "higher_order"
     iters_per_step = []
     if c.get("torch_seed_grads"):
         torch.manual_seed(c["seed"])
-    with mock.patch.object(torch, "dist", counting_dist), mock.patch(
+    with mock.patch.object(torch, "dist", counting_dist), mock.patch.object(
+        torch.linalg, "vector_norm", counting_vn if higher else real_vn
+    ), mock.patch(
         "distributed_shampoo.preconditioner.shampoo_preconditioner_list.matrix_inverse_root", counting_mir
     ):
         for s in range(1, c["steps"] + 1):
@@ -175,7 +234,7 @@ def run_case(name, c):
             dist_calls.clear()
             opt.step()
             # torch.dist is called once before the loop and once per iteration
-            iters_per_step.append([n - 1 for n in dist_calls])
+            iters_per_step.append([n - (2 if higher else 1) for n in dist_calls])
             for i, p in enumerate(params):
                 out[f"norm_s{s}_p{i}"] = np.float64(p.detach().double().norm().item())
     big = max(p.numel() for p in params) > 100_000
@@ -294,12 +353,65 @@ def eig_cases():
     print("eig cases ok")
 
 
+def higher_order_trajectories():
+    """matrix_inverse_root with CoupledHigherOrderConfig on stored inputs: X, iteration count, or the error raised."""
+    g = torch.Generator().manual_seed(13)
+    mats = {}
+    a = torch.randn(64, 256, generator=g)
+    well64 = a @ a.T / 256
+    a = torch.randn(48, 100, generator=g)
+    well48 = a @ a.T / 100
+    a = torch.randn(40, 24, generator=g)
+    rank24 = a @ a.T
+    a = torch.randn(96, 96, generator=g)
+    square96 = a @ a.T
+    for order in (2, 3, 4, 6):
+        mats[f"well64_r4_o{order}"] = (well64, 4, order, 0.0, 0.0, 100, 1e-8)
+    mats["well48_r2_o3"] = (well48, 2, 3, 0.0, 0.0, 100, 1e-8)
+    mats["well48_r3_o3"] = (well48, 3, 3, 0.0, 0.0, 100, 1e-8)
+    mats["well48_r1_o4"] = (well48, 1, 4, 0.0, 0.0, 100, 1e-8)
+    mats["well48_r8_o3_loose"] = (well48, 8, 3, 0.0, 0.0, 100, 1e-4)
+    mats["square96_r4_o3_rel"] = (square96, 4, 3, 1e-5, 0.0, 100, 1e-8)
+    mats["square96_r4_o3_maxit4"] = (square96, 4, 3, 1e-5, 0.0, 4, 1e-8)
+    mats["rank24_r4_o3_abs"] = (rank24, 4, 3, 0.0, 1e-3, 100, 1e-8)
+    mats["rank24_r4_o3_noeps"] = (rank24, 4, 3, 0.0, 0.0, 100, 1e-8)
+    mats["rank24_r2_o5_rel"] = (rank24, 2, 5, 1e-6, 1e-12, 100, 1e-8)
+    out = {}
+    for name, (A, root, order, rel, ab, maxit, tol) in mats.items():
+        calls = [0]
+        real = torch.linalg.vector_norm
+
+        def cv(*aa, **kk):
+            calls[0] += 1
+            return real(*aa, **kk)
+
+        cfg = CoupledHigherOrderConfig(rel_epsilon=rel, abs_epsilon=ab, max_iterations=maxit, tolerance=tol, order=order)
+        raised = ""
+        X = torch.full_like(A, float("nan"))
+        with mock.patch.object(torch.linalg, "vector_norm", cv):
+            try:
+                X = matrix_inverse_root(A, Fraction(root), cfg, 0.0)
+            except ArithmeticError as e:
+                raised = str(e)[:60]
+        out[f"{name}_A"] = A.numpy()
+        out[f"{name}_X"] = X.numpy()
+        out[f"{name}_meta"] = np.array([root, order, maxit, calls[0] - 2, int(bool(raised))], dtype=np.int64)
+        out[f"{name}_eps"] = np.array([rel, ab, tol], dtype=np.float64)
+        print("higher order", name, "iters", calls[0] - 2, "raised", raised)
+    np.savez_compressed(os.path.join(OUT, "higher_order_trajectories.npz"), **out)
+
+
 if __name__ == "__main__":
     torch.set_num_threads(8)
     with open(os.path.join(OUT, "cases.json"), "w") as f:
         json.dump(CASES, f, indent=1)
-    newton_trajectories()
-    eig_cases()
-    cfg1_as_stated()
+    groups = {
+        "newton_trajectories": newton_trajectories, "higher_order_trajectories": higher_order_trajectories,
+        "eig_cases": eig_cases, "cfg1_as_stated": cfg1_as_stated,
+    }
+    for gname, fn in groups.items():
+        if ONLY is None or gname in ONLY:
+            fn()
     for n, c in CASES.items():
-        run_case(n, c)
+        if ONLY is None or n in ONLY:
+            run_case(n, c)

@@ -15,15 +15,23 @@ from tests.golden_cases import GOLDEN, grad_stream, initial_params, load_cases, 
 pytestmark = pytest.mark.gpu
 
 CASES = load_cases()
-NEWTON_CASES = [n for n, c in CASES.items() if c["preconditioner"] == "newton"]
+NEWTON_CASES = [n for n, c in CASES.items() if c["preconditioner"] in ("newton", "higher_order") or c.get("use_trace_scaling")]
 
 
 def native_optimizer(c, params):
     import optimizers_amd as oa
 
+    solver = {
+        "newton": oa.CoupledNewtonConfig(),
+        "eigh": oa.EigenConfig(),
+        "higher_order": oa.CoupledHigherOrderConfig(
+            rel_epsilon=c.get("ho_rel_epsilon", 0.0), abs_epsilon=c.get("ho_abs_epsilon", 0.0), order=c.get("ho_order", 3)
+        ),
+    }[c["preconditioner"]]
     pc = oa.RootInvShampooPreconditionerConfig(
-        amortized_computation_config=oa.CoupledNewtonConfig(),
+        amortized_computation_config=solver,
         inverse_exponent_override={1: {0: 0.0}} if c.get("override_1d") else {},
+        use_trace_scaling=c.get("use_trace_scaling", False), trace_scaling_exponent=c.get("trace_scaling_exponent", 0.5),
     )
     graft = {
         None: None,
@@ -112,7 +120,9 @@ def test_step_matches_oracle_and_reference_fixture(name):
         if want:
             got = ng.last_newton_iterations
             assert len(got) == len(want)
-            assert max(abs(a - b) for a, b in zip(got, want)) <= 1, (got, want)
+            # the higher-order iteration ends on the first error that stops shrinking, a rounding-level event
+            slack = 3 if c["preconditioner"] == "higher_order" else 1
+            assert max(abs(a - b) for a, b in zip(got, want)) <= slack, (got, want)
 
 
 def test_config1_as_stated_raises_like_reference():

@@ -28,7 +28,7 @@ def test_multi_step_matches_reference(name):
             assert p.double().norm().item() == pytest.approx(float(z[f"norm_s{s}_p{i}"]), rel=2e-6)
     for i, p in enumerate(params):
         assert rel_err(p.reshape(-1), z[f"final_p{i}"]) < 5e-6
-    if c["preconditioner"] == "newton":
+    if c["preconditioner"] in ("newton", "higher_order"):
         ref_it = z["newton_iterations"]
         for r, row in enumerate(its):
             assert row == [int(v) for v in ref_it[r] if v >= 0]
@@ -98,6 +98,27 @@ def test_newton_trajectories():
         assert bool(torch.isfinite(X).all()) == bool(finite), n
         if finite:
             assert rel_err(X, z[n + "_X"]) < 1e-5, n
+
+
+def test_higher_order_trajectories():
+    """CoupledHigherOrderConfig on stored inputs: the reference's X, iteration count, or the fact that it raised."""
+    from fractions import Fraction
+
+    z = load_npz("higher_order_trajectories")
+    names = sorted({k[: -len("_meta")] for k in z if k.endswith("_meta")})
+    assert len(names) == 13
+    for n in names:
+        root, order, maxit, iters, raised = (int(v) for v in z[n + "_meta"])
+        rel, ab, tol = (float(v) for v in z[n + "_eps"])
+        A = torch.from_numpy(z[n + "_A"])
+        try:
+            X, _, _, it, _ = O.higher_order_inverse_root(A, Fraction(root), rel, ab, maxit, tol, order)
+        except O.OracleArithmeticError:
+            assert raised, n
+            continue
+        assert not raised, n
+        assert it == iters, n
+        assert rel_err(X, z[n + "_X"]) < 1e-5, n
 
 
 def test_eigh_and_qr_cases():

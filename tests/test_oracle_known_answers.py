@@ -241,3 +241,104 @@ def test_pseudo_inverse_root_matches_numpy_pinv_and_projector_closed_form():
     D = torch.diag(torch.tensor([4.0, 1.0, 0.25], dtype=torch.float64))
     torch.testing.assert_close(O.eigh_pseudo_inverse_root(D, 2, rank_rtol=0.0, rank_atol=0.25),
                                torch.diag(torch.tensor([0.5, 1.0, 0.0], dtype=torch.float64)))
+
+
+# --- coupled higher-order iteration ------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("order", range(2, 7))
+@pytest.mark.parametrize("exp", (1, 2))
+def test_higher_order_known_answers(order, exp):
+    """The reference's own vectors (matrix_functions_test.py:216-273): A^(-exp/2) for a diagonal and a dense 3x3."""
+    from fractions import Fraction
+
+    cases = (
+        (torch.tensor([[1.0, 0.0], [0.0, 4.0]]), torch.tensor([[1.0, 0.0], [0.0, 0.5]])),
+        (
+            torch.tensor([[1195.0, -944.0, -224.0], [-944.0, 746.0, 177.0], [-224.0, 177.0, 42.0]]),
+            torch.tensor([[1.0, 1.0, 1.0], [1.0, 2.0, -3.0], [1.0, -3.0, 18.0]]),
+        ),
+    )
+    for A, root_mat in cases:
+        X, _, _, _, _ = O.higher_order_inverse_root(A, Fraction(2, exp), order=order)
+        torch.testing.assert_close(torch.linalg.matrix_power(root_mat, exp), X, atol=0.05, rtol=1e-2)
+
+
+def test_higher_order_coefficients_are_the_binomial_series():
+    """b_i = (-1)^i binom(-1/p, i): the Taylor coefficients of (1 - x)^(-1/p)."""
+    for p in (1, 2, 3, 4, 8):
+        want, c = [], 1.0
+        for i in range(7):
+            want.append(c)
+            c *= (1.0 / p + i) / (i + 1)
+        assert O.higher_order_coefficients(p, 7) == pytest.approx(want, rel=1e-14)
+        # and the polynomial approximates (1 - x)^(-1/p)
+        x = 0.05
+        assert sum(b * x**i for i, b in enumerate(want)) == pytest.approx((1 - x) ** (-1.0 / p), rel=1e-8)
+
+
+@pytest.mark.parametrize("order", (2, 3, 5))
+@pytest.mark.parametrize("root", (1, 2, 4))
+def test_higher_order_matches_fp64_eigh_truth(order, root):
+    from fractions import Fraction
+
+    g = torch.Generator().manual_seed(3)
+    a = torch.randn(24, 80, generator=g, dtype=torch.float64)
+    A = a @ a.T / 80
+    lam, q = torch.linalg.eigh(A)
+    truth = q * lam.pow(-1.0 / root) @ q.T
+    X, M, flag, it, res = O.higher_order_inverse_root(A, Fraction(root), order=order, tolerance=1e-13)
+    assert flag in ("converged", "early_stop") and it < 30
+    assert float((X - truth).norm() / truth.norm()) < 1e-10
+    assert float((M - torch.eye(24, dtype=torch.float64)).abs().max()) < 1e-10
+    # a transposed or swapped operand in X <- X M_p would break symmetry of X on this non-commuting test:
+    B = A.clone()
+    B[0, 1] += 0.05  # slightly non-symmetric input: X must still invert B^(1/root) to first order
+    Xb, *_ = O.higher_order_inverse_root(B, Fraction(root), order=order, tolerance=1e-13)
+    assert float((torch.linalg.matrix_power(Xb, root) @ B - torch.eye(24, dtype=torch.float64)).abs().max()) < 1e-8
+
+
+def test_higher_order_order_two_is_newton_from_the_trace_start():
+    """order 2 has M_p = I + (I - M) / p, the Newton map: from a common start both give the same iterates."""
+    from fractions import Fraction
+
+    g = torch.Generator().manual_seed(4)
+    a = torch.randn(16, 40, generator=g, dtype=torch.float64)
+    A = a @ a.T / 40
+    X2, *_ = O.higher_order_inverse_root(A, Fraction(4), order=2, tolerance=1e-13)
+    # Newton started at z = (p + 1) / (2 |A|_F) converges to the same matrix
+    Xn, *_ = O.newton_inverse_root(A, 4, 0.0, 100, 1e-13)
+    assert float((X2 - Xn).norm() / Xn.norm()) < 1e-10
+
+
+def test_higher_order_failure_cases_of_the_reference():
+    """matrix_functions_test.py:275-287, 337-370: blow-up after powering, inf input, residual gate."""
+    from fractions import Fraction
+
+    A = torch.tensor([[1.0, 0.0], [0.0, 1e-4]])
+    with pytest.raises(O.OracleArithmeticError, match="after powering for fractions"):
+        O.higher_order_inverse_root(A, Fraction(1, 20))
+    with pytest.raises(O.OracleArithmeticError, match="close to inf"):
+        O.higher_order_inverse_root(torch.tensor([[1.0, 0.0], [0.0, float("inf")]]), Fraction(2))
+    with pytest.raises(O.OracleArithmeticError, match=r"exceeds threshold 1e-1"):
+        O.higher_order_inverse_root(A, Fraction(2), max_iterations=0)
+
+
+def test_trace_scaling_closed_form():
+    """Factor c I_d scaled by trace^(-1/2) is sqrt(c / d) I: without grafting the first preconditioned
+    update of a block whose factors are multiples of the identity has a closed form."""
+    d, c = 8, 3.0
+    A = c * torch.eye(d, dtype=torch.float64)
+    scaled = A * torch.pow(torch.clamp(torch.trace(A), min=1e-12), -0.5)
+    assert torch.allclose(scaled, math.sqrt(c / d) * torch.eye(d, dtype=torch.float64))
+    # through the optimizer: one parameter (d x d), gradient sqrt(c) * Q with Q orthogonal gives L = R = c I
+    q, _ = torch.linalg.qr(torch.randn(d, d, generator=torch.Generator().manual_seed(0), dtype=torch.float64))
+    G = math.sqrt(c) * q
+    W = torch.zeros(d, d, dtype=torch.float64)
+    cfg = O.OracleConfig(lr=1.0, betas=(0.0, 1.0), epsilon=1e-30, max_preconditioner_dim=8, precondition_frequency=1,
+                         start_preconditioning_step=1, preconditioner="eigh", use_trace_scaling=True,
+                         trace_scaling_exponent=0.5)
+    opt = O.ShampooOracle([W], cfg)
+    opt.step([G.clone()])
+    # P = L'^(-1/4) G R'^(-1/4) with L' = R' = sqrt(c / d) I  =>  W = -(c / d)^(-1/4) G
+    assert torch.allclose(W, -((c / d) ** -0.25) * G, rtol=1e-9, atol=1e-12)
