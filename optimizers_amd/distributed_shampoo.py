@@ -632,8 +632,8 @@ class DistributedShampoo(torch.optim.Optimizer):
 
     Arguments, defaults and validation follow the reference constructor
     (distributed_shampoo/distributed_shampoo.py:361-535).  Built natively:
-    `RootInvShampooPreconditionerConfig` with `CoupledNewtonConfig` or `EigenConfig` (`PerturbationConfig` and
-    `PseudoInverseConfig`), `EigenvalueCorrectedShampooPreconditionerConfig` with `QREigendecompositionConfig` or
+    `RootInvShampooPreconditionerConfig` with `CoupledNewtonConfig`, `CoupledHigherOrderConfig` (orders 2..8) or
+    `EigenConfig` (`PerturbationConfig` and `PseudoInverseConfig`), `use_trace_scaling`, `EigenvalueCorrectedShampooPreconditionerConfig` with `QREigendecompositionConfig` or
     `EighEigendecompositionConfig` (including `ignored_basis_change_dims`), grafting with SGD / AdaGrad / RMSprop /
     Adam or none, every `WeightDecayType`, `ClassicMomentumConfig`, `inverse_exponent_override`,
     `SingleDeviceDistributedConfig`, fp32 state with packed factor matrices, blocks of order 1 and 2.
