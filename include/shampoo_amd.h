@@ -208,6 +208,13 @@ int32_t sa_grafting_only_step(sa_plan* plan, const sa_step_scalars* s, void* str
 
 /* Test / measurement aids. */
 
+/* Eigenvalue estimates that belong to the eigenbasis the last sa_refresh_eigenbases_eigh / _qr call on this plan
+ * left for factor `factor` (index in plan order), in the order of the basis' columns: the ascending eigenvalues
+ * of a fresh decomposition, diag(Q^T A Q) of a basis kept by the tolerance criterion, the sorted Rayleigh
+ * quotients of a QR refresh -- the first return value of matrix_eigendecomposition (matrix_functions.py:698-908).
+ * out: device array of that factor's order.  Must directly follow the refresh call; SA_ERR_STATE otherwise. */
+int32_t sa_plan_read_eigenvalues(sa_plan* plan, int32_t factor, float* out, void* stream);
+
 /* Per-block squared norms of the last step: graft_sq[i], precond_sq[i] (host arrays of n_blocks). */
 int32_t sa_plan_read_norms(sa_plan* plan, float* graft_sq, float* precond_sq, void* stream);
 

@@ -358,6 +358,13 @@ __global__ __launch_bounds__(256) void eig_rank_kernel(const RankJob* __restrict
   }
 }
 
+// out[k] = base[(order ? order[k] : k) * stride]
+__global__ __launch_bounds__(256) void gather_strided_kernel(const float* __restrict__ base, long long stride,
+                                                            const int* __restrict__ order, float* __restrict__ out, int n) {
+  const int k = blockIdx.x * 256 + threadIdx.x;
+  if (k < n) out[k] = base[(long long)(order ? order[k] : k) * stride];
+}
+
 // dst[r][k] = src[order[k]][r]: eigenvectors held as rows become sorted columns.  32 x 32 tiles through LDS,
 // grid (ceil(d / 32), ceil(d / 32), factors).
 struct RowsToCols {

@@ -280,6 +280,10 @@ struct sa_plan {
   int* d_nactive = nullptr;
   int* h_pinned = nullptr;  // 4 * F + 16 ints
 
+  // where the eigenvalue estimates of the last eigenbasis refresh sit in the workspace (valid until the next call)
+  struct EigSource { const float* base = nullptr; long long stride = 0; const int* order = nullptr; };
+  std::vector<EigSource> eig_source;
+
   // higher-order iteration: per factor {z, eps, |A|_inf, -}, the kept error and the termination flag
   float* d_ho = nullptr;
   float* d_kept_err = nullptr;
@@ -864,6 +868,19 @@ int32_t sa_apply_update(sa_plan* p, const sa_step_scalars* sc, void* stream) {
   Span span("apply", s, bytes, 1, true);
   hipLaunchKernelGGL(apply_kernel, dim3((unsigned)p->t_chunks.n), dim3(EW_THREADS), 0, s, p->t_blocks.dev,
                      p->t_chunks.dev, *sc, p->n_blocks, p->f(p->off_norms));
+  HIPCHECK(hipGetLastError());
+  return SA_OK;
+}
+
+int32_t sa_plan_read_eigenvalues(sa_plan* p, int32_t factor, float* out, void* stream) {
+  if (!p || !out) return fail(SA_ERR_INVALID, "sa_plan_read_eigenvalues: NULL argument");
+  if (factor < 0 || factor >= (int)p->factors.size()) return fail(SA_ERR_INVALID, "sa_plan_read_eigenvalues: factor out of range");
+  if ((int)p->eig_source.size() != (int)p->factors.size() || !p->eig_source[factor].base)
+    return fail(SA_ERR_STATE, "sa_plan_read_eigenvalues: the last call on this plan did not refresh this factor's eigenbasis");
+  const sa_plan::EigSource& e = p->eig_source[factor];
+  const int d = p->factors[factor].d;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(gather_strided_kernel, dim3((d + 255) / 256), dim3(256), 0, s, e.base, e.stride, e.order, out, d);
   HIPCHECK(hipGetLastError());
   return SA_OK;
 }
@@ -2032,6 +2049,7 @@ int32_t sa_refresh_eigenbases_eigh(sa_plan* p, float bias_correction2, float eps
   SACHECK(ensure_tables(p, nullptr, s));
   const int F = (int)p->factors.size();
   if (F == 0) return SA_OK;
+  p->eig_source.assign(F, sa_plan::EigSource{});
   std::vector<int> todo;
   SACHECK(root_inverse_prologue(p, bias_correction2, epsilon, sweeps_out, status_out, s, &todo));
   if (todo.empty()) return SA_OK;
@@ -2101,8 +2119,13 @@ int32_t sa_refresh_eigenbases_eigh(sa_plan* p, float bias_correction2, float eps
     for (int i : todo) {
       const float norm = std::sqrt(h_all[i]), dnorm = std::sqrt(h_diag[i]);
       const float off = std::sqrt(norm * norm - dnorm * dnorm);
-      if (off <= tolerance * norm) status_out[i] = SA_FACTOR_OK;  // the stored basis stays
-      else solve.push_back(i);
+      if (off <= tolerance * norm) {
+        status_out[i] = SA_FACTOR_OK;  // the stored basis stays; its eigenvalue estimates are diag(Q^T A Q)
+        const Factor& f = p->factors[i];
+        p->eig_source[i] = sa_plan::EigSource{newton_buf(p, NB_S1, f), (long long)f.dpad + 1, nullptr};
+      } else {
+        solve.push_back(i);
+      }
     }
     HIPCHECK(hipMemsetAsync(p->d_err, 0, F * sizeof(int), s));
     if (solve.empty()) return SA_OK;
@@ -2132,6 +2155,7 @@ int32_t sa_refresh_eigenbases_eigh(sa_plan* p, float bias_correction2, float eps
     R.lambda_stride = t ? 1 : (long long)f.dpad + 1;
     R.order = reinterpret_cast<int*>(newton_buf(p, NB_MP0, f));
     R.d = f.d;
+    p->eig_source[solve[k]] = sa_plan::EigSource{R.lambda_in, R.lambda_stride, R.order};
     if (t) {
       RowsToCols& C = p->t_rows2cols.host[n_rows++];
       C.src = newton_buf(p, NB_X0, f); C.lds_ = f.dpad; C.dst = newton_buf(p, NB_S1, f); C.ldd = f.dpad; C.order = R.order; C.d = f.d;
@@ -2319,6 +2343,7 @@ int32_t sa_refresh_eigenbases_qr(sa_plan* p, float bias_correction2, float epsil
   SACHECK(ensure_tables(p, nullptr, s));
   const int F = (int)p->factors.size();
   if (F == 0) return SA_OK;
+  p->eig_source.assign(F, sa_plan::EigSource{});
   std::vector<int> todo;
   SACHECK(root_inverse_prologue(p, bias_correction2, epsilon, iterations_out, status_out, s, &todo));
   if (todo.empty()) return SA_OK;
@@ -2423,6 +2448,7 @@ int32_t sa_refresh_eigenbases_qr(sa_plan* p, float bias_correction2, float epsil
     J.ev = newton_buf(p, NB_S2, f) + 2LL * f.dpad * QR_MAX_PANEL;
     J.order = reinterpret_cast<int*>(J.ev + f.dpad);
     J.d = f.d;
+    p->eig_source[todo[k]] = sa_plan::EigSource{J.ev, 1, J.order};
     Copy2D& C = p->t_copy.host[k];
     std::memset(&C, 0, sizeof(C));
     C.src = newton_buf(p, NB_X1, f); C.lds_ = f.dpad; C.dst = newton_buf(p, NB_X0, f); C.ldd = f.dpad;

@@ -538,9 +538,10 @@ class _NativeGroup:
                 "sa_refresh_eigenbases_eigh",
             )
         elif self.soap:
+            ridge = group[EPSILON] * float(cfg.rank_deficient_stability_config.perturb_before_computation)
             native.check(
                 self.lib.sa_refresh_eigenbases_qr(
-                    self.plan, bc2, group[EPSILON], cfg.max_iterations, cfg.tolerance, self.iterations, self.status, stream
+                    self.plan, bc2, ridge, cfg.max_iterations, cfg.tolerance, self.iterations, self.status, stream
                 ),
                 "sa_refresh_eigenbases_qr",
             )

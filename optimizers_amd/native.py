@@ -34,7 +34,7 @@ EXPORTS = (
     "sa_precondition_eigenvalue_corrected", "sa_update_grafting_and_filtered_grad", "sa_precondition",
     "sa_apply_update", "sa_grafting_only_step", "sa_plan_read_norms", "sa_plan_read_preconditioned",
     "sa_gemm_f32", "sa_copy_f32", "sa_set_profiling", "sa_phase_ms", "sa_phase_flops", "sa_phase_launches", "sa_phase_executed_flops", "sa_set_symmetric_newton", "sa_set_eigh_solver",
-    "sa_plan_set_trace_scaling", "sa_compute_root_inverses_higher_order",
+    "sa_plan_set_trace_scaling", "sa_compute_root_inverses_higher_order", "sa_plan_read_eigenvalues",
 )
 
 
@@ -140,6 +140,7 @@ def load() -> ctypes.CDLL:
     lib.sa_phase_executed_flops.restype = c_double
     lib.sa_set_symmetric_newton.argtypes = [c_int32]
     lib.sa_set_eigh_solver.argtypes = [c_int32]
+    lib.sa_plan_read_eigenvalues.argtypes = [c_void_p, c_int32, c_void_p, c_void_p]
     lib.sa_plan_set_trace_scaling.argtypes = [c_void_p, c_int32, c_float, c_float]
     lib.sa_phase_launches.argtypes = [c_char_p]
     lib.sa_phase_launches.restype = c_int32
