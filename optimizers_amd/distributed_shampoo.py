@@ -103,7 +103,117 @@ class _Arena:
         return self.buffer[self.offsets[i] : self.offsets[i] + n].view(shape)
 
 
-class _NativeGroup:
+class _AmortizedComputation:
+    """Batched amortized computation of one plan with the reference's error semantics.  Needs the attributes
+    lib, plan, preconditioner_config, soap, use_eigh, use_higher_order, n_factors, factor_names, factor_block,
+    factor_roots, iterations, status, max_jacobi_sweeps, bad_root_blocks, failed_counter."""
+
+    def _amortized_computation(self, group: dict[str, Any], bc2: float, stream: int) -> None:
+        """Batched inverse roots + the reference's error semantics
+        (shampoo_preconditioner_list.py:314-443)."""
+        pc = self.preconditioner_config
+        cfg = pc.amortized_computation_config
+        if self.soap and isinstance(cfg, EighEigendecompositionConfig):
+            # epsilon * I is added only when the config perturbs before the computation (matrix_functions.py:869-882)
+            ridge = group[EPSILON] * float(cfg.rank_deficient_stability_config.perturb_before_computation)
+            native.check(
+                self.lib.sa_refresh_eigenbases_eigh(
+                    self.plan, bc2, ridge, cfg.tolerance, self.max_jacobi_sweeps, self.iterations, self.status, stream
+                ),
+                "sa_refresh_eigenbases_eigh",
+            )
+        elif self.soap:
+            ridge = group[EPSILON] * float(cfg.rank_deficient_stability_config.perturb_before_computation)
+            native.check(
+                self.lib.sa_refresh_eigenbases_qr(
+                    self.plan, bc2, ridge, cfg.max_iterations, cfg.tolerance, self.iterations, self.status, stream
+                ),
+                "sa_refresh_eigenbases_qr",
+            )
+        elif self.use_eigh:
+            roots = (ctypes.c_float * max(self.n_factors, 1))(*self.factor_roots)
+            stab = cfg.rank_deficient_stability_config
+            if isinstance(stab, PseudoInverseConfig):
+                # rank_rtol=None is the reference's "order * machine epsilon" (matrix_functions.py:226-229)
+                mode, rtol, atol = 2, (-1.0 if stab.rank_rtol is None else float(stab.rank_rtol)), float(stab.rank_atol)
+            else:
+                mode, rtol, atol = int(stab.perturb_before_computation), 0.0, 0.0
+            native.check(
+                self.lib.sa_compute_root_inverses_eigh(
+                    self.plan, bc2, group[EPSILON], roots, mode, rtol, atol, self.max_jacobi_sweeps,
+                    self.iterations, self.status, stream,
+                ),
+                "sa_compute_root_inverses_eigh",
+            )
+        elif self.use_higher_order:
+            native.check(
+                self.lib.sa_compute_root_inverses_higher_order(
+                    self.plan, bc2, cfg.rel_epsilon, cfg.abs_epsilon, cfg.max_iterations, cfg.tolerance, cfg.order,
+                    self.iterations, self.status, stream,
+                ),
+                "sa_compute_root_inverses_higher_order",
+            )
+        else:
+            native.check(
+                self.lib.sa_compute_root_inverses_newton(
+                    self.plan, bc2, group[EPSILON], cfg.max_iterations, cfg.tolerance, self.iterations, self.status, stream
+                ),
+                "sa_compute_root_inverses_newton",
+            )
+        self.last_newton_iterations = [int(self.iterations[i]) for i in range(self.n_factors)]
+        for i in range(self.n_factors):
+            st = int(self.status[i])
+            name = self.factor_names[i]
+            if st == native.SA_FACTOR_INPUT_NONFINITE:
+                raise PreconditionerValueError(
+                    f"Encountered nan/inf values in factor matrix {name}! "
+                    "To mitigate, check if nan inputs are being passed into the network or nan gradients are being passed to the optimizer. "
+                    "Otherwise, in some cases, this may be due to divergence of the algorithm. To mitigate, try decreasing the learning rate or increasing grafting epsilon."
+                )
+            if st == native.SA_FACTOR_RESULT_NONFINITE:
+                raise PreconditionerValueError(
+                    f"Encountered nan or inf values in name of factor matrix {name}! "
+                    "To mitigate, check factor matrix before the matrix computation."
+                )
+            if st == native.SA_FACTOR_NOT_CONVERGED:
+                if self.soap:
+                    pass
+                elif self.use_higher_order:
+                    logger.warning("Higher order method did not converge and reached maximum number of iterations!")
+                elif self.use_eigh:
+                    logger.warning(f"Eigensolver did not converge for factor matrix {name} ({self.max_jacobi_sweeps} Jacobi sweeps, or 30 QL sweeps per eigenvalue).")
+                else:
+                    logger.warning("Newton did not converge and reached maximum number of iterations!")
+        # a solver failure keeps the block's previous inverse and is tolerated a limited number of consecutive times
+        # (shampoo_preconditioner_list.py:388-443)
+        failed_now = {self.factor_block[i] for i in range(self.n_factors) if int(self.status[i]) == native.SA_FACTOR_SOLVER_FAILED}
+        computed_now = {self.factor_block[i] for i in range(self.n_factors) if int(self.status[i]) != native.SA_FACTOR_SKIPPED}
+        for k in computed_now - failed_now - set(self.bad_root_blocks):
+            self.failed_counter[k] = 0
+        for k in sorted(failed_now):
+            count = self.failed_counter.get(k, 0) + 1
+            self.failed_counter[k] = count
+            names = tuple(n for n, b in zip(self.factor_names, self.factor_block) if b == k)
+            logger.warning(f"Matrix computation failed for factor matrices {names}. Using previous preconditioner and continuing...")
+            if count > pc.num_tolerated_failed_amortized_computations:
+                raise ValueError(
+                    f"The number of failed amortized computations for factors {names} exceeded the allowed tolerance. "
+                    "The last seen exception was an ArithmeticError of the coupled higher-order iteration."
+                )
+        # blocks whose root cannot be used by the coupled Newton iteration fail every time
+        for k, message in self.bad_root_blocks.items():
+            count = self.failed_counter.get(k, 0) + 1
+            self.failed_counter[k] = count
+            logger.warning(f"Matrix computation failed with exception={message!r}. Using previous preconditioner and continuing...")
+            if count > pc.num_tolerated_failed_amortized_computations:
+                names = tuple(n for n, b in zip(self.factor_names, self.factor_block) if b == k)
+                raise ValueError(
+                    f"The number of failed amortized computations for factors {names} exceeded the allowed tolerance. "
+                    f"The last seen exception was {message}."
+                )
+
+
+class _NativeGroup(_AmortizedComputation):
     """Native state and schedule of one parameter group (reference: the per-group state lists
     built in distributed_shampoo.py:563-975 plus `_group_step_body` :1562-1667)."""
 
@@ -522,110 +632,6 @@ class _NativeGroup:
             native.check(lib.sa_apply_update(self.plan, ref, stream), "sa_apply_update")
         # drop the references so param.grad can be freed (distributed_shampoo.py:1666-1667)
         self._grads_alive = None
-
-    def _amortized_computation(self, group: dict[str, Any], bc2: float, stream: int) -> None:
-        """Batched inverse roots + the reference's error semantics
-        (shampoo_preconditioner_list.py:314-443)."""
-        pc = self.preconditioner_config
-        cfg = pc.amortized_computation_config
-        if self.soap and isinstance(cfg, EighEigendecompositionConfig):
-            # epsilon * I is added only when the config perturbs before the computation (matrix_functions.py:869-882)
-            ridge = group[EPSILON] * float(cfg.rank_deficient_stability_config.perturb_before_computation)
-            native.check(
-                self.lib.sa_refresh_eigenbases_eigh(
-                    self.plan, bc2, ridge, cfg.tolerance, self.max_jacobi_sweeps, self.iterations, self.status, stream
-                ),
-                "sa_refresh_eigenbases_eigh",
-            )
-        elif self.soap:
-            ridge = group[EPSILON] * float(cfg.rank_deficient_stability_config.perturb_before_computation)
-            native.check(
-                self.lib.sa_refresh_eigenbases_qr(
-                    self.plan, bc2, ridge, cfg.max_iterations, cfg.tolerance, self.iterations, self.status, stream
-                ),
-                "sa_refresh_eigenbases_qr",
-            )
-        elif self.use_eigh:
-            roots = (ctypes.c_float * max(self.n_factors, 1))(*self.factor_roots)
-            stab = cfg.rank_deficient_stability_config
-            if isinstance(stab, PseudoInverseConfig):
-                # rank_rtol=None is the reference's "order * machine epsilon" (matrix_functions.py:226-229)
-                mode, rtol, atol = 2, (-1.0 if stab.rank_rtol is None else float(stab.rank_rtol)), float(stab.rank_atol)
-            else:
-                mode, rtol, atol = int(stab.perturb_before_computation), 0.0, 0.0
-            native.check(
-                self.lib.sa_compute_root_inverses_eigh(
-                    self.plan, bc2, group[EPSILON], roots, mode, rtol, atol, self.max_jacobi_sweeps,
-                    self.iterations, self.status, stream,
-                ),
-                "sa_compute_root_inverses_eigh",
-            )
-        elif self.use_higher_order:
-            native.check(
-                self.lib.sa_compute_root_inverses_higher_order(
-                    self.plan, bc2, cfg.rel_epsilon, cfg.abs_epsilon, cfg.max_iterations, cfg.tolerance, cfg.order,
-                    self.iterations, self.status, stream,
-                ),
-                "sa_compute_root_inverses_higher_order",
-            )
-        else:
-            native.check(
-                self.lib.sa_compute_root_inverses_newton(
-                    self.plan, bc2, group[EPSILON], cfg.max_iterations, cfg.tolerance, self.iterations, self.status, stream
-                ),
-                "sa_compute_root_inverses_newton",
-            )
-        self.last_newton_iterations = [int(self.iterations[i]) for i in range(self.n_factors)]
-        for i in range(self.n_factors):
-            st = int(self.status[i])
-            name = self.factor_names[i]
-            if st == native.SA_FACTOR_INPUT_NONFINITE:
-                raise PreconditionerValueError(
-                    f"Encountered nan/inf values in factor matrix {name}! "
-                    "To mitigate, check if nan inputs are being passed into the network or nan gradients are being passed to the optimizer. "
-                    "Otherwise, in some cases, this may be due to divergence of the algorithm. To mitigate, try decreasing the learning rate or increasing grafting epsilon."
-                )
-            if st == native.SA_FACTOR_RESULT_NONFINITE:
-                raise PreconditionerValueError(
-                    f"Encountered nan or inf values in name of factor matrix {name}! "
-                    "To mitigate, check factor matrix before the matrix computation."
-                )
-            if st == native.SA_FACTOR_NOT_CONVERGED:
-                if self.soap:
-                    pass
-                elif self.use_higher_order:
-                    logger.warning("Higher order method did not converge and reached maximum number of iterations!")
-                elif self.use_eigh:
-                    logger.warning(f"Eigensolver did not converge for factor matrix {name} ({self.max_jacobi_sweeps} Jacobi sweeps, or 30 QL sweeps per eigenvalue).")
-                else:
-                    logger.warning("Newton did not converge and reached maximum number of iterations!")
-        # a solver failure keeps the block's previous inverse and is tolerated a limited number of consecutive times
-        # (shampoo_preconditioner_list.py:388-443)
-        failed_now = {self.factor_block[i] for i in range(self.n_factors) if int(self.status[i]) == native.SA_FACTOR_SOLVER_FAILED}
-        computed_now = {self.factor_block[i] for i in range(self.n_factors) if int(self.status[i]) != native.SA_FACTOR_SKIPPED}
-        for k in computed_now - failed_now - set(self.bad_root_blocks):
-            self.failed_counter[k] = 0
-        for k in sorted(failed_now):
-            count = self.failed_counter.get(k, 0) + 1
-            self.failed_counter[k] = count
-            names = tuple(n for n, b in zip(self.factor_names, self.factor_block) if b == k)
-            logger.warning(f"Matrix computation failed for factor matrices {names}. Using previous preconditioner and continuing...")
-            if count > pc.num_tolerated_failed_amortized_computations:
-                raise ValueError(
-                    f"The number of failed amortized computations for factors {names} exceeded the allowed tolerance. "
-                    "The last seen exception was an ArithmeticError of the coupled higher-order iteration."
-                )
-        # blocks whose root cannot be used by the coupled Newton iteration fail every time
-        for k, message in self.bad_root_blocks.items():
-            count = self.failed_counter.get(k, 0) + 1
-            self.failed_counter[k] = count
-            logger.warning(f"Matrix computation failed with exception={message!r}. Using previous preconditioner and continuing...")
-            if count > pc.num_tolerated_failed_amortized_computations:
-                names = tuple(n for n, b in zip(self.factor_names, self.factor_block) if b == k)
-                raise ValueError(
-                    f"The number of failed amortized computations for factors {names} exceeded the allowed tolerance. "
-                    f"The last seen exception was {message}."
-                )
 
 
 class DistributedShampoo(torch.optim.Optimizer):
