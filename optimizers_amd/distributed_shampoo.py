@@ -763,6 +763,17 @@ class DistributedShampoo(torch.optim.Optimizer):
             )
 
     @torch.no_grad()
+    def train(self) -> None:
+        """distributed_shampoo.py:1729-1761: switches groups with primal-averaging / schedule-free iterate averaging
+        to the training iterate.  Only `ClassicMomentumConfig` is built here, for which the reference does nothing."""
+        logger.info("Enabling train mode in Distributed Shampoo!")
+
+    @torch.no_grad()
+    def eval(self) -> None:
+        """distributed_shampoo.py:1763-1795; nothing to do without primal-averaging / schedule-free groups."""
+        logger.info("Enabling eval mode in Distributed Shampoo!")
+
+    @torch.no_grad()
     def step(self, closure: Callable[[], float] | None = None) -> float | None:
         """One optimization step (distributed_shampoo.py:1677-1711)."""
         loss = None
