@@ -49,10 +49,17 @@ extern "C" {
 
 typedef struct sa_plan sa_plan;
 
+#define SA_MAX_ORDER 3
+
 /*
- * One block of a (merged) parameter: an fp32 rows x cols strided view, produced by
- * merge_small_dims + multi_dim_split (utils/shampoo_utils.py:38-174).  A 1-D block of
- * length d is rows = d, cols = 1, ld = 1.  State buffers are contiguous (rows*cols).
+ * One block of a (merged) parameter, produced by merge_small_dims + multi_dim_split
+ * (utils/shampoo_utils.py:38-174): an fp32 strided view of order 1, 2 or 3.
+ *   order 2:  rows x cols, row stride ld.                       mid = 0.
+ *   order 1:  length d as rows = d, cols = 1, ld = 1.           mid = 0.
+ *   order 3:  d0 x d1 x d2 with element strides (ld_outer, ld, 1) as rows = d0 * d1, cols = d2, mid = d1:
+ *             row r = i0 * d1 + i1 of the flattened block starts at i0 * ld_outer + i1 * ld.
+ * State buffers are contiguous (rows * cols, the block's own row-major order).  Kronecker factor k belongs to
+ * dim k of the block: for order <= 2 dim 0 = rows, dim 1 = cols; for order 3 dims (d0, d1, d2).
  * Mirrors what BlockInfo + the per-block optimizer state hold
  * (distributor/shampoo_block_info.py:18-65; state keys shampoo_types.py:35-41).
  */
@@ -63,16 +70,18 @@ typedef struct sa_block_desc {
   float* filtered_grad;   /* EMA of the gradient, or NULL when beta1 == 0 */
   float* adagrad;         /* grafting second moment, or NULL */
   float* momentum_buffer; /* classic momentum buffer, or NULL */
-  float* factor[2];       /* packed upper-triangular Kronecker factor of dim 0 / dim 1; NULL = dim not preconditioned */
-  float* inv_factor[2];   /* packed upper-triangular inverse root of that factor (root-inverse Shampoo), or NULL */
-  int32_t root[2];        /* integer inverse root (4 for matrices, 2 for vectors by default) */
-  /* eigenvalue-corrected Shampoo / SOAP (shampoo_preconditioner_list.py:942-1007): dense d x d eigenbasis of
-   * each factor (row-major, columns are eigenvectors) and the second moment kept in the rotated basis
-   * (rows x cols, contiguous).  NULL for root-inverse Shampoo.  eigenvectors[k] with factor[k] == NULL is a
+  float* factor[SA_MAX_ORDER];     /* packed upper-triangular Kronecker factor per dim; NULL = dim not preconditioned */
+  float* inv_factor[SA_MAX_ORDER]; /* packed upper-triangular inverse root of that factor (root-inverse Shampoo), or NULL */
+  int32_t root[SA_MAX_ORDER];      /* integer inverse root (2 * order by default: 2 for vectors, 4 for matrices, 6 for order 3) */
+  /* eigenvalue-corrected Shampoo / SOAP (shampoo_preconditioner_list.py:942-1007), blocks of order <= 2 only: dense
+   * d x d eigenbasis of each factor (row-major, columns are eigenvectors) and the second moment kept in the rotated
+   * basis (rows x cols, contiguous).  NULL for root-inverse Shampoo.  eigenvectors[k] with factor[k] == NULL is a
    * fixed basis: it rotates the block but has no statistics and is never refreshed (a block whose basis
    * changes are all ignored, ignored_basis_change_dims, passes one identity matrix). */
-  float* eigenvectors[2];
+  float* eigenvectors[SA_MAX_ORDER];
   float* corrected_eigenvalues;
+  int32_t mid;            /* d1 of an order-3 block, else 0 */
+  int64_t ld_outer;       /* stride of dim 0 of an order-3 block */
 } sa_block_desc;
 
 /* Scalars of one step, already evaluated by the host exactly as the reference evaluates
@@ -128,7 +137,8 @@ int32_t sa_update_factor_matrices(sa_plan* plan, float beta2, float weighting_fa
  * (matrix_functions.py:368-437 via shampoo_preconditioner_list.py:314-443, 631-680).
  * iterations_out / status_out: host arrays of sa_plan_num_factors() entries.  Inverse roots of
  * factors that precede the first non-finite one are stored into inv_factor (upper triangle);
- * the call synchronises the stream before it returns. */
+ * the call synchronises the stream before it returns.  M_p^root is a square-and-multiply chain of at most
+ * five products: every integer root up to 14, and 16 (SA_ERR_UNSUPPORTED beyond). */
 int32_t sa_compute_root_inverses_newton(sa_plan* plan, float bias_correction2, float epsilon,
                                         int32_t max_iterations, float tolerance,
                                         int32_t* iterations_out, int32_t* status_out, void* stream);

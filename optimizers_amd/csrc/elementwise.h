@@ -38,7 +38,29 @@ struct BlockDev {
   int vec;                // every pointer of this block is 16-byte aligned and rows hold multiples of 4
   int p_vec;              // same for p_src
   int p_is_ghat;          // block has no preconditioned dim: direction = filtered gradient
+  int mid;                // order-3 block d0 x d1 x d2 flattened to rows = d0 * d1: d1, else 0
+  long long ld_outer;     // stride of dim 0 of an order-3 block
+  int contig;             // param / grad view is contiguous in the block's own element order
+  int p_like_grad;        // p_src is the gradient view itself (strided like param / grad)
+  float* g3_dense;        // order 3: dense d0 x d1 x d2 copy of the gradient for the factor updates, or nullptr
+  float* g3_perm;         // order 3: the same permuted to d1 x d0 x d2, or nullptr
+  float* g3_ghat;         // order 3, beta1 == 0: dense copy of the gradient for the mode products, or nullptr
 };
+
+// offset of element e (block's own row-major order) inside the strided param / grad view
+__device__ __forceinline__ long long view_offset(const BlockDev& B, int e) {
+  if (B.contig) return e;
+  const int r = e / B.cols, c = e - r * B.cols;
+  if (B.mid > 0) {
+    const int o = r / B.mid;
+    return (long long)o * B.ld_outer + (long long)(r - o * B.mid) * B.ld + c;
+  }
+  return (long long)r * B.ld + c;
+}
+__device__ __forceinline__ long long direction_offset(const BlockDev& B, int e) {
+  if (B.p_like_grad) return view_offset(B, e);
+  return (B.p_ld == B.cols) ? (long long)e : (long long)(e / B.cols) * B.p_ld + (e % B.cols);
+}
 
 struct ChunkRef { int block; int start; };
 
@@ -134,7 +156,6 @@ __global__ __launch_bounds__(EW_THREADS) void grafting_kernel(const BlockDev* __
   const bool has_m = B.filtered_grad != nullptr, has_v = B.adagrad != nullptr;
   const bool has_mom = B.momentum != nullptr && s.momentum != 0.0f;
   const bool b3 = B.ghat_tmp != nullptr;
-  const bool contig = (B.ld == B.cols);
   float gsum = 0.f, hsum = 0.f;
   constexpr int NIT = EW_CHUNK / (EW_THREADS * 4);
   // Whole, vectorisable chunk (the common case): every load is issued before the first use, so each
@@ -146,7 +167,7 @@ __global__ __launch_bounds__(EW_THREADS) void grafting_kernel(const BlockDev* __
 #pragma unroll
     for (int it = 0; it < NIT; ++it) {
       const int e = cr.start + (it * EW_THREADS + threadIdx.x) * 4;
-      gi[it] = contig ? (long long)e : (long long)(e / B.cols) * B.ld + (e % B.cols);
+      gi[it] = view_offset(B, e);
       g[it] = nt_load4(B.grad + gi[it]);
     }
 #pragma unroll
@@ -187,7 +208,7 @@ __global__ __launch_bounds__(EW_THREADS) void grafting_kernel(const BlockDev* __
   for (int it = 0; it < NIT; ++it) {
     const int e = cr.start + (it * EW_THREADS + threadIdx.x) * 4;
     if (e >= n_el) continue;
-    const long long gi = contig ? (long long)e : (long long)(e / B.cols) * B.ld + (e % B.cols);
+    const long long gi = view_offset(B, e);
     const bool vec = (e + 3 < n_el) && (B.vec != 0);
     if (vec) {
       float4 g = *reinterpret_cast<const float4*>(B.grad + gi);
@@ -217,7 +238,7 @@ __global__ __launch_bounds__(EW_THREADS) void grafting_kernel(const BlockDev* __
     } else {
       for (int k = 0; k < 4 && e + k < n_el; ++k) {
         const int ee = e + k;
-        const long long gk = contig ? (long long)ee : (long long)(ee / B.cols) * B.ld + (ee % B.cols);
+        const long long gk = view_offset(B, ee);
         float g = B.grad[gk];
         float m = has_m ? B.filtered_grad[ee] : 0.f;
         float v = has_v ? B.adagrad[ee] : 0.f;
@@ -287,8 +308,6 @@ __global__ __launch_bounds__(EW_THREADS) void apply_kernel(const BlockDev* __res
   const BlockDev& B = blocks[cr.block];
   const int n_el = B.rows * B.cols;
   const bool has_mom = B.momentum != nullptr && s.momentum != 0.0f;
-  const bool contig = (B.ld == B.cols);
-  const bool p_contig = (B.p_ld == B.cols);
   const float p_div = B.p_is_ghat ? s.bias_correction1 : 1.0f;
   float scale = 1.0f;
   if (s.graft_type != SA_GRAFT_NONE) {
@@ -304,8 +323,8 @@ __global__ __launch_bounds__(EW_THREADS) void apply_kernel(const BlockDev* __res
 #pragma unroll
     for (int it = 0; it < NIT; ++it) {
       const int e = cr.start + (it * EW_THREADS + threadIdx.x) * 4;
-      wi[it] = contig ? (long long)e : (long long)(e / B.cols) * B.ld + (e % B.cols);
-      const long long pi = p_contig ? (long long)e : (long long)(e / B.cols) * B.p_ld + (e % B.cols);
+      wi[it] = view_offset(B, e);
+      const long long pi = direction_offset(B, e);
       p[it] = nt_load4(B.p_src + pi);
       w[it] = nt_load4(B.param + wi[it]);
       mo[it] = has_mom ? nt_load4(B.momentum + e) : make_float4(0, 0, 0, 0);
@@ -325,8 +344,8 @@ __global__ __launch_bounds__(EW_THREADS) void apply_kernel(const BlockDev* __res
   for (int it = 0; it < NIT; ++it) {
     const int e = cr.start + (it * EW_THREADS + threadIdx.x) * 4;
     if (e >= n_el) continue;
-    const long long wi = contig ? (long long)e : (long long)(e / B.cols) * B.ld + (e % B.cols);
-    const long long pi = p_contig ? (long long)e : (long long)(e / B.cols) * B.p_ld + (e % B.cols);
+    const long long wi = view_offset(B, e);
+    const long long pi = direction_offset(B, e);
     const bool vec = (e + 3 < n_el) && (B.vec != 0) && (B.p_vec != 0);
     if (vec) {
       float4 p = *reinterpret_cast<const float4*>(B.p_src + pi);
@@ -341,8 +360,8 @@ __global__ __launch_bounds__(EW_THREADS) void apply_kernel(const BlockDev* __res
     } else {
       for (int k = 0; k < 4 && e + k < n_el; ++k) {
         const int ee = e + k;
-        const long long wk = contig ? (long long)ee : (long long)(ee / B.cols) * B.ld + (ee % B.cols);
-        const long long pk = p_contig ? (long long)ee : (long long)(ee / B.cols) * B.p_ld + (ee % B.cols);
+        const long long wk = view_offset(B, ee);
+        const long long pk = direction_offset(B, ee);
         float w = B.param[wk];
         float mo = has_mom ? B.momentum[ee] : 0.f;
         apply_element(B.p_src[pk] / p_div, w, mo, s, scale, has_mom);
@@ -353,17 +372,39 @@ __global__ __launch_bounds__(EW_THREADS) void apply_kernel(const BlockDev* __res
   }
 }
 
+// Dense (and dim-1-first) copies of the gradient of every order-3 block.  which = 0: for the factor updates
+// (g3_dense, g3_perm); which = 1: for the mode products of a step without filtered gradient (g3_ghat).
+__global__ __launch_bounds__(EW_THREADS) void gather3_kernel(const BlockDev* __restrict__ blocks,
+                                                            const ChunkRef* __restrict__ chunks, int which) {
+  const ChunkRef cr = chunks[blockIdx.x];
+  const BlockDev& B = blocks[cr.block];
+  if (B.mid <= 0) return;
+  float* dense = which == 0 ? B.g3_dense : B.g3_ghat;
+  float* perm = which == 0 ? B.g3_perm : nullptr;
+  if (dense == nullptr && perm == nullptr) return;
+  const int n_el = B.rows * B.cols, d0 = B.rows / B.mid;
+  for (int it = 0; it < EW_CHUNK / EW_THREADS; ++it) {
+    const int e = cr.start + it * EW_THREADS + threadIdx.x;
+    if (e >= n_el) break;
+    const float v = B.grad[view_offset(B, e)];
+    if (dense) dense[e] = v;
+    if (perm) {
+      const int r = e / B.cols, c = e - r * B.cols, i0 = r / B.mid, i1 = r - i0 * B.mid;
+      perm[((long long)i1 * d0 + i0) * B.cols + c] = v;
+    }
+  }
+}
+
 // G += wd * W in place on the gradient.
 __global__ __launch_bounds__(EW_THREADS) void l2_kernel(const BlockDev* __restrict__ blocks,
                                                        const ChunkRef* __restrict__ chunks, float wd) {
   const ChunkRef cr = chunks[blockIdx.x];
   const BlockDev& B = blocks[cr.block];
   const int n_el = B.rows * B.cols;
-  const bool contig = (B.ld == B.cols);
   for (int it = 0; it < EW_CHUNK / EW_THREADS; ++it) {
     const int e = cr.start + it * EW_THREADS + threadIdx.x;
     if (e >= n_el) break;
-    const long long gi = contig ? (long long)e : (long long)(e / B.cols) * B.ld + (e % B.cols);
+    const long long gi = view_offset(B, e);
     B.grad[gi] = B.grad[gi] + wd * B.param[gi];
   }
 }

@@ -221,7 +221,7 @@ struct sa_plan {
   bool tables_valid = false;
   int table_mode = -1;  // 0: ghat from grad, 1: from filtered_grad, 2: from the beta3 temporary
   std::vector<Factor> factors;
-  std::vector<int> block_factor[2];
+  std::vector<int> block_factor[SA_MAX_ORDER];
   std::vector<long long> elem_off;
   std::vector<int> chunk_begin_all, ptile_begin_all;  // per block, over ALL blocks (fixed layout)
   long long total_elems = 0, dense_total = 0, norm_partials_total = 0;
@@ -242,6 +242,9 @@ struct sa_plan {
   // Newton, [0] full products / [1] symmetric products: X*M_p with M_p^2 per parity, power chain, M update per parity
   GemmTable nt_a[2][2], nt_pow[2][8], nt_m[2][2];
   GemmTable nt_h[8];      // Horner products of the higher-order iteration
+  // mode products of order-3 blocks: [mode 1 | mode 0 | mode 2][first stage (divides by bias_correction1)][last stage (norm)]
+  GemmTable g3[3][2][2];
+  bool has_order3 = false;
   Table<HoJob> t_ho;
   std::vector<int> newton_history;  // per factor: iterations of its last converged solve, 0 = none
   Table<SymFactor> t_sym;
@@ -352,20 +355,36 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
     B.ld = d.ld;
     B.rows = d.rows;
     B.cols = d.cols;
+    B.mid = d.mid;
+    B.ld_outer = d.ld_outer;
     const long long eo = p->elem_off[b];
+    // a block is preconditioned if a side has a Kronecker factor or, for eigenvalue-corrected Shampoo, a fixed basis
+    const bool precond = p->block_factor[0][b] >= 0 || p->block_factor[1][b] >= 0 || p->block_factor[2][b] >= 0 ||
+                         (d.corrected_eigenvalues && (d.eigenvectors[0] || d.eigenvectors[1]));
     B.ghat_tmp = (mode == 2) ? ghbuf(p) + eo : nullptr;
-    if (mode == 0) { B.ghat_src = B.grad; B.ghat_ld = d.ld; }
+    if (mode == 0) {
+      if (d.mid > 0 && precond) {
+        // the mode products of an order-3 block read a dense copy of the gradient (gathered before they run)
+        B.ghat_src = ghbuf(p) + eo; B.ghat_ld = d.cols;
+        B.g3_ghat = ghbuf(p) + eo;
+      } else {
+        B.ghat_src = B.grad; B.ghat_ld = d.ld;
+      }
+    }
     else if (mode == 1) { B.ghat_src = d.filtered_grad; B.ghat_ld = d.cols; }
     else { B.ghat_src = ghbuf(p) + eo; B.ghat_ld = d.cols; }
-    // a block is preconditioned if a side has a Kronecker factor or, for eigenvalue-corrected Shampoo, a fixed basis
-    const bool precond = p->block_factor[0][b] >= 0 || p->block_factor[1][b] >= 0 ||
-                         (d.corrected_eigenvalues && (d.eigenvectors[0] || d.eigenvectors[1]));
     B.p_is_ghat = precond ? 0 : 1;
     if (precond) { B.p_src = pbuf(p) + eo; B.p_ld = d.cols; }
-    else { B.p_src = B.ghat_src; B.p_ld = B.ghat_ld; }
-    const bool contig = (d.ld == d.cols);
+    else { B.p_src = B.ghat_src; B.p_ld = B.ghat_ld; B.p_like_grad = (B.ghat_src == B.grad) ? 1 : 0; }
+    if (d.mid > 0 && block_active(p, b)) {
+      // dense copies for the factor updates: d0 x (d1 d2) in the T buffer, d1 x (d0 d2) in the P buffer
+      if (d.factor[0] || d.factor[2]) B.g3_dense = tbuf(p) + eo;
+      if (d.factor[1]) B.g3_perm = pbuf(p) + eo;
+    }
+    const bool contig = (d.ld == d.cols) && (d.mid == 0 || d.ld_outer == (long long)d.mid * d.ld);
+    B.contig = contig ? 1 : 0;
     auto al = [](const void* q) { return q == nullptr || (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
-    const bool shape_ok = contig || (d.cols % 4 == 0 && d.ld % 4 == 0);
+    const bool shape_ok = contig || (d.cols % 4 == 0 && d.ld % 4 == 0 && (d.mid == 0 || d.ld_outer % 4 == 0));
     B.vec = (shape_ok && al(B.param) && al(B.grad) && al(B.filtered_grad) && al(B.adagrad) && al(B.momentum) &&
              al(B.ghat_tmp)) ? 1 : 0;
     const bool p_contig = (B.p_ld == d.cols);
@@ -396,6 +415,23 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
   for (int b : active) {
     const sa_block_desc& d = p->blocks[b];
     const float* G = p->grads[b];
+    if (d.mid > 0) {
+      // order 3, from the dense copies: factor k = unfolding_k unfolding_k^T
+      const BlockDev& B = p->t_blocks.host[b];
+      const int d0 = d.rows / d.mid, d1 = d.mid, d2 = d.cols;
+      auto gram = [&](const float* T, long long ld, int dim, int K, float* C, bool k_major) {
+        GemmProblem q{};
+        q.A = T; q.B = T; q.C = C;
+        q.lda = ld; q.ldb = ld; q.ldc = 0;
+        q.M = dim; q.N = dim; q.K = K;
+        q.a_vec = q.b_vec = vec_ok(T, ld);
+        (k_major ? p->syrk1 : p->syrk0).add(q, true);
+      };
+      if (d.factor[0]) gram(B.g3_dense, (long long)d1 * d2, d0, d1 * d2, d.factor[0], false);
+      if (d.factor[1]) gram(B.g3_perm, (long long)d0 * d2, d1, d0 * d2, d.factor[1], false);
+      if (d.factor[2]) gram(B.g3_dense, d2, d2, d0 * d1, d.factor[2], true);
+      continue;
+    }
     if (d.factor[0]) {  // L = G G^T  (rows x rows, K = cols)
       GemmProblem q{};
       q.A = G; q.B = G; q.C = d.factor[0];
@@ -468,13 +504,66 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
 
   // preconditioning tables (root-inverse Shampoo)
   p->g1_store.clear(); p->g1_norm.clear(); p->g2_norm.clear(); p->g2g_norm.clear();
+  for (auto& a : p->g3) for (auto& b2 : a) for (auto& g : b2) g.clear();
   for (int b : active) {
     if (p->eigenvalue_corrected) break;
     const sa_block_desc& d = p->blocks[b];
-    const BlockDev& B = p->t_blocks.host[b];
+    BlockDev& B = p->t_blocks.host[b];
     const int f0 = p->block_factor[0][b], f1 = p->block_factor[1][b];
     const long long eo = p->elem_off[b];
     float* part = p->f(p->off_ptile_partial) + p->ptile_begin_all[b];
+    if (d.mid > 0) {
+      // P = Ghat x_1 X1 x_0 X0 x_2 X2 on dense buffers (mode products commute; each dim keeps its place)
+      const int f2 = p->block_factor[2][b];
+      const int d0 = d.rows / d.mid, d1 = d.mid, d2 = d.cols;
+      const int kinds[3] = {f1, f0, f2};  // stage order: mode 1, mode 0, mode 2
+      int n_stages = 0;
+      for (int k : kinds) n_stages += k >= 0 ? 1 : 0;
+      const float* src = B.ghat_src;  // dense d0 x d1 x d2
+      float* pong[2] = {tbuf(p) + eo, t2buf(p) + eo};
+      int done = 0;
+      for (int kind = 0; kind < 3; ++kind) {
+        if (kinds[kind] < 0) continue;
+        const Factor& F = p->factors[kinds[kind]];
+        const float* X = p->f(p->off_inv_dense) + F.dense_off;
+        const bool first = done == 0, last = done == n_stages - 1;
+        float* out = last ? pbuf(p) + eo : pong[done & 1];
+        GemmTable& tab = p->g3[kind][first ? 1 : 0][last ? 1 : 0];
+        auto tile_count = [](long long m, long long n) { return (int)(((m + BM - 1) / BM) * ((n + BN - 1) / BN)); };
+        if (kind == 0) {  // every slice i0: X1 (d1 x d1) . src[i0] (d1 x d2)
+          const int per = tile_count(d1, d2);
+          for (int i0 = 0; i0 < d0; ++i0) {
+            GemmProblem q{};
+            q.A = X; q.lda = F.dpad; q.a_vec = 1;
+            q.B = src + (long long)i0 * d1 * d2; q.ldb = d2; q.b_vec = vec_ok(q.B, q.ldb);
+            q.C = out + (long long)i0 * d1 * d2; q.ldc = d2;
+            q.M = d1; q.N = d2; q.K = d1;
+            if (last) q.C2 = part + (long long)i0 * per;
+            tab.add(q, false);
+          }
+          if (last) B.ptile_end = B.ptile_begin + d0 * per;
+        } else if (kind == 1) {  // X0 (d0 x d0) . src as d0 x (d1 d2)
+          GemmProblem q{};
+          q.A = X; q.lda = F.dpad; q.a_vec = 1;
+          q.B = src; q.ldb = (long long)d1 * d2; q.b_vec = vec_ok(q.B, q.ldb);
+          q.C = out; q.ldc = (long long)d1 * d2;
+          q.M = d0; q.N = d1 * d2; q.K = d0;
+          if (last) { q.C2 = part; B.ptile_end = B.ptile_begin + tile_count(d0, (long long)d1 * d2); }
+          tab.add(q, false);
+        } else {  // src as (d0 d1) x d2 . X2 (d2 x d2)
+          GemmProblem q{};
+          q.A = src; q.lda = d2; q.a_vec = vec_ok(q.A, q.lda);
+          q.B = X; q.ldb = F.dpad; q.b_vec = 1;
+          q.C = out; q.ldc = d2;
+          q.M = d0 * d1; q.N = d2; q.K = d2;
+          if (last) { q.C2 = part; B.ptile_end = B.ptile_begin + tile_count((long long)d0 * d1, d2); }
+          tab.add(q, false);
+        }
+        src = out;
+        ++done;
+      }
+      continue;
+    }
     if (f0 >= 0) {
       const Factor& F = p->factors[f0];
       GemmProblem q{};
@@ -504,6 +593,8 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
   SACHECK(p->g1_norm.commit(s));
   SACHECK(p->g2_norm.commit(s));
   SACHECK(p->g2g_norm.commit(s));
+  for (auto& a : p->g3) for (auto& b2 : a) for (auto& g : b2) SACHECK(g.commit(s));
+  if (p->has_order3) SACHECK(p->t_blocks.upload(s));  // ptile ranges of order-3 blocks were set above
   p->tables_valid = true;
   p->table_mode = mode;
   return SA_OK;
@@ -565,7 +656,8 @@ int refresh_inverse_cache(sa_plan* p, hipStream_t s) {
 extern "C" {
 
 const char* sa_last_error(void) { return g_err.c_str(); }
-int32_t sa_abi_version(void) { return 1; }
+int32_t sa_abi_version(void) { return 2; }
+static_assert(sizeof(sa_block_desc) == 160, "sa_block_desc layout changed: bump sa_abi_version and the ctypes mirror");
 
 int32_t sa_set_profiling(int32_t enabled) {
   g_profiling = enabled != 0;
@@ -622,8 +714,7 @@ int32_t sa_plan_create(const sa_block_desc* blocks, int32_t n_blocks, sa_plan** 
   p->n_blocks = n_blocks;
   p->blocks.assign(blocks, blocks + n_blocks);
   p->grads.assign(n_blocks, nullptr);
-  p->block_factor[0].assign(n_blocks, -1);
-  p->block_factor[1].assign(n_blocks, -1);
+  for (auto& bf : p->block_factor) bf.assign(n_blocks, -1);
   p->elem_off.resize(n_blocks);
   p->chunk_begin_all.resize(n_blocks + 1);
   p->ptile_begin_all.resize(n_blocks + 1);
@@ -639,13 +730,34 @@ int32_t sa_plan_create(const sa_block_desc* blocks, int32_t n_blocks, sa_plan** 
       delete p;
       return fail(SA_ERR_UNSUPPORTED, "sa_plan_create: block with 2^31 or more elements");
     }
+    if (d.mid < 0 || (d.mid > 0 && (d.rows % d.mid != 0 || d.ld_outer < (long long)d.mid * d.ld))) {
+      delete p;
+      return fail(SA_ERR_INVALID, "sa_plan_create: block " + std::to_string(b) + " has a bad order-3 shape (mid, ld_outer)");
+    }
+    if (d.mid == 0 && (d.factor[2] || d.eigenvectors[2])) {
+      delete p;
+      return fail(SA_ERR_INVALID, "sa_plan_create: a third factor needs an order-3 block (mid > 0)");
+    }
+    if (d.mid > 0 && (d.corrected_eigenvalues || d.eigenvectors[0] || d.eigenvectors[1] || d.eigenvectors[2])) {
+      delete p;
+      return fail(SA_ERR_UNSUPPORTED, "sa_plan_create: eigenvalue-corrected blocks of order 3 are not built");
+    }
+    if (d.mid > 0) p->has_order3 = true;
     p->elem_off[b] = eo;
     eo += round_up((long long)d.rows * d.cols, 64);
     p->chunk_begin_all[b] = chunks;
     chunks += (int)(((long long)d.rows * d.cols + EW_CHUNK - 1) / EW_CHUNK);
     p->ptile_begin_all[b] = ptiles;
-    ptiles += ((d.rows + BM - 1) / BM) * ((d.cols + BN - 1) / BN);
-    for (int side = 0; side < 2; ++side) {
+    {
+      auto tiles = [](long long m, long long n) { return (int)(((m + BM - 1) / BM) * ((n + BN - 1) / BN)); };
+      int need = tiles(d.rows, d.cols);
+      if (d.mid > 0) {  // the last mode product of an order-3 block may be any of the three
+        const int d0 = d.rows / d.mid;
+        need = std::max(need, std::max(d0 * tiles(d.mid, d.cols), tiles(d0, (long long)d.mid * d.cols)));
+      }
+      ptiles += need;
+    }
+    for (int side = 0; side < SA_MAX_ORDER; ++side) {
       if (!d.factor[side]) {
         if (d.eigenvectors[side] && d.corrected_eigenvalues) p->eigenvalue_corrected = true;  // fixed basis
         continue;
@@ -660,7 +772,8 @@ int32_t sa_plan_create(const sa_block_desc* blocks, int32_t n_blocks, sa_plan** 
       }
       Factor f{};
       f.block = b; f.side = side;
-      f.d = side == 0 ? d.rows : d.cols;
+      if (d.mid > 0) f.d = side == 0 ? d.rows / d.mid : (side == 1 ? d.mid : d.cols);
+      else f.d = side == 0 ? d.rows : d.cols;
       f.dpad = (int)round_up(f.d, BM);
       f.root = d.root[side];
       f.factor = d.factor[side];
@@ -709,6 +822,7 @@ void sa_plan_destroy(sa_plan* p) {
     g->t.destroy();
   for (auto& row : p->nt_pow) for (auto& g : row) g.t.destroy();
   for (auto& g : p->nt_h) g.t.destroy();
+  for (auto& a : p->g3) for (auto& b2 : a) for (auto& g : b2) g.t.destroy();
   p->t_ho.destroy();
   p->t_sym.destroy(); p->t_normjobs.destroy(); p->t_ids.destroy();
   p->t_jacobi.destroy(); p->t_sched.destroy(); p->t_eiginit.destroy(); p->t_eigfinal.destroy(); p->eig_gemm.t.destroy();
@@ -782,6 +896,10 @@ int32_t sa_update_factor_matrices(sa_plan* p, float beta2, float weighting_facto
   for (const GemmTable* g : {&p->syrk0, &p->syrk1})
     for (const GemmProblem& q : g->build) flops += (double)q.N * q.N * q.K;  // symmetric half: d^2 k
   int launches = (p->syrk0.total_tiles ? 1 : 0) + (p->syrk1.total_tiles ? 1 : 0);
+  if (p->has_order3 && p->t_chunks.n) {
+    hipLaunchKernelGGL(gather3_kernel, dim3((unsigned)p->t_chunks.n), dim3(EW_THREADS), 0, s, p->t_blocks.dev, p->t_chunks.dev, 0);
+    HIPCHECK(hipGetLastError());
+  }
   Span span("syrk", s, flops, launches, true);
   SACHECK((launch_gemm_auto<A_MK, B_NK, EPI_SYRK_EMA>(p->syrk0, sc, s)));
   SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_SYRK_EMA>(p->syrk1, sc, s)));
@@ -833,6 +951,14 @@ int32_t sa_precondition(sa_plan* p, const sa_step_scalars* sc, void* stream) {
     for (const GemmProblem& q : g->build) flops += 2.0 * q.M * q.N * q.K;
     launches += g->total_tiles ? 1 : 0;
   }
+  for (auto& a : p->g3) for (auto& b2 : a) for (auto& g : b2) {
+    for (const GemmProblem& q : g.build) flops += 2.0 * q.M * q.N * q.K;
+    launches += g.total_tiles ? 1 : 0;
+  }
+  if (p->has_order3 && p->table_mode == 0 && p->t_chunks.n) {
+    hipLaunchKernelGGL(gather3_kernel, dim3((unsigned)p->t_chunks.n), dim3(EW_THREADS), 0, s, p->t_blocks.dev, p->t_chunks.dev, 1);
+    HIPCHECK(hipGetLastError());
+  }
   {
     Span span("precondition_gemm", s, flops, launches, true);
     GemmScalars a = unit_scalars();
@@ -843,6 +969,14 @@ int32_t sa_precondition(sa_plan* p, const sa_step_scalars* sc, void* stream) {
     GemmScalars c = unit_scalars();
     c.a_div = sc->bias_correction1;
     SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE_SQNORM>(p->g2g_norm, c, s)));
+    // order-3 blocks: mode 1, mode 0, mode 2; the stage that reads the filtered gradient divides it
+    for (int kind = 0; kind < 3; ++kind)
+      for (int first = 0; first < 2; ++first) {
+        GemmScalars g = unit_scalars();
+        if (first) (kind == 2 ? g.a_div : g.b_div) = sc->bias_correction1;
+        SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE>(p->g3[kind][first][0], g, s)));
+        SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE_SQNORM>(p->g3[kind][first][1], g, s)));
+      }
   }
   if (p->n_active_blocks) {
     hipLaunchKernelGGL(reduce_norms_kernel, dim3(p->n_active_blocks), dim3(EW_THREADS), 0, s, p->t_blocks.dev,
@@ -912,24 +1046,30 @@ int32_t sa_plan_read_preconditioned(sa_plan* p, int32_t block, float* out, void*
 // Batched coupled inverse Newton
 // --------------------------------------------------------------------------------------------
 
+// Products that raise a matrix to the power `root` by left-to-right binary exponentiation: after the leading bit,
+// every lower bit is a squaring ('S'), followed by a product with the base ('M') when the bit is set.
+// The first squaring shares a launch with X M_p; at most four further products fit the per-iteration tables.
+static int power_ops(int root, std::vector<char>* ops) {
+  ops->clear();
+  if (root < 1) return fail(SA_ERR_INVALID, "root must be positive");
+  int top = 0;
+  while ((root >> (top + 1)) != 0) ++top;
+  for (int bit = top - 1; bit >= 0; --bit) {
+    ops->push_back('S');
+    if ((root >> bit) & 1) ops->push_back('M');
+  }
+  if (ops->size() > 5) return fail(SA_ERR_UNSUPPORTED, "root " + std::to_string(root) + " needs too many products for the power chain");
+  return SA_OK;
+}
+
 // `symmetric[i]` selects the product variant of ids[i].
 static int newton_batch(sa_plan* p, const std::vector<int>& ids, const std::vector<char>& symmetric, int root, float eps,
                         float bc2, int max_iter, float tol, hipStream_t s, double* flops_acc, int* launches_acc) {
   const int n = (int)ids.size();
   if (n == 0) return SA_OK;
-  // torch.linalg.matrix_power(M_p, root): squarings (and one extra product for root 3)
-  int squarings = 0;
-  bool cube = false;
-  if (root == 3) { squarings = 1; cube = true; }
-  else {
-    int r = root;
-    while (r > 1) {
-      if (r & 1) return fail(SA_ERR_UNSUPPORTED, "coupled Newton is built for roots 1, 2, 3 and powers of two; got " + std::to_string(root));
-      r >>= 1;
-      ++squarings;
-    }
-  }
-  if (std::max(squarings - 1, 0) + (cube ? 1 : 0) > 4) return fail(SA_ERR_UNSUPPORTED, "root too large for the power chain");
+  // torch.linalg.matrix_power(M_p, root) as a chain of products
+  std::vector<char> ops;
+  SACHECK(power_ops(root, &ops));
   const float alpha = (float)(-1.0 / root);          // M.mul(alpha)
   const float one_minus_alpha = (float)(1.0 - (-1.0 / root));  // .add_(I, alpha = 1 - alpha)
 
@@ -992,20 +1132,16 @@ static int newton_batch(sa_plan* p, const std::vector<int>& ids, const std::vect
       float* S2 = newton_buf(p, NB_S2, f);
       // launch A: X <- X M_p, and the first squaring if the root needs one
       p->nt_a[v][par].add(prob(f, X, Mp, Xn), sym);
-      if (squarings >= 1) p->nt_a[v][par].add(prob(f, Mp, Mp, S1), sym);
-      // remaining chain reads only S1/S2/Mp of this parity; build it for parity-specific Mp when cube
-      const float* cur = (squarings >= 1) ? S1 : Mp;
+      if (!ops.empty()) p->nt_a[v][par].add(prob(f, Mp, Mp, S1), sym);
+      // the remaining chain reads only S1 / S2 / M_p of this parity
+      const float* cur = ops.empty() ? Mp : S1;
       int slot = par * 4;  // nt_pow[0..3] parity 0, [4..7] parity 1
       float* pong[2] = {S2, S1};
       int which = 0;
-      for (int q = 1; q < squarings; ++q) {
-        p->nt_pow[v][slot++].add(prob(f, cur, cur, pong[which]), sym);
+      for (size_t q = 1; q < ops.size(); ++q) {
+        p->nt_pow[v][slot++].add(prob(f, cur, ops[q] == 'S' ? cur : Mp, pong[which]), sym);
         cur = pong[which];
         which ^= 1;
-      }
-      if (cube) {
-        p->nt_pow[v][slot++].add(prob(f, cur, Mp, pong[which]), sym);
-        cur = pong[which];
       }
       power = cur;
       GemmProblem m = prob(f, power, M, Mn);
@@ -1031,7 +1167,7 @@ static int newton_batch(sa_plan* p, const std::vector<int>& ids, const std::vect
   GemmScalars msc = unit_scalars();
   msc.mp_scale = alpha;
   msc.mp_diag = one_minus_alpha;
-  const int gemms_per_iter = 1 + squarings + (cube ? 1 : 0) + 1;
+  const int gemms_per_iter = 1 + (int)ops.size() + 1;
   for (int it = 0; it < max_iter; ++it) {
     double flops = 0.0, executed = 0.0;
     int live = 0;
@@ -1270,34 +1406,12 @@ int32_t sa_compute_root_inverses_newton(sa_plan* p, float bias_correction2, floa
 
 constexpr int HO_MAX_ORDER = 8;
 
-// Binary power chain of `base` for exponent `root` (1, 2, 3 or a power of two) into the S1 / S2 arrays of `f`;
-// stage k goes to `stages[k]`.  Returns the array that holds the power.
-struct PowerChain {
-  int squarings = 0;
-  bool cube = false;
-  int stages() const { return std::max(squarings - 1, 0) + (cube ? 1 : 0); }
-};
-static int power_chain_for(int root, PowerChain* pc) {
-  pc->squarings = 0; pc->cube = false;
-  if (root == 3) { pc->squarings = 1; pc->cube = true; return SA_OK; }
-  int r = root;
-  while (r > 1) {
-    if (r & 1) return fail(SA_ERR_UNSUPPORTED, "coupled iterations are built for roots 1, 2, 3 and powers of two; got " + std::to_string(root));
-    r >>= 1;
-    ++pc->squarings;
-  }
-  if (pc->stages() > 4) return fail(SA_ERR_UNSUPPORTED, "root too large for the power chain");
-  return SA_OK;
-}
-
 static int higher_order_batch(sa_plan* p, const std::vector<int>& ids, int root, int order, float rel_eps, float abs_eps,
                               float bc2, int max_iter, float tol, hipStream_t s, double* flops_acc, int* launches_acc) {
   const int n = (int)ids.size();
   if (n == 0) return SA_OK;
-  PowerChain pc;
-  SACHECK(power_chain_for(root, &pc));
-  const int squarings = pc.squarings;
-  const bool cube = pc.cube;
+  std::vector<char> ops;
+  SACHECK(power_ops(root, &ops));
   const int horner = order - 2;  // products that build M_p from I - M
   // b_0 = 1, b_i = b_{i-1} (1 + (i - 1) p) / (i p): exact integer products, one division per entry
   std::vector<double> b(order, 1.0);
@@ -1365,19 +1479,15 @@ static int higher_order_batch(sa_plan* p, const std::vector<int>& ids, int root,
       const float* Mp = (order == 2 && par == 1) ? Mp0 : Mp1;
       float* seed = (order == 2 && par == 1) ? Mp1 : Mp0;
       p->nt_a[0][par].add(prob(f, X, Mp, Xn), false);
-      if (squarings >= 1) p->nt_a[0][par].add(prob(f, Mp, Mp, S1), false);
-      const float* cur = (squarings >= 1) ? S1 : Mp;
+      if (!ops.empty()) p->nt_a[0][par].add(prob(f, Mp, Mp, S1), false);
+      const float* cur = ops.empty() ? Mp : S1;
       int slot = par * 4;
       float* pong[2] = {S2, S1};
       int which = 0;
-      for (int q = 1; q < squarings; ++q) {
-        p->nt_pow[0][slot++].add(prob(f, cur, cur, pong[which]), false);
+      for (size_t q = 1; q < ops.size(); ++q) {
+        p->nt_pow[0][slot++].add(prob(f, cur, ops[q] == 'S' ? cur : Mp, pong[which]), false);
         cur = pong[which];
         which ^= 1;
-      }
-      if (cube) {
-        p->nt_pow[0][slot++].add(prob(f, cur, Mp, pong[which]), false);
-        cur = pong[which];
       }
       GemmProblem m = prob(f, cur, M, Mn);
       m.C2 = seed;
@@ -1409,7 +1519,7 @@ static int higher_order_batch(sa_plan* p, const std::vector<int>& ids, int root,
   if (order == 2) { msc.mp_scale = (float)(-b[1]); msc.mp_diag = (float)(b[1] + b[0]); }
   else { msc.mp_scale = -1.0f; msc.mp_diag = 1.0f; }
   for (int it = 0; it <= max_iter; ++it) {
-    const int gemms = 1 + squarings + (cube ? 1 : 0) + 1 + (it >= 1 ? horner : 0);
+    const int gemms = 1 + (int)ops.size() + 1 + (it >= 1 ? horner : 0);
     double flops = 0.0;
     int live = 0;
     for (int i = 0; i < n; ++i)
@@ -1456,8 +1566,8 @@ static int higher_order_residuals(sa_plan* p, const std::vector<int>& ids, const
                                   hipStream_t s) {
   const int n = (int)ids.size();
   if (n == 0) return SA_OK;
-  PowerChain pc;
-  SACHECK(power_chain_for(root, &pc));
+  std::vector<char> ops;
+  SACHECK(power_ops(root, &ops));
   SACHECK(p->t_eiginit.begin(n));
   SACHECK(p->t_ho.begin(n));
   int tiles = 0, dpadmax = 0;
@@ -1499,14 +1609,10 @@ static int higher_order_residuals(sa_plan* p, const std::vector<int>& ids, const
     int slot = 0;
     float* pong[2] = {S1, S2};
     int which = 0;
-    for (int q = 0; q < pc.squarings; ++q) {
-      p->nt_pow[0][slot++].add(prob(cur, cur, pong[which]), false);
+    for (char op : ops) {
+      p->nt_pow[0][slot++].add(prob(cur, op == 'S' ? cur : X, pong[which]), false);
       cur = pong[which];
       which ^= 1;
-    }
-    if (pc.cube) {
-      p->nt_pow[0][slot++].add(prob(cur, X, pong[which]), false);
-      cur = pong[which];
     }
     GemmProblem m = prob(newton_buf(p, NB_MP0, f), cur, newton_buf(p, par[ids[i]] ? NB_M0 : NB_M1, f));
     m.C2 = newton_buf(p, NB_MP1, f);

@@ -251,9 +251,13 @@ class _NativeGroup(_AmortizedComputation):
             self.num_blocks_per_param.append(len(specs))
             self.block_specs.extend(specs)
         for s in self.block_specs:
-            if s.order > 2:
+            if s.order > 3:
                 raise NotImplementedError(
-                    f"block of order {s.order} (shape {s.shape}): the native step covers blocks of order 1 and 2"
+                    f"block of order {s.order} (shape {s.shape}): the native step covers blocks of order 1 to 3"
+                )
+            if s.order == 3 and isinstance(pc, EigenvalueCorrectedShampooPreconditionerConfig):
+                raise NotImplementedError(
+                    f"block of order 3 (shape {s.shape}): eigenvalue-corrected Shampoo is built for blocks of order 1 and 2"
                 )
 
         # native blocks = blocks with at least one element
@@ -318,8 +322,11 @@ class _NativeGroup(_AmortizedComputation):
             d = descs[k]
             if s.order == 1:
                 d.rows, d.cols, d.ld = s.shape[0], 1, 1
-            else:
+            elif s.order == 2:
                 d.rows, d.cols, d.ld = s.shape[0], s.shape[1], s.strides[0]
+            else:  # d0 x d1 x d2 flattened to (d0 d1) x d2
+                d.rows, d.cols, d.ld = s.shape[0] * s.shape[1], s.shape[2], s.strides[1]
+                d.mid, d.ld_outer = s.shape[1], s.strides[0]
             d.param = p.data_ptr() + 4 * s.offset
             shampoo_state: dict[str, Any] = (
                 {"factor_matrices": {}, "factor_matrices_eigenvectors": {}}
@@ -643,7 +650,8 @@ class DistributedShampoo(torch.optim.Optimizer):
     `EigenConfig` (`PerturbationConfig` and `PseudoInverseConfig`), `use_trace_scaling`, `EigenvalueCorrectedShampooPreconditionerConfig` with `QREigendecompositionConfig` or
     `EighEigendecompositionConfig` (including `ignored_basis_change_dims`), grafting with SGD / AdaGrad / RMSprop /
     Adam or none, every `WeightDecayType`, `ClassicMomentumConfig`, `inverse_exponent_override`,
-    `SingleDeviceDistributedConfig`, fp32 state with packed factor matrices, blocks of order 1 and 2.
+    `SingleDeviceDistributedConfig`, fp32 state with packed factor matrices, blocks of order 1 to 3 (order 3, e.g.
+    convolution weights, with root-inverse Shampoo only).
     Anything else raises NotImplementedError at construction.
     """
 

@@ -9,8 +9,8 @@ Differences from the reference, all at rounding level or documented limits:
  * input and output are fp32 tensors on a HIP device (there is no CPU path);
  * `matrix_inverse_root` returns the mirrored upper triangle of the solver's result, which is what the
    optimizer stores (shampoo_preconditioner_list.py:678);
- * `CoupledNewtonConfig` / `CoupledHigherOrderConfig` take roots 1, 2, 3 and powers of two, the higher-order
-   iteration no fractional roots;
+ * `CoupledNewtonConfig` / `CoupledHigherOrderConfig` take integer roots whose power chain has at most five
+   products (every root up to 14, and 16), the higher-order iteration no fractional roots;
  * `eigendecomposition_offload_device` must be "" and `retry_double_precision` is not needed (the solvers
    do not fail on finite input);
  * a non-finite input or result comes back as a matrix of NaN, where the reference's LAPACK call would raise.

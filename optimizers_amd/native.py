@@ -38,6 +38,9 @@ EXPORTS = (
 )
 
 
+SA_MAX_ORDER = 3
+
+
 class BlockDesc(ctypes.Structure):
     _fields_ = [
         ("rows", c_int32),
@@ -47,11 +50,13 @@ class BlockDesc(ctypes.Structure):
         ("filtered_grad", c_void_p),
         ("adagrad", c_void_p),
         ("momentum_buffer", c_void_p),
-        ("factor", c_void_p * 2),
-        ("inv_factor", c_void_p * 2),
-        ("root", c_int32 * 2),
-        ("eigenvectors", c_void_p * 2),
+        ("factor", c_void_p * SA_MAX_ORDER),
+        ("inv_factor", c_void_p * SA_MAX_ORDER),
+        ("root", c_int32 * SA_MAX_ORDER),
+        ("eigenvectors", c_void_p * SA_MAX_ORDER),
         ("corrected_eigenvalues", c_void_p),
+        ("mid", c_int32),
+        ("ld_outer", c_int64),
     ]
 
 

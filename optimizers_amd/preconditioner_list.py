@@ -9,7 +9,7 @@ distributed_shampoo.py:659-759) and expose its three operations (preconditioner/
     compress_preconditioner_list(local_grad_selector)
 
 Everything numerical runs in libshampoo_amd.so on the blocks' device; torch only allocates.  Limits of the native
-step apply: fp32, blocks of order 0..2, packed factor matrices, integer roots for the coupled iterations.
+step apply: fp32, blocks of order 0..3 (0..2 for the eigenvalue-corrected list), packed factor matrices, integer roots for the coupled iterations.
 """
 
 from __future__ import annotations
@@ -137,8 +137,8 @@ class _NativeShampooPreconditionerList(PreconditionerList, _AmortizedComputation
         for b in self._blocks:
             if b.device.type != "cuda" or b.dtype != torch.float32:
                 raise RuntimeError(f"the native preconditioner list runs on an MI355X only: fp32 blocks on a HIP device, got {b.dtype} on {b.device}")
-            if b.dim() > 2:
-                raise NotImplementedError(f"blocks of order {b.dim()} are not built natively")
+            if b.dim() > 3 or (b.dim() == 3 and self.soap):
+                raise NotImplementedError(f"blocks of order {b.dim()} are not built natively for this list")
         self.device = self._blocks[0].device if self._blocks else torch.device("cuda:0")
         acc = preconditioner_config.amortized_computation_config
         self.use_eigh = isinstance(acc, EigenConfig)
@@ -229,10 +229,16 @@ class _NativeShampooPreconditionerList(PreconditionerList, _AmortizedComputation
         self._destroy_plan()
 
     @staticmethod
-    def _row_stride(t: Tensor) -> int:
-        return 1 if t.dim() < 2 else max(int(t.stride(0)), int(t.shape[1]))
+    def _row_stride(t: Tensor) -> tuple[int, ...]:
+        """Strides the plan needs: (row stride,) of a matrix, (dim-0 stride, dim-1 stride) of an order-3 block."""
+        if t.dim() < 2:
+            return (1,)
+        if t.dim() == 2:
+            return (max(int(t.stride(0)), int(t.shape[1])),)
+        inner = max(int(t.stride(1)), int(t.shape[2]))
+        return (max(int(t.stride(0)), inner * int(t.shape[1])), inner)
 
-    def _ensure_plan(self, strides: tuple[int, ...]) -> None:
+    def _ensure_plan(self, strides: tuple[tuple[int, ...], ...]) -> None:
         """(Re)creates the plan when the row strides of the gradient blocks differ from the ones it was built for."""
         if self.plan and strides == self._plan_strides:
             return
@@ -243,8 +249,11 @@ class _NativeShampooPreconditionerList(PreconditionerList, _AmortizedComputation
         descs = (native.BlockDesc * nb)()
         for k, (block, st, selector) in enumerate(zip(self._blocks, self._states, self._selectors)):
             d = descs[k]
-            if block.dim() == 2:
-                d.rows, d.cols, d.ld = block.shape[0], block.shape[1], strides[k]
+            if block.dim() == 3:
+                d.rows, d.cols, d.ld = block.shape[0] * block.shape[1], block.shape[2], strides[k][1]
+                d.mid, d.ld_outer = block.shape[1], strides[k][0]
+            elif block.dim() == 2:
+                d.rows, d.cols, d.ld = block.shape[0], block.shape[1], strides[k][0]
             else:
                 d.rows, d.cols, d.ld = max(block.numel(), 1), 1, 1
             d.param = block.data_ptr()  # never written: only the factor update and the preconditioning run on this plan
@@ -284,8 +293,8 @@ class _NativeShampooPreconditionerList(PreconditionerList, _AmortizedComputation
                 raise ValueError(f"gradient block {k} has shape {tuple(g.shape)}, the parameter block {tuple(self._blocks[k].shape)}")
             if g.dtype != torch.float32 or g.device != self.device:
                 raise NotImplementedError("gradients must be fp32 on the blocks' device")
-            if g.dim() == 2 and g.stride(1) != 1 and g.shape[1] > 1:
-                raise NotImplementedError("gradient blocks must have unit column stride")
+            if g.dim() >= 2 and g.stride(-1) != 1 and g.shape[-1] > 1:
+                raise NotImplementedError("gradient blocks must have unit stride in their last dim")
             strides[k] = self._row_stride(g)
         self._ensure_plan(tuple(strides))
         ptrs = (ctypes.c_void_p * max(len(self._blocks), 1))()

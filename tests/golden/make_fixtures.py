@@ -128,6 +128,18 @@ CASES = {
         preconditioner="higher_order", override_1d=False, grafting=None,
         ho_order=5, ho_rel_epsilon=1e-3, ho_abs_epsilon=0.0,
     ),
+    "conv_like_eigh": dict(  # order-3 blocks (conv weights): splits along dim 0, the middle dim and the last dim
+        shapes=[[20, 6, 3, 3], [6, 20, 3, 3], [5, 4, 20], [7]], seed=10, grad_scale=1.0, steps=8,
+        lr=1e-2, betas=[0.9, 0.99], epsilon=1e-8, weight_decay=1e-3, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=16, precondition_frequency=2, start_preconditioning_step=4,
+        preconditioner="eigh", override_1d=True, grafting="adam", grafting_beta2=0.99, grafting_epsilon=1e-8,
+    ),
+    "conv_like_newton": dict(  # the same with the coupled Newton iteration (root 6) and no filtered gradient
+        shapes=[[20, 6, 3, 3], [6, 20, 3, 3], [5, 4, 20], [7]], seed=11, grad_scale=1.0, steps=8,
+        lr=1e-2, betas=[0.0, 0.99], epsilon=1e-6, weight_decay=0.0, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=16, precondition_frequency=2, start_preconditioning_step=4,
+        preconditioner="newton", override_1d=True, grafting="adagrad", grafting_epsilon=1e-8,
+    ),
     "cfg1_override": dict(  # benchmark configuration 1 with 1-D blocks left to grafting
         shapes=[[512, 512], [512]], seed=0, grad_scale=1.0, steps=10, zero_init=True, torch_seed_grads=True,
         lr=1e-3, betas=[0.9, 0.999], epsilon=1e-12, weight_decay=0.0, weight_decay_type="DECOUPLED",

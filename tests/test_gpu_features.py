@@ -282,3 +282,43 @@ def test_zero_dimensional_empty_and_tiny_parameters(kind):
     # the 1-D block's factor has rank one with epsilon = 1e-4: loose bound, the others are well conditioned
     for p, r, tol in zip(params[2:], ref_p[2:], (5e-3, 1e-5, 1e-5)):
         assert rel_err(p.detach().cpu(), r) < tol
+
+
+@pytest.mark.parametrize("kind", ["newton", "eigh"])
+def test_order_three_blocks_with_every_kind_of_split(kind):
+    """A conv weight whose merged shape 192 x 160 x 9 splits (max_preconditioner_dim = 128) into four order-3
+    blocks, two of them views with a split middle dim, against the oracle for three steps."""
+    import optimizers_amd as oa
+    from oracle.shampoo_oracle import OracleConfig, ShampooOracle
+
+    g = torch.Generator().manual_seed(33)
+    shapes = [(192, 160, 3, 3), (40,)]
+    init = [0.1 * torch.randn(*s, generator=g) for s in shapes]
+    kw = dict(lr=1e-2, betas=(0.9, 0.99), epsilon=1e-6, max_preconditioner_dim=128, precondition_frequency=1,
+              start_preconditioning_step=2, weight_decay=1e-3)
+    acc = oa.CoupledNewtonConfig() if kind == "newton" else oa.EigenConfig()
+    params = [torch.nn.Parameter(t.clone().to(DEV)) for t in init]
+    opt = oa.DistributedShampoo(
+        params, preconditioner_config=oa.RootInvShampooPreconditionerConfig(
+            amortized_computation_config=acc, inverse_exponent_override={1: {0: 0.0}}),  # the rank-3 factor of the vector is left out
+        grafting_config=oa.AdamPreconditionerConfig(beta2=0.99, epsilon=1e-8), **kw)
+    assert [opt._groups[0].block_specs[i].shape for i in range(4)] == [(128, 128, 9), (128, 32, 9), (64, 128, 9), (64, 32, 9)]
+    ref_p = [t.clone() for t in init]
+    ref = ShampooOracle(ref_p, OracleConfig(preconditioner=kind, grafting="adam", grafting_beta2=0.99,
+                                            grafting_epsilon=1e-8, inverse_exponent_override={1: {0: 0.0}}, **kw))
+    for _ in range(3):
+        grads = [torch.randn(*s, generator=g) for s in shapes]
+        for q, gr in zip(params, grads):
+            q.grad = gr.to(DEV)
+        opt.step()
+        ref.step([x.clone() for x in grads])
+    ng = opt._groups[0]
+    for k, bi in enumerate(ng.native_index):
+        spec = ng.block_specs[bi]
+        st = opt.state[params[spec.param_index]][spec.block_key]
+        for j, f in enumerate(ref.state[bi]["factors"]):
+            assert rel_err(st["shampoo"]["factor_matrices"][j].cpu(), f) < 1e-5
+        for j, f in enumerate(ref.state[bi]["inv"]):
+            assert rel_err(st["shampoo"]["inv_factor_matrices"][j].cpu(), f) < 1e-3
+    for q, r in zip(params, ref_p):
+        assert rel_err(q.detach().cpu(), r) < 1e-4

@@ -247,3 +247,34 @@ def test_eigenvalue_corrected_list_matches_oracle_formulas(kind):
     rot = rot / ((v / (1 - 0.95**3)).sqrt() + 1e-8)
     want = Q[0] @ rot @ Q[1].T
     assert float((out.cpu().double() - want).norm() / want.norm()) < 1e-4
+
+
+def test_order_three_blocks():
+    """tensordot semantics of the reference for a conv-like block and a middle-dim split view of it
+    (shampoo_preconditioner_list.py:1490-1578), rebuilt in fp64."""
+    from optimizers_amd.preconditioner_list import BlockInfo, RootInvShampooPreconditionerList
+
+    g = torch.Generator().manual_seed(2)
+    param = torch.randn(12, 40, 9, generator=g).to(DEV)
+    blocks = torch.split(param, 32, dim=1)  # 12 x 32 x 9 and 12 x 8 x 9: the middle dim is split
+    state = {param: {"block_0": {}, "block_1": {}}}
+    infos = tuple(BlockInfo(param=param, composable_block_ids=(0, f"block_{k}")) for k in range(2))
+    pl = RootInvShampooPreconditionerList(block_list=blocks, state=state, block_info_list=infos,
+                                          preconditioner_config=_config("eigh"), beta2=1.0, weighting_factor=1.0, epsilon=1e-6)
+    assert state[param]["block_0"]["shampoo"].roots == (6.0, 6.0, 6.0)
+    grads = [torch.randn(12, 40, 9, generator=g) for _ in range(3)]
+    for step, G in enumerate(grads, start=1):
+        pl.update_preconditioners(masked_grad_list=torch.split(G.to(DEV), 32, dim=1), step=torch.tensor(step),
+                                  perform_amortized_computation=step == 3)
+    out = pl.precondition(masked_grad_list=torch.split(grads[-1].to(DEV), 32, dim=1))
+    for k, sl in enumerate((slice(0, 32), slice(32, 40))):
+        Gs = [G[:, sl, :].double() for G in grads]
+        want = Gs[-1]
+        for dim in range(3):
+            rest = [d for d in range(3) if d != dim]
+            F = sum(torch.tensordot(x, x, dims=[rest, rest]) for x in Gs)
+            lam, q = torch.linalg.eigh(F + 1e-6 * torch.eye(F.shape[0], dtype=torch.float64))
+            X = q * lam.pow(-1.0 / 6.0) @ q.T
+            want = torch.tensordot(want, X, dims=([0], [0]))  # contracts dim 0, appends the result: rotates the dims
+        assert out[k].shape == want.shape
+        assert float((out[k].cpu().double() - want).norm() / want.norm()) < 1e-3

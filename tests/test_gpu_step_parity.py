@@ -15,7 +15,10 @@ from tests.golden_cases import GOLDEN, grad_stream, initial_params, load_cases, 
 pytestmark = pytest.mark.gpu
 
 CASES = load_cases()
-NEWTON_CASES = [n for n, c in CASES.items() if c["preconditioner"] in ("newton", "higher_order") or c.get("use_trace_scaling")]
+NEWTON_CASES = [
+    n for n, c in CASES.items()
+    if c["preconditioner"] in ("newton", "higher_order") or c.get("use_trace_scaling") or n.startswith("conv_like")
+]
 
 
 def native_optimizer(c, params):
