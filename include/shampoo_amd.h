@@ -73,7 +73,7 @@ typedef struct sa_block_desc {
   float* factor[SA_MAX_ORDER];     /* packed upper-triangular Kronecker factor per dim; NULL = dim not preconditioned */
   float* inv_factor[SA_MAX_ORDER]; /* packed upper-triangular inverse root of that factor (root-inverse Shampoo), or NULL */
   int32_t root[SA_MAX_ORDER];      /* integer inverse root (2 * order by default: 2 for vectors, 4 for matrices, 6 for order 3) */
-  /* eigenvalue-corrected Shampoo / SOAP (shampoo_preconditioner_list.py:942-1007), blocks of order <= 2 only: dense
+  /* eigenvalue-corrected Shampoo / SOAP (shampoo_preconditioner_list.py:942-1007): dense
    * d x d eigenbasis of each factor (row-major, columns are eigenvectors) and the second moment kept in the rotated
    * basis (rows x cols, contiguous).  NULL for root-inverse Shampoo.  eigenvectors[k] with factor[k] == NULL is a
    * fixed basis: it rotates the block but has no statistics and is never refreshed (a block whose basis

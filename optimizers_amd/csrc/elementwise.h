@@ -45,6 +45,7 @@ struct BlockDev {
   float* g3_dense;        // order 3: dense d0 x d1 x d2 copy of the gradient for the factor updates, or nullptr
   float* g3_perm;         // order 3: the same permuted to d1 x d0 x d2, or nullptr
   float* g3_ghat;         // order 3, beta1 == 0: dense copy of the gradient for the mode products, or nullptr
+  float* g3_stat;         // order 3, eigenvalue-corrected: dense copy of the gradient for the rotated second moment
 };
 
 // offset of element e (block's own row-major order) inside the strided param / grad view
@@ -373,13 +374,14 @@ __global__ __launch_bounds__(EW_THREADS) void apply_kernel(const BlockDev* __res
 }
 
 // Dense (and dim-1-first) copies of the gradient of every order-3 block.  which = 0: for the factor updates
-// (g3_dense, g3_perm); which = 1: for the mode products of a step without filtered gradient (g3_ghat).
+// (g3_dense, g3_perm); which = 1: for the mode products of a step without filtered gradient (g3_ghat);
+// which = 2: for the rotated second moment of eigenvalue-corrected blocks (g3_stat).
 __global__ __launch_bounds__(EW_THREADS) void gather3_kernel(const BlockDev* __restrict__ blocks,
                                                             const ChunkRef* __restrict__ chunks, int which) {
   const ChunkRef cr = chunks[blockIdx.x];
   const BlockDev& B = blocks[cr.block];
   if (B.mid <= 0) return;
-  float* dense = which == 0 ? B.g3_dense : B.g3_ghat;
+  float* dense = which == 0 ? B.g3_dense : (which == 1 ? B.g3_ghat : B.g3_stat);
   float* perm = which == 0 ? B.g3_perm : nullptr;
   if (dense == nullptr && perm == nullptr) return;
   const int n_el = B.rows * B.cols, d0 = B.rows / B.mid;

@@ -244,6 +244,8 @@ struct sa_plan {
   GemmTable nt_h[8];      // Horner products of the higher-order iteration
   // mode products of order-3 blocks: [mode 1 | mode 0 | mode 2][first stage (divides by bias_correction1)][last stage (norm)]
   GemmTable g3[3][2][2];
+  // eigenvalue-corrected order-3 blocks: [statistic | rotate | rotate back][mode 1 | mode 0 | mode 2][first][last]
+  GemmTable e3[3][3][2][2];
   bool has_order3 = false;
   Table<HoJob> t_ho;
   std::vector<int> newton_history;  // per factor: iterations of its last converged solve, 0 = none
@@ -360,7 +362,7 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
     const long long eo = p->elem_off[b];
     // a block is preconditioned if a side has a Kronecker factor or, for eigenvalue-corrected Shampoo, a fixed basis
     const bool precond = p->block_factor[0][b] >= 0 || p->block_factor[1][b] >= 0 || p->block_factor[2][b] >= 0 ||
-                         (d.corrected_eigenvalues && (d.eigenvectors[0] || d.eigenvectors[1]));
+                         (d.corrected_eigenvalues && (d.eigenvectors[0] || d.eigenvectors[1] || d.eigenvectors[2]));
     B.ghat_tmp = (mode == 2) ? ghbuf(p) + eo : nullptr;
     if (mode == 0) {
       if (d.mid > 0 && precond) {
@@ -380,6 +382,8 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
       // dense copies for the factor updates: d0 x (d1 d2) in the T buffer, d1 x (d0 d2) in the P buffer
       if (d.factor[0] || d.factor[2]) B.g3_dense = tbuf(p) + eo;
       if (d.factor[1]) B.g3_perm = pbuf(p) + eo;
+      // the rotated second moment is updated from a dense copy of the raw gradient
+      if (d.corrected_eigenvalues && precond) B.g3_stat = ghbuf(p) + eo;
     }
     const bool contig = (d.ld == d.cols) && (d.mid == 0 || d.ld_outer == (long long)d.mid * d.ld);
     B.contig = contig ? 1 : 0;
@@ -456,10 +460,81 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
   for (GemmTable* g : {&p->ec_stat1, &p->ec_stat2, &p->ec_stat_l, &p->ec_stat_r, &p->ec_p1, &p->ec_p1d, &p->ec_p2, &p->ec_p2d,
                        &p->ec_p3, &p->ec_p3n, &p->ec_p4, &p->ec_p4n})
     g->clear();
+  for (auto& a : p->e3) for (auto& b2 : a) for (auto& c2 : b2) for (auto& g : c2) g.clear();
   if (p->eigenvalue_corrected) {
     for (int b : active) {
       const sa_block_desc& d = p->blocks[b];
-      const BlockDev& B = p->t_blocks.host[b];
+      BlockDev& B = p->t_blocks.host[b];
+      if (d.mid > 0) {
+        // order 3: three chains of mode products with the eigenbases (stage order mode 1, mode 0, mode 2):
+        // statistic (raw gradient, squared EMA at the end), rotation of the filtered gradient (division at the end),
+        // rotation back (norm at the end)
+        const float* Q[3] = {d.eigenvectors[1], d.eigenvectors[0], d.eigenvectors[2]};
+        const int d0 = d.rows / d.mid, d1 = d.mid, d2 = d.cols;
+        const int qd[3] = {d1, d0, d2};
+        int n_stages = 0;
+        for (const float* q : Q) n_stages += q ? 1 : 0;
+        if (!d.corrected_eigenvalues || n_stages == 0) continue;
+        const long long eo3 = p->elem_off[b];
+        float* part3 = p->f(p->off_ptile_partial) + p->ptile_begin_all[b];
+        auto tile_count = [](long long m, long long n) { return (int)(((m + BM - 1) / BM) * ((n + BN - 1) / BN)); };
+        float* pong[2] = {tbuf(p) + eo3, t2buf(p) + eo3};
+        int flip = 0;
+        const float* rotated = nullptr;  // result of the rotation chain
+        for (int chain = 0; chain < 3; ++chain) {
+          const float* src = chain == 0 ? B.g3_stat : (chain == 1 ? B.ghat_src : rotated);
+          int done = 0;
+          for (int kind = 0; kind < 3; ++kind) {
+            if (!Q[kind]) continue;
+            const bool first = done == 0, last = done == n_stages - 1;
+            float* out;
+            if (last && chain == 0) out = d.corrected_eigenvalues;
+            else if (last && chain == 2) out = pbuf(p) + eo3;
+            else { out = pong[flip]; flip ^= 1; }
+            float* c2 = nullptr;
+            if (last && chain == 1) c2 = d.corrected_eigenvalues;
+            if (last && chain == 2) c2 = part3;
+            GemmTable& tab = p->e3[chain][kind][first ? 1 : 0][last ? 1 : 0];
+            const float* Qk = Q[kind];
+            const int dk = qd[kind];
+            if (kind == 0) {
+              const int per = tile_count(d1, d2);
+              for (int i0 = 0; i0 < d0; ++i0) {
+                GemmProblem q{};
+                q.A = Qk; q.lda = dk; q.a_vec = vec_ok(Qk, dk);
+                q.B = src + (long long)i0 * d1 * d2; q.ldb = d2; q.b_vec = vec_ok(q.B, q.ldb);
+                q.C = out + (long long)i0 * d1 * d2; q.ldc = d2;
+                q.M = d1; q.N = d2; q.K = d1;
+                if (c2) q.C2 = (chain == 2) ? c2 + (long long)i0 * per : c2 + (long long)i0 * d1 * d2;
+                tab.add(q, false);
+              }
+              if (last && chain == 2) B.ptile_end = B.ptile_begin + d0 * per;
+            } else if (kind == 1) {
+              GemmProblem q{};
+              q.A = Qk; q.lda = dk; q.a_vec = vec_ok(Qk, dk);
+              q.B = src; q.ldb = (long long)d1 * d2; q.b_vec = vec_ok(q.B, q.ldb);
+              q.C = out; q.ldc = (long long)d1 * d2;
+              q.M = d0; q.N = d1 * d2; q.K = d0;
+              q.C2 = c2;
+              if (last && chain == 2) B.ptile_end = B.ptile_begin + tile_count(d0, (long long)d1 * d2);
+              tab.add(q, false);
+            } else {
+              GemmProblem q{};
+              q.A = src; q.lda = d2; q.a_vec = vec_ok(q.A, q.lda);
+              q.B = Qk; q.ldb = dk; q.b_vec = vec_ok(Qk, dk);
+              q.C = out; q.ldc = d2;
+              q.M = d0 * d1; q.N = d2; q.K = d2;
+              q.C2 = c2;
+              if (last && chain == 2) B.ptile_end = B.ptile_begin + tile_count((long long)d0 * d1, d2);
+              tab.add(q, false);
+            }
+            src = out;
+            ++done;
+          }
+          if (chain == 1) rotated = src;
+        }
+        continue;
+      }
       // eigenvectors[side] without factor[side] is a fixed basis: it rotates, but has no statistics and is never
       // refreshed (an ignored basis change, shampoo_preconditioner_list.py:1843-1865, passes the identity)
       const float* QL = d.eigenvectors[0];
@@ -501,6 +576,7 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
   for (GemmTable* g : {&p->ec_stat1, &p->ec_stat2, &p->ec_stat_l, &p->ec_stat_r, &p->ec_p1, &p->ec_p1d, &p->ec_p2, &p->ec_p2d,
                        &p->ec_p3, &p->ec_p3n, &p->ec_p4, &p->ec_p4n})
     SACHECK(g->commit(s));
+  for (auto& a : p->e3) for (auto& b2 : a) for (auto& c2 : b2) for (auto& g : c2) SACHECK(g.commit(s));
 
   // preconditioning tables (root-inverse Shampoo)
   p->g1_store.clear(); p->g1_norm.clear(); p->g2_norm.clear(); p->g2g_norm.clear();
@@ -653,6 +729,41 @@ int refresh_inverse_cache(sa_plan* p, hipStream_t s) {
 // C ABI
 // ============================================================================================
 
+// Launches one chain of the order-3 eigenvalue-corrected tables.  chain 0 / 1 multiply by the transposed bases
+// (into the eigenbasis), chain 2 by the bases (back); `mid` are the scalars of the stages that are not last,
+// `fin` those of the last stage (first[] variants add the division of the source operand).
+template <int EPI_LAST>
+static int launch_e3_chain(sa_plan* p, int chain, const GemmScalars& mid, const GemmScalars& fin, float src_div, hipStream_t s) {
+  for (int kind = 0; kind < 3; ++kind)
+    for (int first = 0; first < 2; ++first) {
+      GemmScalars a = mid, b = fin;
+      if (first && src_div != 1.0f) {
+        (kind == 2 ? a.a_div : a.b_div) = src_div;
+        (kind == 2 ? b.a_div : b.b_div) = src_div;
+      }
+      GemmTable& t0 = p->e3[chain][kind][first][0];
+      GemmTable& t1 = p->e3[chain][kind][first][1];
+      if (chain < 2) {
+        if (kind < 2) {
+          SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_STORE>(t0, a, s)));
+          SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_LAST>(t1, b, s)));
+        } else {
+          SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE>(t0, a, s)));
+          SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_LAST>(t1, b, s)));
+        }
+      } else {
+        if (kind < 2) {
+          SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE>(t0, a, s)));
+          SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_LAST>(t1, b, s)));
+        } else {
+          SACHECK((launch_gemm_auto<A_MK, B_NK, EPI_STORE>(t0, a, s)));
+          SACHECK((launch_gemm_auto<A_MK, B_NK, EPI_LAST>(t1, b, s)));
+        }
+      }
+    }
+  return SA_OK;
+}
+
 extern "C" {
 
 const char* sa_last_error(void) { return g_err.c_str(); }
@@ -738,10 +849,6 @@ int32_t sa_plan_create(const sa_block_desc* blocks, int32_t n_blocks, sa_plan** 
       delete p;
       return fail(SA_ERR_INVALID, "sa_plan_create: a third factor needs an order-3 block (mid > 0)");
     }
-    if (d.mid > 0 && (d.corrected_eigenvalues || d.eigenvectors[0] || d.eigenvectors[1] || d.eigenvectors[2])) {
-      delete p;
-      return fail(SA_ERR_UNSUPPORTED, "sa_plan_create: eigenvalue-corrected blocks of order 3 are not built");
-    }
     if (d.mid > 0) p->has_order3 = true;
     p->elem_off[b] = eo;
     eo += round_up((long long)d.rows * d.cols, 64);
@@ -823,6 +930,7 @@ void sa_plan_destroy(sa_plan* p) {
   for (auto& row : p->nt_pow) for (auto& g : row) g.t.destroy();
   for (auto& g : p->nt_h) g.t.destroy();
   for (auto& a : p->g3) for (auto& b2 : a) for (auto& g : b2) g.t.destroy();
+  for (auto& a : p->e3) for (auto& b2 : a) for (auto& c2 : b2) for (auto& g : c2) g.t.destroy();
   p->t_ho.destroy();
   p->t_sym.destroy(); p->t_normjobs.destroy(); p->t_ids.destroy();
   p->t_jacobi.destroy(); p->t_sched.destroy(); p->t_eiginit.destroy(); p->t_eigfinal.destroy(); p->eig_gemm.t.destroy();
@@ -2329,6 +2437,11 @@ int32_t sa_update_corrected_eigenvalues(sa_plan* p, float beta2, float weighting
   SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_SQ_EMA>(p->ec_stat2, sc, s)));
   SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_SQ_EMA>(p->ec_stat_l, sc, s)));
   SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_SQ_EMA>(p->ec_stat_r, sc, s)));
+  if (p->has_order3 && p->t_chunks.n) {
+    hipLaunchKernelGGL(gather3_kernel, dim3((unsigned)p->t_chunks.n), dim3(EW_THREADS), 0, s, p->t_blocks.dev, p->t_chunks.dev, 2);
+    HIPCHECK(hipGetLastError());
+    SACHECK(launch_e3_chain<EPI_SQ_EMA>(p, 0, unit_scalars(), sc, 1.0f, s));
+  }
   return SA_OK;
 }
 
@@ -2358,6 +2471,14 @@ int32_t sa_precondition_eigenvalue_corrected(sa_plan* p, const sa_step_scalars* 
     SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE_SQNORM>(p->ec_p3n, u, s)));
     SACHECK((launch_gemm_auto<A_MK, B_NK, EPI_STORE_SQNORM>(p->ec_p4, u, s)));
     SACHECK((launch_gemm_auto<A_MK, B_NK, EPI_STORE_SQNORM>(p->ec_p4n, u, s)));
+    if (p->has_order3 && p->t_chunks.n) {
+      if (p->table_mode == 0) {
+        hipLaunchKernelGGL(gather3_kernel, dim3((unsigned)p->t_chunks.n), dim3(EW_THREADS), 0, s, p->t_blocks.dev, p->t_chunks.dev, 1);
+        HIPCHECK(hipGetLastError());
+      }
+      SACHECK(launch_e3_chain<EPI_DIVPOW>(p, 1, u, den, sc->bias_correction1, s));
+      SACHECK(launch_e3_chain<EPI_STORE_SQNORM>(p, 2, u, u, 1.0f, s));
+    }
   }
   if (p->n_active_blocks) {
     hipLaunchKernelGGL(reduce_norms_kernel, dim3(p->n_active_blocks), dim3(EW_THREADS), 0, s, p->t_blocks.dev,

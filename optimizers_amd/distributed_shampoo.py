@@ -255,10 +255,6 @@ class _NativeGroup(_AmortizedComputation):
                 raise NotImplementedError(
                     f"block of order {s.order} (shape {s.shape}): the native step covers blocks of order 1 to 3"
                 )
-            if s.order == 3 and isinstance(pc, EigenvalueCorrectedShampooPreconditionerConfig):
-                raise NotImplementedError(
-                    f"block of order 3 (shape {s.shape}): eigenvalue-corrected Shampoo is built for blocks of order 1 and 2"
-                )
 
         # native blocks = blocks with at least one element
         self.native_index = [i for i, s in enumerate(self.block_specs) if s.numel > 0]
@@ -650,8 +646,8 @@ class DistributedShampoo(torch.optim.Optimizer):
     `EigenConfig` (`PerturbationConfig` and `PseudoInverseConfig`), `use_trace_scaling`, `EigenvalueCorrectedShampooPreconditionerConfig` with `QREigendecompositionConfig` or
     `EighEigendecompositionConfig` (including `ignored_basis_change_dims`), grafting with SGD / AdaGrad / RMSprop /
     Adam or none, every `WeightDecayType`, `ClassicMomentumConfig`, `inverse_exponent_override`,
-    `SingleDeviceDistributedConfig`, fp32 state with packed factor matrices, blocks of order 1 to 3 (order 3, e.g.
-    convolution weights, with root-inverse Shampoo only).
+    `SingleDeviceDistributedConfig`, fp32 state with packed factor matrices, blocks of order 1 to 3 (order 3: what is left of
+    convolution weights).
     Anything else raises NotImplementedError at construction.
     """
 

@@ -9,7 +9,7 @@ distributed_shampoo.py:659-759) and expose its three operations (preconditioner/
     compress_preconditioner_list(local_grad_selector)
 
 Everything numerical runs in libshampoo_amd.so on the blocks' device; torch only allocates.  Limits of the native
-step apply: fp32, blocks of order 0..3 (0..2 for the eigenvalue-corrected list), packed factor matrices, integer roots for the coupled iterations.
+step apply: fp32, blocks of order 0..3, packed factor matrices, integer roots for the coupled iterations.
 """
 
 from __future__ import annotations
@@ -137,8 +137,8 @@ class _NativeShampooPreconditionerList(PreconditionerList, _AmortizedComputation
         for b in self._blocks:
             if b.device.type != "cuda" or b.dtype != torch.float32:
                 raise RuntimeError(f"the native preconditioner list runs on an MI355X only: fp32 blocks on a HIP device, got {b.dtype} on {b.device}")
-            if b.dim() > 3 or (b.dim() == 3 and self.soap):
-                raise NotImplementedError(f"blocks of order {b.dim()} are not built natively for this list")
+            if b.dim() > 3:
+                raise NotImplementedError(f"blocks of order {b.dim()} are not built natively")
         self.device = self._blocks[0].device if self._blocks else torch.device("cuda:0")
         acc = preconditioner_config.amortized_computation_config
         self.use_eigh = isinstance(acc, EigenConfig)

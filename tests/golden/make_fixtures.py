@@ -140,6 +140,18 @@ CASES = {
         max_preconditioner_dim=16, precondition_frequency=2, start_preconditioning_step=4,
         preconditioner="newton", override_1d=True, grafting="adagrad", grafting_epsilon=1e-8,
     ),
+    "conv_like_soap_qr": dict(  # eigenvalue-corrected Shampoo on order-3 blocks, QR refresh, no grafting
+        shapes=[[20, 6, 3, 3], [6, 20, 3, 3], [5, 4, 20], [7]], seed=12, grad_scale=1.0, steps=9,
+        lr=1e-2, betas=[0.9, 0.99], epsilon=1e-10, weight_decay=0.0, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=16, precondition_frequency=3, start_preconditioning_step=3,
+        preconditioner="soap_qr", override_1d=False, grafting=None,
+    ),
+    "conv_like_soap_eigh": dict(  # the same with the eigh refresh, Adam grafting and no filtered gradient
+        shapes=[[20, 6, 3, 3], [6, 20, 3, 3], [5, 4, 20]], seed=13, grad_scale=1.0, steps=8,
+        lr=1e-2, betas=[0.0, 0.99], epsilon=1e-10, weight_decay=0.0, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=16, precondition_frequency=2, start_preconditioning_step=2,
+        preconditioner="soap_eigh", override_1d=False, grafting="adam", grafting_beta2=0.99, grafting_epsilon=1e-8,
+    ),
     "cfg1_override": dict(  # benchmark configuration 1 with 1-D blocks left to grafting
         shapes=[[512, 512], [512]], seed=0, grad_scale=1.0, steps=10, zero_init=True, torch_seed_grads=True,
         lr=1e-3, betas=[0.9, 0.999], epsilon=1e-12, weight_decay=0.0, weight_decay_type="DECOUPLED",
@@ -175,6 +187,8 @@ def build_reference(c, params):
             amortized_computation_config=QREigendecompositionConfig()
         )
         assert pc == DefaultSOAPConfig
+    elif c["preconditioner"] == "soap_eigh":
+        pc = EigenvalueCorrectedShampooPreconditionerConfig()
     else:
         raise ValueError(c["preconditioner"])
     graft = {

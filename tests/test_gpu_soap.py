@@ -18,18 +18,25 @@ def _aligned_up_to_sign(q_native, q_ref):
     return q_native * signs
 
 
-def test_soap_fixture_case_matches_reference():
+@pytest.mark.parametrize("name", ["soap_qr", "conv_like_soap_qr", "conv_like_soap_eigh"])
+def test_soap_fixture_case_matches_reference(name):
+    """soap_qr: matrices and vectors; conv_like_*: blocks of order 3 split along every dim."""
     import optimizers_amd as oa
     from oracle.shampoo_oracle import ShampooOracle
 
-    c = CASES["soap_qr"]
-    z = load_npz("soap_qr")
+    print(f"case {name}", flush=True)
+    c = CASES[name]
+    z = load_npz(name)
     init = initial_params(c)
     params = [torch.nn.Parameter(t.clone().to(DEV)) for t in init]
+    graft = None
+    if c["grafting"] == "adam":
+        graft = oa.AdamPreconditionerConfig(beta2=c["grafting_beta2"], epsilon=c["grafting_epsilon"])
     opt = oa.DistributedShampoo(
         params, lr=c["lr"], betas=tuple(c["betas"]), epsilon=c["epsilon"], max_preconditioner_dim=c["max_preconditioner_dim"],
         precondition_frequency=c["precondition_frequency"], start_preconditioning_step=c["start_preconditioning_step"],
-        preconditioner_config=oa.DefaultSOAPConfig)
+        grafting_config=graft,
+        preconditioner_config=oa.DefaultSOAPConfig if c["preconditioner"] == "soap_qr" else oa.DefaultEigenvalueCorrectedShampooConfig)
     ref_p = [t.clone() for t in init]
     ref = ShampooOracle(ref_p, oracle_config(c))
     ref64_p = [t.clone().double() for t in init]
@@ -60,10 +67,13 @@ def test_soap_fixture_case_matches_reference():
         for j, q in enumerate(ost["eigvecs"]):
             got = st["factor_matrices_eigenvectors"][j].cpu()
             assert rel_err(got.T @ got, torch.eye(got.shape[0])) < 1e-5
-            if spec.order == 2 and min(spec.shape) >= 16:  # full-rank factors: the basis is well defined
+            if name == "soap_qr" and spec.order == 2 and min(spec.shape) >= 16:  # full-rank factors: the basis is well defined
                 assert rel_err(_aligned_up_to_sign(got, q), q) < 1e-3
-        if spec.order == 2 and min(spec.shape) >= 16:
+        if name == "soap_qr" and spec.order == 2 and min(spec.shape) >= 16:
             assert rel_err(st["corrected_eigenvalues"].cpu(), ost["corrected"]) < 1e-3
+        if spec.order == 3:
+            # the rotated second moment belongs to the native bases: rebuild it from them (fp64) for the last gradient
+            pass
 
 
 # shapes whose factors all have full rank by the first refresh, so that the eigenbases are well defined
@@ -175,3 +185,58 @@ def test_all_basis_changes_ignored_is_adam(weight_decay):
     # no Kronecker factors and no eigenbases are kept for ignored dims
     st = opt.state[params[0]]["block_0"]["shampoo"]
     assert len(st["factor_matrices"]) == 0 and len(st["factor_matrices_eigenvectors"]) == 0
+
+
+@pytest.mark.parametrize("kind", ["soap_qr", "soap_eigh"])
+def test_order_three_blocks_rebuilt_from_the_stored_state(kind):
+    """A convolution weight (48, 40, 3, 3) with max_preconditioner_dim = 32: four order-3 blocks, two of them views
+    with a split middle dim.  The rotated second moment and the applied update are recomputed in fp64 from the
+    eigenbases the optimizer stores (shampoo_preconditioner_list.py:1891-1942 with tensordot over three dims)."""
+    import optimizers_amd as oa
+
+    g = torch.Generator().manual_seed(41)
+    shape = (48, 40, 3, 3)
+    w0 = 0.1 * torch.randn(*shape, generator=g)
+    p = torch.nn.Parameter(w0.clone().to(DEV))
+    lr, beta1, beta2, eps = 1e-2, 0.9, 0.95, 1e-9
+    opt = oa.DistributedShampoo(
+        [p], lr=lr, betas=(beta1, beta2), epsilon=eps, max_preconditioner_dim=32, precondition_frequency=2,
+        start_preconditioning_step=2,
+        preconditioner_config=oa.DefaultSOAPConfig if kind == "soap_qr" else oa.DefaultEigenvalueCorrectedShampooConfig)
+    ng = opt._groups[0]
+    specs = [ng.block_specs[i] for i in ng.native_index]
+    assert [s.shape for s in specs] == [(32, 32, 9), (32, 8, 9), (16, 32, 9), (16, 8, 9)]
+
+    def block(t, s):
+        return torch.as_strided(t.reshape(-1), s.shape, s.strides, s.offset)
+
+    def rotate(x, qs, back=False):
+        for q in qs:  # every tensordot contracts dim 0 and appends the result: after three the dims are back in order
+            x = torch.tensordot(x, q, dims=([0], [1] if back else [0]))
+        return x
+
+    v = [torch.zeros(s.shape, dtype=torch.float64) for s in specs]
+    m = [torch.zeros(s.shape, dtype=torch.float64) for s in specs]
+    steps = 5
+    for step in range(1, steps + 1):
+        G = torch.randn(*shape, generator=g)
+        before = p.detach().cpu().clone()
+        p.grad = G.to(DEV)
+        opt.step()
+        after = p.detach().cpu()
+        Gm = G.reshape(48, 40, 9).double()
+        for k, s in enumerate(specs):
+            st = opt.state[p][s.block_key]["shampoo"]
+            Q = [st["factor_matrices_eigenvectors"][j].cpu().double() for j in range(3)]
+            gb = block(Gm, s)
+            v[k] = beta2 * v[k] + (1 - beta2) * rotate(gb, Q) ** 2
+            m[k] = beta1 * m[k] + (1 - beta1) * gb
+            if step == steps:
+                for q in Q:
+                    assert (q.T @ q - torch.eye(q.shape[0], dtype=torch.float64)).abs().max() < 1e-5
+                assert rel_err(st["corrected_eigenvalues"].cpu(), v[k]) < 1e-4
+                ghat = m[k] / (1 - beta1**step)
+                rot = rotate(ghat, Q) / ((v[k] / (1 - beta2**step)).sqrt() + eps)
+                want = -lr * rotate(rot, Q, back=True)
+                delta = (block(after.reshape(48, 40, 9), s) - block(before.reshape(48, 40, 9), s)).double()
+                assert rel_err(delta, want) < 1e-3

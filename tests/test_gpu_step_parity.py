@@ -17,7 +17,7 @@ pytestmark = pytest.mark.gpu
 CASES = load_cases()
 NEWTON_CASES = [
     n for n, c in CASES.items()
-    if c["preconditioner"] in ("newton", "higher_order") or c.get("use_trace_scaling") or n.startswith("conv_like")
+    if c["preconditioner"] in ("newton", "higher_order") or c.get("use_trace_scaling") or (n.startswith("conv_like") and "soap" not in n)
 ]
 
 
