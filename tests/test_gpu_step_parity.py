@@ -160,3 +160,32 @@ def test_block_partition_is_bit_exact_on_device_views():
         for spec, w in zip(got, want):
             assert spec.shape == tuple(w.shape)
             assert spec.offset == w.storage_offset() and spec.strides == tuple(w.stride())
+
+
+@pytest.mark.parametrize("kind", ["newton", "eigh", "higher_order"])
+def test_twenty_steps_at_moderate_size(kind):
+    """Twenty steps (the horizon of the parity criterion) of a small transformer-like parameter set with ragged
+    blocks, every solver, against the oracle: parameters within 1e-3 (+ the reference algorithm's own fp32 noise
+    floor, see run_both) at every step, factors within 1e-5 and inverse roots within 1e-3 at the end."""
+    c = dict(
+        shapes=[[768, 256], [256, 768], [256, 256], [364, 256], [256], [256]], seed=77, grad_scale=0.02, steps=20,
+        lr=1e-3, betas=[0.9, 0.999], epsilon=1e-12, weight_decay=1e-2, weight_decay_type="DECOUPLED",
+        # the 108-row tail block of the 364 x 256 parameter feeds an order-256 factor: full rank from step 3 on
+        max_preconditioner_dim=256, precondition_frequency=1, start_preconditioning_step=4,
+        preconditioner=kind, override_1d=True, grafting="adam", grafting_beta2=0.999, grafting_epsilon=1e-8,
+        ho_order=3, ho_rel_epsilon=1e-7, ho_abs_epsilon=1e-12,
+    )
+    print(f"solver {kind}", flush=True)
+    opt, params, ref, ref_params, worst = run_both(c)
+    assert worst < 0.0, worst
+    for p, r in zip(params, ref_params):
+        assert rel_err(p.detach().cpu(), r) < 1e-3
+    ng = opt._groups[0]
+    for k, bi in enumerate(ng.native_index):
+        spec = ng.block_specs[bi]
+        st = opt.state[params[spec.param_index]][spec.block_key]
+        ost = ref.state[bi]
+        for j, f in enumerate(ost["factors"]):
+            assert rel_err(st["shampoo"]["factor_matrices"][j].cpu(), f) < 1e-5
+        for j, f in enumerate(ost["inv"]):
+            assert rel_err(st["shampoo"]["inv_factor_matrices"][j].cpu(), f) < 1e-3, (k, j)
