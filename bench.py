@@ -204,10 +204,17 @@ def cpu_baseline(workload: dict, name: str, budget_s: float = 25.0) -> dict:
     what = (f"{len(refresh)} full steps at {refresh_ms:.1f} ms/step" if sample_freq == 1 else
             f"{len(plain)} plain steps at {plain_ms:.1f} ms and {len(refresh)} steps with the amortized computation at "
             f"{refresh_ms:.1f} ms, combined for one amortized computation every {freq} steps")
+    model = "unknown CPU"
+    try:
+        with open("/proc/cpuinfo") as f:
+            model = next((line.split(":", 1)[1].strip() for line in f if line.startswith("model name")), model)
+    except OSError:
+        pass
     return {
         "value": ms * total / acc,
         "unit": "ms/step",
         "cores": torch.get_num_threads(),
+        "host": f"{model}, os.cpu_count() = {os.cpu_count()}, torch threads = {torch.get_num_threads()}",
         "kind": "port",
         "sample": f"oracle (torch CPU fp32) on parameters {sample} of {name}, {what}, scaled x{total / acc:.2f} by "
                   "d^3-weighted factor work",
