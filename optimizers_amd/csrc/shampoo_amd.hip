@@ -1071,8 +1071,10 @@ int32_t sa_precondition(sa_plan* p, const sa_step_scalars* sc, void* stream) {
     Span span("precondition_gemm", s, flops, launches, true);
     GemmScalars a = unit_scalars();
     a.b_div = sc->bias_correction1;
-    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE>(p->g1_store, a, s)));
-    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE_SQNORM>(p->g1_norm, a, s)));
+    // the left factor is the mirrored inverse root: exactly symmetric, so it is read through its transpose, whose
+    // slabs load and store as 16-byte rows (same values, same results)
+    SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_STORE>(p->g1_store, a, s)));
+    SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_STORE_SQNORM>(p->g1_norm, a, s)));
     SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE_SQNORM>(p->g2_norm, unit_scalars(), s)));
     GemmScalars c = unit_scalars();
     c.a_div = sc->bias_correction1;
@@ -1298,13 +1300,15 @@ static int newton_batch(sa_plan* p, const std::vector<int>& ids, const std::vect
       Span span("newton_gemm", s, flops, nl, false);
       if (g_profiling) g_phases["newton_gemm"].executed += executed;
       // the two variants touch disjoint factors, so their launches of one stage are independent
-      SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, true>(p->nt_a[1][parity], unit, s)));
+      // symmetric variant: every operand is an exactly mirrored matrix, so A is read through its transpose (slabs
+      // load and store as 16-byte rows instead of four scalar LDS stores per thread; same values, same results)
+      SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, false, true>(p->nt_a[1][parity], unit, s)));
       SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, false>(p->nt_a[0][parity], unit, s)));
       for (int k = 0; k < 4; ++k) {
-        SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, true>(p->nt_pow[1][parity * 4 + k], unit, s)));
+        SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, false, true>(p->nt_pow[1][parity * 4 + k], unit, s)));
         SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, false>(p->nt_pow[0][parity * 4 + k], unit, s)));
       }
-      SACHECK((launch_gemm<A_MK, B_KN, EPI_NEWTON_M, false, true>(p->nt_m[1][parity], msc, s)));
+      SACHECK((launch_gemm<A_KM, B_KN, EPI_NEWTON_M, false, true>(p->nt_m[1][parity], msc, s)));
       SACHECK((launch_gemm<A_MK, B_KN, EPI_NEWTON_M, false, false>(p->nt_m[0][parity], msc, s)));
       *flops_acc += flops;
       *launches_acc += nl;
