@@ -1,0 +1,137 @@
+"""The reference's equivalence suites on the MI355X (gpu_tests/shampoo_grafting_test.py:68-266,
+gpu_tests/weight_decay_test.py): with start_preconditioning_step = inf, Distributed Shampoo with a grafting
+method is that method, so five steps on the reference's toy problem (tests/shampoo_test_utils.py: seed 42,
+unit-norm inputs, a learnable 0-D scalar plus linear layers (10, 1, 1) filled with ones, MSE against zero) must give
+the weights and the loss of torch.optim.{Adagrad, Adam, AdamW, RMSprop, SGD} run on the same device."""
+
+import math
+from functools import partial
+from itertools import pairwise
+
+import pytest
+import torch
+from torch import nn
+from torch.optim import SGD, Adagrad, Adam, AdamW, RMSprop
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+
+class _Model(nn.Module):
+    def __init__(self, dims):
+        super().__init__()
+        self.scalar = nn.Parameter(torch.zeros(()))
+        self.linear_layers = nn.Sequential(*(nn.Linear(a, b, bias=False) for a, b in pairwise(dims)))
+
+    def forward(self, x):
+        return self.linear_layers(x) + self.scalar
+
+
+def _train(optim_factory, dims, steps=5):
+    torch.manual_seed(42)
+    data = torch.randn(dims[0], dtype=torch.float)
+    data /= torch.linalg.norm(data)
+    model = _Model(dims).to(DEV)
+    for m in model.linear_layers:
+        nn.init.constant_(m.weight, 1.0)
+    loss = nn.MSELoss()
+    target = torch.tensor([[0.0] * dims[-1]], device=DEV)
+    opt = optim_factory(model.parameters())
+    torch.manual_seed(42)
+    train = torch.randn(steps, dims[0], dtype=torch.float)
+    train /= torch.linalg.norm(train, dim=-1, keepdim=True)
+    train = train.to(DEV)
+    for s in range(steps):
+        opt.zero_grad()
+        loss(model(train[s]), target).backward()
+        opt.step()
+    final = loss(model(data.to(DEV).unsqueeze(0)), target)
+    return [p.detach().clone() for p in model.parameters()], final.detach()
+
+
+def _compare(control, experimental, dims=(10, 1, 1)):
+    want_p, want_l = _train(control, dims)
+    got_p, got_l = _train(experimental, dims)
+    torch.testing.assert_close(got_l, want_l)
+    torch.testing.assert_close(got_p, want_p)
+
+
+def _configs():
+    import optimizers_amd as oa
+
+    return (oa.DefaultShampooConfig, oa.DefaultEigenvalueCorrectedShampooConfig, oa.DefaultSOAPConfig)
+
+
+def _shampoo(params, **kw):
+    import optimizers_amd as oa
+
+    kw["weight_decay_type"] = getattr(oa.WeightDecayType, kw["weight_decay_type"])
+    return oa.DistributedShampoo(params, max_preconditioner_dim=10, precondition_frequency=1,
+                                 start_preconditioning_step=math.inf, **kw)
+
+
+@pytest.mark.parametrize("which", range(3))
+@pytest.mark.parametrize("weight_decay", (0.0, 0.3))
+def test_adagrad_grafting(weight_decay, which):
+    import optimizers_amd as oa
+
+    _compare(partial(Adagrad, lr=0.01, weight_decay=weight_decay, eps=1e-10),
+             partial(_shampoo, lr=0.01, weight_decay=weight_decay, betas=(0.0, 1.0), epsilon=1e-10, weight_decay_type="L2",
+                     grafting_config=oa.AdaGradPreconditionerConfig(epsilon=1e-10), preconditioner_config=_configs()[which]))
+
+
+@pytest.mark.parametrize("which", range(3))
+@pytest.mark.parametrize("weight_decay", (0.0, 0.3))
+def test_adam_grafting(weight_decay, which):
+    import optimizers_amd as oa
+
+    _compare(partial(Adam, lr=0.001, betas=(0.9, 0.999), weight_decay=weight_decay, eps=1e-8),
+             partial(_shampoo, lr=0.001, betas=(0.9, 0.999), weight_decay=weight_decay, epsilon=1e-8, weight_decay_type="L2",
+                     grafting_config=oa.AdamPreconditionerConfig(beta2=0.999, epsilon=1e-8),
+                     preconditioner_config=_configs()[which]))
+
+
+@pytest.mark.parametrize("which", range(3))
+@pytest.mark.parametrize("weight_decay", (0.0, 0.3))
+def test_adamw_grafting(weight_decay, which):
+    import optimizers_amd as oa
+
+    _compare(partial(AdamW, lr=0.001, betas=(0.9, 0.999), weight_decay=weight_decay, eps=1e-8),
+             partial(_shampoo, lr=0.001, betas=(0.9, 0.999), weight_decay=weight_decay, epsilon=1e-8,
+                     weight_decay_type="DECOUPLED", grafting_config=oa.AdamPreconditionerConfig(beta2=0.999, epsilon=1e-8),
+                     preconditioner_config=_configs()[which]))
+
+
+@pytest.mark.parametrize("which", range(3))
+@pytest.mark.parametrize("weight_decay", (0.0, 0.3))
+def test_rmsprop_grafting(weight_decay, which):
+    import optimizers_amd as oa
+
+    _compare(partial(RMSprop, lr=0.01, weight_decay=weight_decay, alpha=0.99, eps=1e-8),
+             partial(_shampoo, lr=0.01, weight_decay=weight_decay, betas=(0.0, 0.99), epsilon=1e-8, use_bias_correction=False,
+                     weight_decay_type="L2", grafting_config=oa.RMSpropPreconditionerConfig(beta2=0.99, epsilon=1e-8),
+                     preconditioner_config=_configs()[which]))
+
+
+@pytest.mark.parametrize("which", range(3))
+@pytest.mark.parametrize("weight_decay", (0.0, 0.3))
+def test_sgd_grafting(weight_decay, which):
+    import optimizers_amd as oa
+
+    _compare(partial(SGD, lr=0.1, weight_decay=weight_decay),
+             partial(_shampoo, lr=0.1, weight_decay=weight_decay, betas=(0.0, 1.0), epsilon=1e-10, weight_decay_type="L2",
+                     grafting_config=oa.SGDPreconditionerConfig(), preconditioner_config=_configs()[which]),
+             dims=(10, 10))
+
+
+@pytest.mark.parametrize("nesterov", (False, True))
+def test_sgd_momentum_through_classic_momentum(nesterov):
+    """gpu_tests/iterate_averaging_test.py: ClassicMomentumConfig on top of SGD grafting is torch's SGD momentum."""
+    import optimizers_amd as oa
+
+    _compare(partial(SGD, lr=0.1, momentum=0.5, nesterov=nesterov),
+             partial(_shampoo, lr=0.1, weight_decay=0.0, betas=(0.0, 1.0), epsilon=1e-10, weight_decay_type="L2",
+                     grafting_config=oa.SGDPreconditionerConfig(),
+                     iterate_averaging_config=oa.ClassicMomentumConfig(momentum=0.5, use_nesterov=nesterov),
+                     preconditioner_config=oa.DefaultShampooConfig),
+             dims=(10, 10))
