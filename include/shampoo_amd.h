@@ -237,6 +237,22 @@ int32_t sa_gemm_f32(const float* A, const float* B, float* C, int32_t M, int32_t
                     int64_t lda, int64_t ldb, int64_t ldc, int32_t a_layout, int32_t b_layout,
                     int32_t batch, int64_t stride_a, int64_t stride_b, int64_t stride_c, void* stream);
 
+/* A strided fp32 view of device memory of at most SA_MAX_ORDER dims: what a torch view of a parameter block
+ * is (sizes and element strides, outermost dim first; order 0 = one element). */
+typedef struct sa_view {
+  void* data;
+  int32_t order;
+  int64_t size[SA_MAX_ORDER];
+  int64_t stride[SA_MAX_ORDER];
+} sa_view;
+
+/* dst[i] += src[i] for n pairs of views of equal sizes: `Distributor.update_params`
+ * (distributor/shampoo_distributor.py:335-365, one `torch._foreach_add_` over the masked blocked parameters and
+ * their search directions).  The tables are host arrays read during the call; no device memory is allocated (the
+ * jobs travel as kernel arguments, 24 pairs per launch).  All pairs are validated before the first launch.
+ * Destination views must not alias each other. */
+int32_t sa_add_to_views(const sa_view* dst, const sa_view* src, int32_t n, void* stream);
+
 /* dst[i] = src[i] for n floats with a plain float4 copy kernel (n % 4 == 0, 16-byte aligned): the
  * known-traffic kernel that hardware HBM counters are calibrated against. */
 int32_t sa_copy_f32(const float* src, float* dst, int64_t n, void* stream);

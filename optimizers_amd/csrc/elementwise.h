@@ -807,4 +807,45 @@ __global__ void copy_strided_kernel(const float* __restrict__ src, long long lds
     dst[e] = src[(e / cols) * lds_ + (e % cols)];
 }
 
+// dst += src over up to VIEW_ADD_BATCH pairs of strided views of at most three dims (the parameter update of the
+// default distributor: every block of a parameter is a view into it, the directions are usually dense).  The jobs
+// travel as a kernel argument, so a call needs no device table.  Work is cut into runs of 4 elements of the
+// innermost dim: blockIdx.y is the job, the x grid strides over its runs.
+constexpr int VIEW_ADD_BATCH = 24;
+struct ViewAddJob {
+  float* dst;
+  const float* src;
+  unsigned int n0, n1, n2;      // sizes, outermost first (unused leading dims are 1)
+  unsigned int vec;             // both innermost strides are 1 and every run start is 16-byte aligned
+  long long d0, d1, d2;         // element strides of dst
+  long long s0, s1, s2;         // element strides of src
+};
+struct ViewAddBatch {
+  ViewAddJob job[VIEW_ADD_BATCH];
+};
+
+__global__ __launch_bounds__(256) void view_add_kernel(ViewAddBatch batch) {
+  const ViewAddJob& J = batch.job[blockIdx.y];
+  const unsigned int runs_per_row = (J.n2 + 3u) >> 2;
+  const unsigned long long rows = (unsigned long long)J.n0 * J.n1;
+  const unsigned long long runs = rows * runs_per_row;
+  for (unsigned long long r = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x; r < runs;
+       r += (unsigned long long)gridDim.x * blockDim.x) {
+    const unsigned long long row = r / runs_per_row;
+    const unsigned int c = (unsigned int)(r - row * runs_per_row) << 2;
+    const unsigned int i0 = (unsigned int)(row / J.n1), i1 = (unsigned int)(row - (unsigned long long)i0 * J.n1);
+    float* d = J.dst + i0 * J.d0 + i1 * J.d1 + c * J.d2;
+    const float* s = J.src + i0 * J.s0 + i1 * J.s1 + c * J.s2;
+    if (J.vec) {
+      float4 a = *reinterpret_cast<float4*>(d);
+      const float4 b = *reinterpret_cast<const float4*>(s);
+      a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+      *reinterpret_cast<float4*>(d) = a;
+    } else {
+      const unsigned int m = min(4u, J.n2 - c);
+      for (unsigned int k = 0; k < m; ++k) d[k * J.d2] += s[k * J.s2];
+    }
+  }
+}
+
 }  // namespace sa

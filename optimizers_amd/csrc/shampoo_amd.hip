@@ -2775,4 +2775,73 @@ int32_t sa_copy_f32(const float* src, float* dst, int64_t n, void* stream) {
   return SA_OK;
 }
 
+int32_t sa_add_to_views(const sa_view* dst, const sa_view* src, int32_t n, void* stream) {
+  if (n < 0 || (n > 0 && (!dst || !src))) return fail(SA_ERR_INVALID, "sa_add_to_views: null view table");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // validate everything before the first launch: a bad pair must leave every destination untouched
+  for (int i = 0; i < n; ++i) {
+    const sa_view &D = dst[i], &S = src[i];
+    if (D.order < 0 || D.order > SA_MAX_ORDER || S.order != D.order)
+      return fail(SA_ERR_INVALID, "sa_add_to_views: pair " + std::to_string(i) + ": orders must agree and be at most " +
+                                      std::to_string(SA_MAX_ORDER));
+    for (int k = 0; k < D.order; ++k) {
+      if (D.size[k] != S.size[k] || D.size[k] < 0 || D.size[k] > 0x7fffffffLL)
+        return fail(SA_ERR_INVALID, "sa_add_to_views: pair " + std::to_string(i) + ": sizes differ in dim " + std::to_string(k));
+      if (D.size[k] > 1 && D.stride[k] <= 0)
+        return fail(SA_ERR_INVALID, "sa_add_to_views: pair " + std::to_string(i) + ": destination views must not overlap themselves");
+    }
+    long long numel = 1;
+    for (int k = 0; k < D.order; ++k) numel *= D.size[k];
+    if (numel > 0 && (!D.data || !S.data)) return fail(SA_ERR_INVALID, "sa_add_to_views: pair " + std::to_string(i) + ": null data pointer");
+  }
+  ViewAddBatch batch;
+  int filled = 0;
+  unsigned long long most_runs = 0;
+  double bytes = 0.0;
+  bool first_launch = true;
+  auto flush = [&]() -> int32_t {
+    if (filled == 0) return SA_OK;
+    const unsigned int gx = (unsigned int)std::min<unsigned long long>((most_runs + 255) / 256, 1024);
+    Span span("view_add", s, bytes, 1, first_launch);
+    first_launch = false;
+    hipLaunchKernelGGL(view_add_kernel, dim3(gx, filled), dim3(256), 0, s, batch);
+    HIPCHECK(hipGetLastError());
+    filled = 0;
+    most_runs = 0;
+    bytes = 0.0;
+    return SA_OK;
+  };
+  for (int i = 0; i < n; ++i) {
+    const sa_view &D = dst[i], &S = src[i];
+    ViewAddJob J{};
+    unsigned int sz[3] = {1, 1, 1};
+    long long ds[3] = {0, 0, 0}, ss[3] = {0, 0, 0};
+    for (int k = 0; k < D.order; ++k) {  // right-align: a 2-D view is (1, rows, cols)
+      sz[3 - D.order + k] = (unsigned int)D.size[k];
+      ds[3 - D.order + k] = D.stride[k];
+      ss[3 - D.order + k] = S.stride[k];
+    }
+    const unsigned long long numel = (unsigned long long)sz[0] * sz[1] * sz[2];
+    if (numel == 0) continue;
+    if (sz[2] == 1) { ds[2] = 1; ss[2] = 1; }  // strides of extent-1 dims are arbitrary
+    J.dst = static_cast<float*>(D.data);
+    J.src = static_cast<const float*>(S.data);
+    J.n0 = sz[0]; J.n1 = sz[1]; J.n2 = sz[2];
+    J.d0 = ds[0]; J.d1 = ds[1]; J.d2 = ds[2];
+    J.s0 = ss[0]; J.s1 = ss[1]; J.s2 = ss[2];
+    auto rows_aligned = [&](const void* p, const long long* st) {
+      return (reinterpret_cast<uintptr_t>(p) & 15) == 0 && (sz[0] == 1 || (st[0] & 3) == 0) && (sz[1] == 1 || (st[1] & 3) == 0);
+    };
+    J.vec = (ds[2] == 1 && ss[2] == 1 && (sz[2] & 3) == 0 && rows_aligned(D.data, ds) && rows_aligned(S.data, ss)) ? 1u : 0u;
+    batch.job[filled++] = J;
+    most_runs = std::max<unsigned long long>(most_runs, (unsigned long long)sz[0] * sz[1] * ((sz[2] + 3) / 4));
+    bytes += 12.0 * (double)numel;
+    if (filled == VIEW_ADD_BATCH) {
+      const int32_t st = flush();
+      if (st != SA_OK) return st;
+    }
+  }
+  return flush();
+}
+
 }  // extern "C"

@@ -34,7 +34,7 @@ EXPORTS = (
     "sa_precondition_eigenvalue_corrected", "sa_update_grafting_and_filtered_grad", "sa_precondition",
     "sa_apply_update", "sa_grafting_only_step", "sa_plan_read_norms", "sa_plan_read_preconditioned",
     "sa_gemm_f32", "sa_copy_f32", "sa_set_profiling", "sa_phase_ms", "sa_phase_flops", "sa_phase_launches", "sa_phase_executed_flops", "sa_set_symmetric_newton", "sa_set_eigh_solver",
-    "sa_plan_set_trace_scaling", "sa_compute_root_inverses_higher_order", "sa_plan_read_eigenvalues",
+    "sa_plan_set_trace_scaling", "sa_compute_root_inverses_higher_order", "sa_plan_read_eigenvalues", "sa_add_to_views",
 )
 
 
@@ -76,6 +76,25 @@ class StepScalars(ctypes.Structure):
         ("dampening", c_float),
         ("use_nesterov", c_int32),
     ]
+
+
+class View(ctypes.Structure):
+    """sa_view: a strided fp32 view of device memory (sizes and element strides, outermost dim first)."""
+
+    _fields_ = [
+        ("data", c_void_p),
+        ("order", c_int32),
+        ("size", c_int64 * SA_MAX_ORDER),
+        ("stride", c_int64 * SA_MAX_ORDER),
+    ]
+
+
+def fill_view(view: View, t: torch.Tensor) -> None:
+    view.data = t.data_ptr()
+    view.order = t.dim()
+    for k in range(t.dim()):
+        view.size[k] = t.size(k)
+        view.stride[k] = t.stride(k)
 
 
 class NativeError(RuntimeError):
@@ -136,6 +155,7 @@ def load() -> ctypes.CDLL:
         c_int32, c_int64, c_int64, c_int64, c_void_p,
     ]
     lib.sa_copy_f32.argtypes = [c_void_p, c_void_p, c_int64, c_void_p]
+    lib.sa_add_to_views.argtypes = [POINTER(View), POINTER(View), c_int32, c_void_p]
     lib.sa_set_profiling.argtypes = [c_int32]
     lib.sa_phase_ms.argtypes = [c_char_p]
     lib.sa_phase_ms.restype = c_double
