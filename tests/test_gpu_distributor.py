@@ -58,7 +58,7 @@ def test_update_params(setup):
     torch.testing.assert_close(dist.local_masked_blocked_params, directions, rtol=0, atol=0)
     # the blocks are views: the parameter itself moved (columns 0-4 and 5-9 of the 5 x 10 weight)
     torch.testing.assert_close(model.linear_layers[0].weight.detach(), torch.cat(directions, dim=1), rtol=0, atol=0)
-    assert float(model.scalar) == 0.0 and float(model.linear_layers[0].bias.abs().sum()) == 0.0
+    assert float(model.scalar.detach()) == 0.0 and float(model.linear_layers[0].bias.detach().abs().sum()) == 0.0
 
 
 def test_local_grad_selector(setup):
@@ -132,7 +132,7 @@ def test_empty_parameter():
     torch.testing.assert_close(dist.local_masked_blocked_params, (torch.ones((1,), device=DEV),), rtol=0, atol=0)
     # all blocks, masked or not
     dist.update_params((torch.ones((1,), device=DEV), torch.zeros((0,), device=DEV)), use_masked_tensors=False)
-    assert float(model.scalar) == 2.0
+    assert float(model.scalar.detach()) == 2.0
 
 
 def test_update_params_rejects_a_wrong_count(setup):
