@@ -7,7 +7,8 @@ roots, grafting, preconditioning, parameter update) over one batch of synthetic 
 that already sit in HBM.  Prints ONE JSON line with the metric, a roofline object for the
 dominant kernel (the grouped fp32 MFMA GEMM of the Newton iteration, timed live with HIP
 events on the stream it is launched on) and a cpu_baseline object (the CPU oracle timed on
-this box's host cores on a bounded sample of the same workload).
+this box's host cores on a bounded sample of the same workload), next to a torch_gpu_baseline object (the same
+oracle's torch ops on this GPU: what the reference's own code path costs here).
 """
 
 from __future__ import annotations
@@ -136,6 +137,71 @@ def make_grads(workload: dict, params, step: int, device):
     return out
 
 
+def _time_oracle(workload: dict, shapes, device, budget_s: float):
+    """ms/step of the oracle (the reference's algorithm as plain torch ops) on `device` for parameters of the given
+    shapes, with the workload's schedule: grafting-only steps, then full steps.  Where the workload amortizes the
+    root inverse / eigenbasis refresh over k > 1 steps, plain steps and steps with the amortized computation are
+    timed separately (the sample alternates them) and combined for one amortized computation every k steps."""
+    import torch
+
+    from oracle.shampoo_oracle import OracleConfig, ShampooOracle
+
+    on_gpu = device.type == "cuda"
+    gen = torch.Generator(device=device).manual_seed(0)
+    params = [0.02 * torch.randn(*s, device=device, generator=gen) for s in shapes]
+    kind = workload.get("preconditioner", "newton")
+    freq = workload.get("precondition_frequency", 1)
+    sample_freq = 1 if freq == 1 else 2
+    # Newton: one more grafting-only step than the native run, so that the order-2048 factor of a 1024 x 2048 block has
+    # seen three gradients (rank 3072) before its first root inverse; with two its rank is exactly 2048 and whether
+    # the fp32 iteration overflows depends on the draw
+    start = workload.get("start_preconditioning_step", START_PRECONDITIONING_STEP) if on_gpu else START_PRECONDITIONING_STEP
+    start += 1 if kind == "newton" else 0
+    if sample_freq > 1:
+        start = 2
+    cfg = OracleConfig(
+        lr=workload["lr"], betas=workload["betas"], epsilon=workload["epsilon"],
+        max_preconditioner_dim=workload["max_preconditioner_dim"],
+        precondition_frequency=sample_freq, start_preconditioning_step=start, preconditioner=kind,
+        inverse_exponent_override={1: {0: 0.0}} if kind == "newton" else {}, grafting=workload.get("grafting", "adam"),
+        grafting_beta2=workload.get("graft_beta2", 0.999), grafting_epsilon=workload.get("graft_eps", 1e-8),
+    )
+    opt = ShampooOracle(params, cfg)
+    sample_workload = dict(workload, shapes=list(shapes))
+    # gradients are drawn outside the timed region; the spectrum workload cycles through two of them like the native run
+    pool = [make_grads(sample_workload, params, k, device) for k in range(2)] if "spectrum" in workload else None
+    refresh, plain = [], []
+    t_start = time.perf_counter()
+    for step in range(1, start + 6):
+        grads = [g.clone() for g in pool[step % 2]] if pool else make_grads(sample_workload, params, step, device)
+        if on_gpu:
+            torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        opt.step(grads)
+        if on_gpu:
+            torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        if step > start:  # steps after the first (cold) preconditioned one
+            (refresh if step % sample_freq == 0 else plain).append(dt)
+        if time.perf_counter() - t_start > budget_s and refresh and (plain or sample_freq == 1):
+            break
+    refresh_ms = 1e3 * sum(refresh) / len(refresh)
+    plain_ms = 1e3 * sum(plain) / len(plain) if plain else refresh_ms
+    ms = plain_ms + (refresh_ms - plain_ms) / freq if sample_freq > 1 else refresh_ms
+    what = (f"{len(refresh)} full steps at {refresh_ms:.1f} ms/step" if sample_freq == 1 else
+            f"{len(plain)} plain steps at {plain_ms:.1f} ms and {len(refresh)} steps with the amortized computation at "
+            f"{refresh_ms:.1f} ms, combined for one amortized computation every {freq} steps")
+    return ms, what
+
+
+def torch_gpu_baseline(workload: dict, name: str, device, budget_s: float = 40.0) -> dict:
+    """The reference's own code path on this GPU: the oracle's torch ops (rocBLAS GEMMs, rocSOLVER eigh / QR, a
+    Python loop over blocks and factors) on device tensors, whole workload, same schedule as the CPU baseline."""
+    ms, what = _time_oracle(workload, workload["shapes"], device, budget_s)
+    return {"value": ms, "unit": "ms/step", "kind": "port",
+            "sample": f"oracle (torch ops on {device}, fp32) on every parameter of {name}, {what}"}
+
+
 def cpu_baseline(workload: dict, name: str, budget_s: float = 25.0) -> dict:
     """Times the CPU oracle (port of the reference algorithm, plain torch on the host cores) on
     a bounded sample: the first parameters of the workload whose estimated CPU time fits the
@@ -144,7 +210,6 @@ def cpu_baseline(workload: dict, name: str, budget_s: float = 25.0) -> dict:
     import torch
 
     from optimizers_amd.blocking import partition_parameter
-    from oracle.shampoo_oracle import OracleConfig, ShampooOracle
 
     b = workload["max_preconditioner_dim"]
 
@@ -164,46 +229,7 @@ def cpu_baseline(workload: dict, name: str, budget_s: float = 25.0) -> dict:
             break
         sample.append(s)
         acc += cost(s)
-    torch.manual_seed(0)
-    params = [0.02 * torch.randn(*s) for s in sample]
-    kind = workload.get("preconditioner", "newton")
-    freq = workload.get("precondition_frequency", 1)
-    # the amortized computation every second step of the sample when the workload amortizes it over more steps:
-    # its extra cost is then spread over the workload's own frequency
-    sample_freq = 1 if freq == 1 else 2
-    grafting = workload.get("grafting", "adam")
-    # Newton: one more grafting-only step than the GPU run, so that the order-2048 factor of a 1024 x 2048 block has
-    # seen three gradients (rank 3072) before its first root inverse; with two its rank is exactly 2048 and whether
-    # the fp32 iteration overflows depends on the draw
-    start = START_PRECONDITIONING_STEP + (1 if kind == "newton" else 0)
-    cfg = OracleConfig(
-        lr=workload["lr"], betas=workload["betas"], epsilon=workload["epsilon"], max_preconditioner_dim=b,
-        precondition_frequency=sample_freq, start_preconditioning_step=start, preconditioner=kind,
-        inverse_exponent_override={1: {0: 0.0}} if kind == "newton" else {}, grafting=grafting,
-        grafting_beta2=workload.get("graft_beta2", 0.999), grafting_epsilon=workload.get("graft_eps", 1e-8),
-    )
-    opt = ShampooOracle(params, cfg)
-    cpu = torch.device("cpu")
-    sample_workload = dict(workload, shapes=sample)
-    # gradients are drawn outside the timed region; the spectrum workload cycles through two of them like the GPU run
-    pool = [make_grads(sample_workload, params, k, cpu) for k in range(2)] if "spectrum" in workload else None
-    refresh, plain = [], []
-    t_start = time.perf_counter()
-    for step in range(1, 8):
-        grads = [g.clone() for g in pool[step % 2]] if pool else make_grads(sample_workload, params, step, cpu)
-        t0 = time.perf_counter()
-        opt.step(grads)
-        dt = time.perf_counter() - t0
-        if step > start:  # steps after the first (cold) preconditioned one
-            (refresh if step % sample_freq == 0 else plain).append(dt)
-        if time.perf_counter() - t_start > budget_s and refresh and (plain or sample_freq == 1):
-            break
-    refresh_ms = 1e3 * sum(refresh) / len(refresh)
-    plain_ms = 1e3 * sum(plain) / len(plain) if plain else refresh_ms
-    ms = plain_ms + (refresh_ms - plain_ms) / freq if sample_freq > 1 else refresh_ms
-    what = (f"{len(refresh)} full steps at {refresh_ms:.1f} ms/step" if sample_freq == 1 else
-            f"{len(plain)} plain steps at {plain_ms:.1f} ms and {len(refresh)} steps with the amortized computation at "
-            f"{refresh_ms:.1f} ms, combined for one amortized computation every {freq} steps")
+    ms, what = _time_oracle(workload, sample, torch.device("cpu"), budget_s)
     model = "unknown CPU"
     try:
         with open("/proc/cpuinfo") as f:
@@ -380,6 +406,11 @@ def main() -> None:
         "phases": detail,
     }
     if not args.no_cpu_baseline:
+        # the native optimizer's state is released first: the oracle keeps dense factors and inverse roots of its own
+        del opt, params, grads
+        torch.cuda.empty_cache()
+        out["torch_gpu_baseline"] = torch_gpu_baseline(workload, args.workload, device)
+        torch.cuda.empty_cache()
         out["cpu_baseline"] = cpu_baseline(workload, args.workload)
     print(json.dumps(out))
 

@@ -151,8 +151,9 @@ __device__ __forceinline__ float wave_max_nan(float v) {
 }
 
 // TRI: the product is known to be symmetric (coupled Newton: every operand is a polynomial in the
-// same matrix).  Only tiles on or above the diagonal are computed; an off-diagonal tile is stored
-// twice, as computed and transposed, which halves the MFMA work of a square product.
+// same matrix).  Only tiles on or above the diagonal are computed; everything above the diagonal is stored
+// twice, as computed and transposed, which halves the MFMA work of a square product and leaves an exactly
+// mirrored matrix (so a later product may read it through its transpose).
 template <int AL, int BL, int EPI, bool EDGE, bool TRI = (EPI == EPI_SYRK_EMA)>
 __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(
     const GemmProblem* __restrict__ problems, int n_problems, int total_tiles, GemmScalars sc) {
@@ -298,9 +299,12 @@ __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(
       for (int e = 0; e < 16; ++e) {
         const int row = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
         const float v = acc[i][j][e];
+        // A diagonal tile of a symmetric product recomputes its lower half; that half is dropped and replaced by the
+        // mirror image of the upper one, so that every symmetric product leaves an exactly mirrored matrix.
+        const bool lower = TRI && (EPI == EPI_STORE || EPI == EPI_NEWTON_M) && tm == tn && row > col;
         if (EPI == EPI_STORE) {
-          if (!EDGE || (row < M && col < N)) C[(long long)row * ldc + col] = v;
-          if (TRI && EDGE && tm != tn && row < M && col < N) C[(long long)col * ldc + row] = v;
+          if (!lower && (!EDGE || (row < M && col < N))) C[(long long)row * ldc + col] = v;
+          if (TRI && EDGE && (tm != tn || row < col) && row < M && col < N) C[(long long)col * ldc + row] = v;
         } else if (EPI == EPI_STORE_SQNORM) {
           if (!EDGE || (row < M && col < N)) {
             C[(long long)row * ldc + col] = v;
@@ -340,33 +344,41 @@ __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(
           C[o] = r;
         } else if (EPI == EPI_NEWTON_M) {
           // operands are zero padded to the tile grid, so every (row, col) is in bounds
-          C[(long long)row * ldc + col] = v;
-          float mp = __fmul_rn(v, sc.mp_scale);
-          if (row == col && row < P.d) mp = __fadd_rn(mp, sc.mp_diag);
-          P.C2[(long long)row * ldc + col] = mp;
-          if (TRI && EDGE && tm != tn) {
-            C[(long long)col * ldc + row] = v;
-            P.C2[(long long)col * ldc + row] = mp;
-          }
-          if (row < P.d && col < P.d) {
-            const float dv = fabsf(v - (row == col ? 1.0f : 0.0f));
-            if (dv != dv) local_nan = true;
-            local = fmaxf(local, dv);
+          if (!lower) {
+            C[(long long)row * ldc + col] = v;
+            float mp = __fmul_rn(v, sc.mp_scale);
+            if (row == col && row < P.d) mp = __fadd_rn(mp, sc.mp_diag);
+            P.C2[(long long)row * ldc + col] = mp;
+            if (TRI && EDGE && (tm != tn || row < col)) {
+              C[(long long)col * ldc + row] = v;
+              P.C2[(long long)col * ldc + row] = mp;
+            }
+            if (row < P.d && col < P.d) {
+              const float dv = fabsf(v - (row == col ? 1.0f : 0.0f));
+              if (dv != dv) local_nan = true;
+              local = fmaxf(local, dv);
+            }
           }
         }
       }
     }
   }
   if (TRI && !EDGE && (EPI == EPI_STORE || EPI == EPI_NEWTON_M)) {
-    // Mirror image of an off-diagonal tile: each 32 x 32 accumulator block is transposed through the (now idle)
-    // operand buffers, one private region per wavefront, and leaves as 16-byte stores along the rows of C.
-    if (tm != tn) {
+    // Mirror image of everything above the diagonal: each 32 x 32 accumulator block is transposed through the (now
+    // idle) operand buffers, one private region per wavefront, and leaves as 16-byte stores along the rows of C.
+    // In a diagonal tile the blocks below the diagonal are skipped (their computed values are dropped) and the
+    // blocks on it mirror only their strictly upper part, element by element.
+    const bool diag = (tm == tn);
+    if (!diag || wm <= wn) {
       constexpr int TS = 36;  // 32 + 4: keeps float4 alignment
       float* stage = ((wave < 2) ? &As[0][0] : &Bs[0][0]) + (wave & 1) * (BK * LDS_STRIDE);
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
+          const int br = wm * 2 + i, bc = wn * 2 + j;  // position of the block inside the tile, in blocks of 32
+          if (diag && br > bc) continue;
+          const bool on_diagonal = diag && br == bc;
 #pragma unroll
           for (int q = 0; q < 4; ++q)  // stage[col][row]: the four accumulator values of a group are four consecutive rows
             *reinterpret_cast<float4*>(stage + l32 * TS + 8 * q + 4 * h) =
@@ -378,10 +390,20 @@ __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(
             const int c = (lane >> 3) + 8 * it, r4 = (lane & 7) * 4;
             const float4 v = *reinterpret_cast<const float4*>(stage + c * TS + r4);
             const long long o = (long long)(n0 + wn * 64 + j * 32 + c) * ldc + (m0 + wm * 64 + i * 32 + r4);
-            *reinterpret_cast<float4*>(C + o) = v;
-            if (EPI == EPI_NEWTON_M)  // off-diagonal tile: M_p has no diagonal term here
-              *reinterpret_cast<float4*>(P.C2 + o) = make_float4(__fmul_rn(v.x, sc.mp_scale), __fmul_rn(v.y, sc.mp_scale),
-                                                                 __fmul_rn(v.z, sc.mp_scale), __fmul_rn(v.w, sc.mp_scale));
+            if (!on_diagonal) {
+              *reinterpret_cast<float4*>(C + o) = v;
+              if (EPI == EPI_NEWTON_M)  // strictly below the diagonal: M_p has no diagonal term here
+                *reinterpret_cast<float4*>(P.C2 + o) = make_float4(__fmul_rn(v.x, sc.mp_scale), __fmul_rn(v.y, sc.mp_scale),
+                                                                   __fmul_rn(v.z, sc.mp_scale), __fmul_rn(v.w, sc.mp_scale));
+            } else {
+              const float vv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+              for (int k = 0; k < 4; ++k)
+                if (c > r4 + k) {  // target (row c, column r4 + k) of the block lies strictly below the diagonal
+                  C[o + k] = vv[k];
+                  if (EPI == EPI_NEWTON_M) P.C2[o + k] = __fmul_rn(vv[k], sc.mp_scale);
+                }
+            }
           }
           __builtin_amdgcn_wave_barrier();
           asm volatile("" ::: "memory");

@@ -182,3 +182,36 @@ def test_larger_matrices_against_fp64(d):
     Qd = Q.cpu().double()
     assert (Qd.T @ Qd - torch.eye(d, dtype=torch.float64)).abs().max() < 1e-5
     assert rel_err(Qd * L.cpu().double() @ Qd.T, A.double()) < 1e-5
+
+
+@pytest.mark.parametrize("d", (200, 768, 1024))
+def test_symmetric_products_converge_like_full_products(d, caplog):
+    """Product policy 1 (every Newton product computed on the upper-triangle tiles and mirrored, operands read
+    through their transpose) must converge in the iterations the reference's full products need (+-1 where the error
+    hovers at the tolerance) and give the same inverse root to well below the 1e-3 bar: every symmetric product has to
+    leave an exactly mirrored matrix, diagonal tiles included."""
+    import optimizers_amd as oa
+    from optimizers_amd import native
+    from optimizers_amd.matrix_functions import _plan_for, matrix_inverse_root
+
+    gen = torch.Generator().manual_seed(d)
+    G = torch.randn(d, 3 * d // 2, generator=gen, dtype=torch.float64)
+    A = (G @ G.T / G.shape[1]).float().to(DEV)
+    lib = native.load()
+    results, counts = [], []
+    try:
+        for policy in (0, 1):
+            lib.sa_set_symmetric_newton(policy)
+            with caplog.at_level(logging.WARNING):
+                caplog.clear()
+                X = matrix_inverse_root(A=A, root=Fraction(4), root_inv_config=oa.CoupledNewtonConfig(), epsilon=1e-12)
+            assert not any("did not converge" in r.message for r in caplog.records), f"policy {policy} did not converge"
+            results.append(X)
+            counts.append(int(_plan_for(A, False, 4).iterations[0]))
+    finally:
+        lib.sa_set_symmetric_newton(2)
+    assert abs(counts[0] - counts[1]) <= 1, counts
+    assert rel_err(results[1], results[0]) <= 1e-4
+    lam, Q = torch.linalg.eigh(A.double().cpu())
+    truth = (Q * lam.pow(-0.25)) @ Q.T
+    assert rel_err(results[1].double().cpu(), truth) <= 1e-3
