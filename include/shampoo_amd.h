@@ -191,6 +191,21 @@ int32_t sa_refresh_eigenbases_eigh(sa_plan* plan, float bias_correction2, float 
 int32_t sa_refresh_eigenbases_qr(sa_plan* plan, float bias_correction2, float epsilon, int32_t max_iterations,
                                  float tolerance, int32_t* iterations_out, int32_t* status_out, void* stream);
 
+/* Eigendecomposed Shampoo (EigendecomposedShampooPreconditionerConfig): a block descriptor gives `factor`,
+ * `eigenvectors` AND `inv_factor` for each preconditioned dim and no `corrected_eigenvalues`.  The amortized
+ * computation (shampoo_preconditioner_list.py:763-940: matrix_eigendecomposition of the bias-corrected factor, started
+ * from the stored eigenvectors for the QR algorithm) is sa_refresh_eigenbases_eigh / sa_refresh_eigenbases_qr followed
+ * by sa_plan_read_eigenvalues into the caller's eigenvalue state; this call then forms
+ * X = Q diag(w) Q^T, w from matrix_inverse_root_from_eigendecomposition (matrix_functions.py:179-279; `stability`,
+ * `rank_rtol`, `rank_atol` and `roots` as in sa_compute_root_inverses_eigh), and stores it in `inv_factor`, which
+ * sa_precondition uses.  The reference forms the same product in every step (:1793-1832); it only changes with
+ * (Q, lambda).  `eigenvalues[i]`: device pointer to the d eigenvalues of factor i (plan order).  Call it again after
+ * writing eigenvectors / eigenvalues from outside (checkpoint load).  status_out: SA_FACTOR_OK, _SKIPPED or
+ * _RESULT_NONFINITE. */
+int32_t sa_compute_root_inverses_from_eigendecomposition(sa_plan* plan, const float* const* eigenvalues, float epsilon,
+                                                         const float* roots, int32_t stability, float rank_rtol,
+                                                         float rank_atol, int32_t* status_out, void* stream);
+
 /* corrected_eigenvalues <- beta2 * corrected_eigenvalues + w * (Q_L^T G Q_R)^2 with the raw gradient
  * (shampoo_preconditioner_list.py:1891-1912). */
 int32_t sa_update_corrected_eigenvalues(sa_plan* plan, float beta2, float weighting_factor, void* stream);

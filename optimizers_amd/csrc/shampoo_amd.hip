@@ -272,7 +272,8 @@ struct sa_plan {
   Table<Copy2D> t_copy;
   Table<NormPair> t_normpair;
   Table<SortJob> t_sort;
-  bool eigenvalue_corrected = false;
+  bool eigenvalue_corrected = false;  // blocks carry a second moment in the eigenbasis (corrected_eigenvalues)
+  bool has_eigvec = false;            // some factor stores its eigenvectors (eigenvalue-corrected or eigendecomposed Shampoo)
   int n_active_blocks = 0;
 
   // Newton control state (device) and pinned readback
@@ -866,16 +867,21 @@ int32_t sa_plan_create(const sa_block_desc* blocks, int32_t n_blocks, sa_plan** 
     }
     for (int side = 0; side < SA_MAX_ORDER; ++side) {
       if (!d.factor[side]) {
-        if (d.eigenvectors[side] && d.corrected_eigenvalues) p->eigenvalue_corrected = true;  // fixed basis
+        if (d.eigenvectors[side] && d.corrected_eigenvalues) { p->eigenvalue_corrected = true; p->has_eigvec = true; }  // fixed basis
         continue;
       }
       if ((!d.inv_factor[side] && !d.eigenvectors[side]) || (d.inv_factor[side] && d.root[side] < 1)) {
         delete p;
         return fail(SA_ERR_INVALID, "sa_plan_create: factor without inverse / eigenvector storage or with root < 1");
       }
-      if (d.eigenvectors[side] && !d.corrected_eigenvalues) {
+      if (d.eigenvectors[side] && !d.corrected_eigenvalues && !d.inv_factor[side]) {
         delete p;
-        return fail(SA_ERR_INVALID, "sa_plan_create: eigenvectors without corrected_eigenvalues");
+        return fail(SA_ERR_INVALID, "sa_plan_create: eigenvectors need corrected_eigenvalues (eigenvalue-corrected Shampoo) or "
+                                    "an inverse root (eigendecomposed Shampoo)");
+      }
+      if (d.eigenvectors[side] && d.corrected_eigenvalues && d.inv_factor[side]) {
+        delete p;
+        return fail(SA_ERR_INVALID, "sa_plan_create: a factor has either corrected_eigenvalues or an inverse root, not both");
       }
       Factor f{};
       f.block = b; f.side = side;
@@ -891,7 +897,8 @@ int32_t sa_plan_create(const sa_block_desc* blocks, int32_t n_blocks, sa_plan** 
       f.norm_off = normp;
       f.norm_chunks = (int)(((long long)f.d * (f.d + 1) / 2 + NORM_CHUNK - 1) / NORM_CHUNK);
       normp += f.norm_chunks;
-      if (f.eigvec) p->eigenvalue_corrected = true;
+      if (f.eigvec) p->has_eigvec = true;
+      if (f.eigvec && d.corrected_eigenvalues) p->eigenvalue_corrected = true;
       p->block_factor[side][b] = (int)p->factors.size();
       p->factors.push_back(f);
     }
@@ -2261,7 +2268,7 @@ int32_t sa_compute_root_inverses_eigh(sa_plan* p, float bias_correction2, float 
 int32_t sa_refresh_eigenbases_eigh(sa_plan* p, float bias_correction2, float epsilon, float tolerance, int32_t max_sweeps,
                                    int32_t* sweeps_out, int32_t* status_out, void* stream) {
   if (!p || !sweeps_out || !status_out) return fail(SA_ERR_INVALID, "sa_refresh_eigenbases_eigh: NULL argument");
-  if (!p->eigenvalue_corrected) return fail(SA_ERR_STATE, "plan has no eigenvector state");
+  if (!p->has_eigvec) return fail(SA_ERR_STATE, "plan has no eigenvector state");
   if (!(bias_correction2 != 0.0f) || max_sweeps < 1) return fail(SA_ERR_INVALID, "bad bias correction or max_sweeps");
   hipStream_t s = static_cast<hipStream_t>(stream);
   SACHECK(ensure_tables(p, nullptr, s));
@@ -2425,6 +2432,86 @@ int32_t sa_refresh_eigenbases_eigh(sa_plan* p, float bias_correction2, float eps
   return SA_OK;
 }
 
+// Inverse roots of eigendecomposed Shampoo from the stored eigendecompositions: X = Q diag(w) Q^T with the weights
+// of matrix_inverse_root_from_eigendecomposition (matrix_functions.py:179-279), the same post-processing as the eigh
+// root inverse.  The reference forms these products in every step (shampoo_preconditioner_list.py:1793-1832); they
+// change only when (Q, lambda) change, so they are formed once per amortized computation (and after a checkpoint
+// load) and kept like the inverse roots of root-inverse Shampoo.
+int32_t sa_compute_root_inverses_from_eigendecomposition(sa_plan* p, const float* const* eigenvalues, float epsilon,
+                                                         const float* roots, int32_t stability, float rank_rtol, float rank_atol,
+                                                         int32_t* status_out, void* stream) {
+  if (!p || !eigenvalues || !roots || !status_out)
+    return fail(SA_ERR_INVALID, "sa_compute_root_inverses_from_eigendecomposition: NULL argument");
+  if (!p->has_eigvec || p->eigenvalue_corrected) return fail(SA_ERR_STATE, "plan is not an eigendecomposed-Shampoo plan");
+  if (stability < 0 || stability > 2) return fail(SA_ERR_INVALID, "stability must be 0, 1 or 2");
+  if (stability == 2 && epsilon != 0.0f)
+    return fail(SA_ERR_INVALID, "epsilon=" + std::to_string(epsilon) + " should be 0.0 when using pseudo-inverse!");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SACHECK(ensure_tables(p, nullptr, s));
+  const int F = (int)p->factors.size();
+  std::vector<int> todo;
+  for (int i = 0; i < F; ++i) {
+    status_out[i] = SA_FACTOR_SKIPPED;
+    const Factor& f = p->factors[i];
+    if (!block_active(p, f.block)) continue;
+    if (!f.eigvec || !f.inv) return fail(SA_ERR_STATE, "factor " + std::to_string(i) + " has no eigenvector or inverse-root storage");
+    if (!eigenvalues[i]) return fail(SA_ERR_INVALID, "eigenvalues[" + std::to_string(i) + "] is NULL");
+    if (!(roots[i] > 0.0f)) return fail(SA_ERR_INVALID, "Root " + std::to_string(roots[i]) + " should be positive!");
+    todo.push_back(i);
+  }
+  if (todo.empty()) return SA_OK;
+  // factors that are not recomputed below must keep a valid dense copy of their stored inverse
+  SACHECK(refresh_inverse_cache(p, s));
+  const int n = (int)todo.size();
+  SACHECK(p->t_copy.begin(n));
+  SACHECK(p->t_eigfinal.begin(n));
+  p->eig_gemm.clear();
+  int slabs = 0;
+  for (int k = 0; k < n; ++k) {
+    const Factor& f = p->factors[todo[k]];
+    float* V = newton_buf(p, NB_X0, f);
+    // zero padded copy of Q (the state keeps it d x d)
+    HIPCHECK(hipMemsetAsync(V, 0, sizeof(float) * (size_t)f.dpad * f.dpad, s));
+    Copy2D& C = p->t_copy.host[k];
+    std::memset(&C, 0, sizeof(C));
+    C.src = f.eigvec; C.lds_ = f.d; C.dst = V; C.ldd = f.dpad; C.rows = f.d; C.cols = f.d;
+    EigFinal& J = p->t_eigfinal.host[k];
+    std::memset(&J, 0, sizeof(J));
+    J.lambda_in = eigenvalues[todo[k]];
+    J.lambda_stride = 1;
+    J.V = V;
+    J.Vs = newton_buf(p, NB_S1, f);
+    J.lambda_out = newton_buf(p, NB_MP0, f);
+    J.weight_out = newton_buf(p, NB_MP0, f) + f.dpad;
+    J.d = f.d; J.dpad = f.dpad;
+    J.exponent = -1.0f / roots[todo[k]];
+    J.row_begin = slabs;
+    J.enabled = 1;
+    J.scale_cols = 1;
+    slabs += f.dpad / 8;
+    GemmProblem q{};
+    q.A = J.Vs; q.B = J.V; q.C = newton_buf(p, NB_X1, f);
+    q.lda = q.ldb = q.ldc = f.dpad;
+    q.M = q.N = q.K = f.dpad;
+    q.a_vec = q.b_vec = 1;
+    p->eig_gemm.add(q, false);
+  }
+  SACHECK(p->t_copy.upload(s));
+  SACHECK(p->t_eigfinal.upload(s));
+  SACHECK(p->eig_gemm.commit(s));
+  hipLaunchKernelGGL(copy2d_kernel, dim3(64, n), dim3(256), 0, s, p->t_copy.dev);
+  hipLaunchKernelGGL(eig_weights_kernel, dim3(n), dim3(256), 0, s, p->t_eigfinal.dev, epsilon, stability, rank_rtol, rank_atol);
+  hipLaunchKernelGGL(eig_scale_cols_kernel, dim3(slabs), dim3(256), 0, s, p->t_eigfinal.dev, n);
+  HIPCHECK(hipGetLastError());
+  SACHECK((launch_gemm<A_MK, B_NK, EPI_STORE, false, false>(p->eig_gemm, unit_scalars(), s)));  // (Q w) Q^T
+  std::vector<const float*> X(n);
+  for (int k = 0; k < n; ++k) X[k] = newton_buf(p, NB_X1, p->factors[todo[k]]);
+  size_t ok = 0;
+  SACHECK(root_inverse_epilogue(p, todo, X, status_out, s, &ok));
+  for (size_t i = 0; i < ok; ++i) status_out[todo[i]] = SA_FACTOR_OK;
+  return SA_OK;
+}
+
 int32_t sa_update_corrected_eigenvalues(sa_plan* p, float beta2, float weighting_factor, void* stream) {
   if (!p) return fail(SA_ERR_INVALID, "NULL plan");
   if (!p->eigenvalue_corrected) return fail(SA_ERR_STATE, "plan has no eigenvector state");
@@ -2568,7 +2655,7 @@ static int qr_accumulate(sa_plan* p, const std::vector<int>& ids, hipStream_t s)
 int32_t sa_refresh_eigenbases_qr(sa_plan* p, float bias_correction2, float epsilon, int32_t max_iterations, float tolerance,
                                  int32_t* iterations_out, int32_t* status_out, void* stream) {
   if (!p || !iterations_out || !status_out) return fail(SA_ERR_INVALID, "sa_refresh_eigenbases_qr: NULL argument");
-  if (!p->eigenvalue_corrected) return fail(SA_ERR_STATE, "plan has no eigenvector state");
+  if (!p->has_eigvec) return fail(SA_ERR_STATE, "plan has no eigenvector state");
   if (!(bias_correction2 != 0.0f) || max_iterations < 0) return fail(SA_ERR_INVALID, "bad bias correction or max_iterations");
   hipStream_t s = static_cast<hipStream_t>(stream);
   SACHECK(ensure_tables(p, nullptr, s));

@@ -65,6 +65,7 @@ from optimizers_amd.shampoo_types import (
     DefaultShampooRuntimeConfig,
     DefaultSingleDeviceDistributedConfig,
     DistributedConfig,
+    EigendecomposedShampooPreconditionerConfig,
     EigenvalueCorrectedShampooPreconditionerConfig,
     IterateAveragingConfig,
     PreconditionerConfig,
@@ -113,7 +114,8 @@ class _AmortizedComputation:
         (shampoo_preconditioner_list.py:314-443)."""
         pc = self.preconditioner_config
         cfg = pc.amortized_computation_config
-        if self.soap and isinstance(cfg, EighEigendecompositionConfig):
+        refreshes_basis = self.soap or getattr(self, "eigendecomposed", False)
+        if refreshes_basis and isinstance(cfg, EighEigendecompositionConfig):
             # epsilon * I is added only when the config perturbs before the computation (matrix_functions.py:869-882)
             ridge = group[EPSILON] * float(cfg.rank_deficient_stability_config.perturb_before_computation)
             native.check(
@@ -122,8 +124,8 @@ class _AmortizedComputation:
                 ),
                 "sa_refresh_eigenbases_eigh",
             )
-        elif self.soap:
-            ridge = group[EPSILON] * float(cfg.rank_deficient_stability_config.perturb_before_computation)
+        elif refreshes_basis:
+            ridge = group[EPSILON] * float(getattr(cfg.rank_deficient_stability_config, "perturb_before_computation", False))
             native.check(
                 self.lib.sa_refresh_eigenbases_qr(
                     self.plan, bc2, ridge, cfg.max_iterations, cfg.tolerance, self.iterations, self.status, stream
@@ -176,7 +178,7 @@ class _AmortizedComputation:
                     "To mitigate, check factor matrix before the matrix computation."
                 )
             if st == native.SA_FACTOR_NOT_CONVERGED:
-                if self.soap:
+                if refreshes_basis:
                     pass
                 elif self.use_higher_order:
                     logger.warning("Higher order method did not converge and reached maximum number of iterations!")
@@ -200,6 +202,16 @@ class _AmortizedComputation:
                     f"The number of failed amortized computations for factors {names} exceeded the allowed tolerance. "
                     "The last seen exception was an ArithmeticError of the coupled higher-order iteration."
                 )
+        if getattr(self, "eigendecomposed", False):
+            # the eigenvalues of every factor that was decomposed go into the state; the inverse roots
+            # Q diag(w) Q^T follow from the stored (Q, lambda) of all active factors
+            for i in range(self.n_factors):
+                if int(self.status[i]) in (native.SA_FACTOR_OK, native.SA_FACTOR_NOT_CONVERGED):
+                    native.check(
+                        self.lib.sa_plan_read_eigenvalues(self.plan, i, self.eigenvalue_tensors[i].data_ptr(), stream),
+                        "sa_plan_read_eigenvalues",
+                    )
+            self._inverse_roots_from_eigendecomposition(group, stream)
         # blocks whose root cannot be used by the coupled Newton iteration fail every time
         for k, message in self.bad_root_blocks.items():
             count = self.failed_counter.get(k, 0) + 1
@@ -210,6 +222,30 @@ class _AmortizedComputation:
                 raise ValueError(
                     f"The number of failed amortized computations for factors {names} exceeded the allowed tolerance. "
                     f"The last seen exception was {message}."
+                )
+
+
+    def _inverse_roots_from_eigendecomposition(self, group: dict[str, Any], stream: int) -> None:
+        """Eigendecomposed Shampoo: X = Q diag(w(lambda)) Q^T of every active factor
+        (matrix_functions.py:179-279 as called from shampoo_preconditioner_list.py:1793-1832)."""
+        stab = self.preconditioner_config.amortized_computation_config.rank_deficient_stability_config
+        if isinstance(stab, PseudoInverseConfig):
+            mode, rtol, atol = 2, (-1.0 if stab.rank_rtol is None else float(stab.rank_rtol)), float(stab.rank_atol)
+        else:
+            mode, rtol, atol = int(stab.perturb_before_computation), 0.0, 0.0
+        roots = (ctypes.c_float * max(self.n_factors, 1))(*self.factor_roots)
+        status = (ctypes.c_int32 * max(self.n_factors, 1))()
+        native.check(
+            self.lib.sa_compute_root_inverses_from_eigendecomposition(
+                self.plan, self.eigenvalue_ptrs, group[EPSILON], roots, mode, rtol, atol, status, stream
+            ),
+            "sa_compute_root_inverses_from_eigendecomposition",
+        )
+        for i in range(self.n_factors):
+            if int(status[i]) == native.SA_FACTOR_RESULT_NONFINITE:
+                raise PreconditionerValueError(
+                    f"Encountered nan or inf values in the inverse root formed from the eigendecomposition of factor matrix "
+                    f"{self.factor_names[i]}! To mitigate, check the stored eigenvalues (non-positive after the epsilon shift?)."
                 )
 
 
@@ -268,6 +304,7 @@ class _NativeGroup(_AmortizedComputation):
         self.selectors: list[tuple[bool, ...]] = []
         self.roots: list[tuple[float, ...]] = []
         self.soap = isinstance(pc, EigenvalueCorrectedShampooPreconditionerConfig)
+        self.eigendecomposed = isinstance(pc, EigendecomposedShampooPreconditionerConfig)
         for i in self.native_index:
             order = self.block_specs[i].order
             if self.soap:
@@ -294,7 +331,9 @@ class _NativeGroup(_AmortizedComputation):
         packed = [d * (d + 1) // 2 for d in fdims]
         self.factor_arena = _Arena(packed, self.device)
         self.inv_arena = _Arena(packed, self.device) if not self.soap else None
-        self.eigvec_arena = _Arena([d * d for d in fdims], self.device) if self.soap else None
+        self.eigvec_arena = _Arena([d * d for d in fdims], self.device) if (self.soap or self.eigendecomposed) else None
+        self.eigenvalue_arena = _Arena(list(fdims), self.device) if self.eigendecomposed else None
+        self.eigenvalue_tensors: list[torch.Tensor] = []
         self.corrected_arena = _Arena(numels, self.device) if self.soap else None
         self.filtered_arena = _Arena(numels, self.device) if beta1 != 0.0 else None
         self.adagrad_arena = _Arena(numels, self.device) if self.graft_type == native.SA_GRAFT_ADAGRAD else None
@@ -305,7 +344,7 @@ class _NativeGroup(_AmortizedComputation):
         self.factor_names: list[str] = []
         self.factor_block: list[int] = []
         self.factor_roots: list[float] = []
-        self.use_eigh = isinstance(pc.amortized_computation_config, EigenConfig)
+        self.use_eigh = isinstance(pc.amortized_computation_config, EigenConfig) or self.eigendecomposed
         self.use_higher_order = isinstance(pc.amortized_computation_config, CoupledHigherOrderConfig)
         self._slots: list[tuple[torch.Tensor, str, tuple, torch.Tensor]] = []
         self.bad_root_blocks: dict[int, str] = {}
@@ -327,6 +366,8 @@ class _NativeGroup(_AmortizedComputation):
             shampoo_state: dict[str, Any] = (
                 {"factor_matrices": {}, "factor_matrices_eigenvectors": {}}
                 if self.soap
+                else {"factor_matrices": {}, "factor_matrices_eigenvectors": {}, "factor_matrices_eigenvalues": {}}
+                if self.eigendecomposed
                 else {"factor_matrices": {}, "inv_factor_matrices": {}}
             )
             if self.soap:
@@ -348,19 +389,27 @@ class _NativeGroup(_AmortizedComputation):
                 shampoo_state["factor_matrices"][slot] = f
                 d.factor[dim] = f.data_ptr()
                 self._slots.append((p, s.block_key, (SHAMPOO, "factor_matrices", slot), f))
-                if self.soap:
+                if self.soap or self.eigendecomposed:
                     q = self.eigvec_arena.view(fi, (n, n))
                     q.copy_(torch.eye(n, device=self.device))
                     shampoo_state["factor_matrices_eigenvectors"][slot] = q
                     d.eigenvectors[dim] = q.data_ptr()
                     self._slots.append((p, s.block_key, (SHAMPOO, "factor_matrices_eigenvectors", slot), q))
-                else:
+                if self.eigendecomposed:
+                    # eigenvalues start at one, eigenvectors at the identity (shampoo_preconditioner_list.py:730-750)
+                    lam = self.eigenvalue_arena.view(fi, (n,))
+                    lam.fill_(1.0)
+                    shampoo_state["factor_matrices_eigenvalues"][slot] = lam
+                    self.eigenvalue_tensors.append(lam)
+                    self._slots.append((p, s.block_key, (SHAMPOO, "factor_matrices_eigenvalues", slot), lam))
+                if not self.soap:
                     inv = self.inv_arena.view(fi, (n * (n + 1) // 2,))
                     idx = torch.arange(n, device=self.device)
                     inv[idx * n - idx * (idx - 1) // 2] = 1.0  # packed identity
-                    shampoo_state["inv_factor_matrices"][slot] = inv
                     d.inv_factor[dim] = inv.data_ptr()
-                    self._slots.append((p, s.block_key, (SHAMPOO, "inv_factor_matrices", slot), inv))
+                    if not self.eigendecomposed:  # eigendecomposed Shampoo keeps Q diag(w) Q^T as a private cache
+                        shampoo_state["inv_factor_matrices"][slot] = inv
+                        self._slots.append((p, s.block_key, (SHAMPOO, "inv_factor_matrices", slot), inv))
                 root = Fraction(self.roots[k][slot])
                 self.factor_roots.append(float(self.roots[k][slot]))
                 if self.use_eigh or self.soap:
@@ -425,6 +474,8 @@ class _NativeGroup(_AmortizedComputation):
             self.n_factors = 0
         self.iterations = (ctypes.c_int32 * max(self.n_factors, 1))()
         self.status = (ctypes.c_int32 * max(self.n_factors, 1))()
+        self.eigenvalue_ptrs = (ctypes.c_void_p * max(self.n_factors, 1))(*(t.data_ptr() for t in self.eigenvalue_tensors))
+        self.inverse_roots_stale = False  # set when (Q, lambda) were written from outside (checkpoint load)
         self.grad_ptrs = (ctypes.c_void_p * max(nb, 1))()
         self.last_newton_iterations: list[int] = []
         self.max_jacobi_sweeps = 30
@@ -452,10 +503,24 @@ class _NativeGroup(_AmortizedComputation):
     def _check_supported(group: dict[str, Any], pc: PreconditionerConfig) -> None:
         if not isinstance(group[DISTRIBUTED_CONFIG], SingleDeviceDistributedConfig):
             raise NotImplementedError(f"{group[DISTRIBUTED_CONFIG]=} not supported!")
-        if not isinstance(pc, (RootInvShampooPreconditionerConfig, EigenvalueCorrectedShampooPreconditionerConfig)):
+        if not isinstance(
+            pc,
+            (RootInvShampooPreconditionerConfig, EigenvalueCorrectedShampooPreconditionerConfig, EigendecomposedShampooPreconditionerConfig),
+        ):
             raise NotImplementedError(f"{pc=} not supported!")
         acc = pc.amortized_computation_config
-        if isinstance(pc, EigenvalueCorrectedShampooPreconditionerConfig):
+        if isinstance(pc, EigendecomposedShampooPreconditionerConfig):
+            if not isinstance(acc, (QREigendecompositionConfig, EighEigendecompositionConfig)):
+                raise NotImplementedError(
+                    f"Eigendecomposition config is not implemented! Specified eigendecomposition config is {type(acc).__name__}."
+                )
+            if not isinstance(acc.rank_deficient_stability_config, (PerturbationConfig, PseudoInverseConfig)):
+                raise NotImplementedError(f"{acc.rank_deficient_stability_config=} is not supported.")
+            if isinstance(acc, EighEigendecompositionConfig) and acc.eigendecomposition_offload_device != "":
+                raise NotImplementedError("eigendecomposition_offload_device: the decomposition runs on the MI355X")
+            if pc.factor_matrix_eigenvectors_dtype != torch.float32 or pc.factor_matrix_eigenvalues_dtype != torch.float32:
+                raise NotImplementedError("eigenvectors and eigenvalues are fp32 in the native step")
+        elif isinstance(pc, EigenvalueCorrectedShampooPreconditionerConfig):
             if not isinstance(acc, (QREigendecompositionConfig, EighEigendecompositionConfig)):
                 raise NotImplementedError(
                     f"Eigendecomposition config is not implemented! Specified eigendecomposition config is {type(acc).__name__}."
@@ -583,6 +648,10 @@ class _NativeGroup(_AmortizedComputation):
             bc2 = float(torch.tensor(1.0) - beta2**step)
         if amortize:
             self._amortized_computation(group, bc2, stream)
+            self.inverse_roots_stale = False
+        elif self.eigendecomposed and self.inverse_roots_stale and not graft_only:
+            self._inverse_roots_from_eigendecomposition(group, stream)
+            self.inverse_roots_stale = False
         if self.soap:
             native.check(
                 lib.sa_update_corrected_eigenvalues(self.plan, beta2, weighting, stream), "sa_update_corrected_eigenvalues"
@@ -643,8 +712,9 @@ class DistributedShampoo(torch.optim.Optimizer):
     Arguments, defaults and validation follow the reference constructor
     (distributed_shampoo/distributed_shampoo.py:361-535).  Built natively:
     `RootInvShampooPreconditionerConfig` with `CoupledNewtonConfig`, `CoupledHigherOrderConfig` (orders 2..8) or
-    `EigenConfig` (`PerturbationConfig` and `PseudoInverseConfig`), `use_trace_scaling`, `EigenvalueCorrectedShampooPreconditionerConfig` with `QREigendecompositionConfig` or
-    `EighEigendecompositionConfig` (including `ignored_basis_change_dims`), grafting with SGD / AdaGrad / RMSprop /
+    `EigenConfig` (`PerturbationConfig` and `PseudoInverseConfig`), `use_trace_scaling`,
+    `EigenvalueCorrectedShampooPreconditionerConfig` and `EigendecomposedShampooPreconditionerConfig` with
+    `QREigendecompositionConfig` or `EighEigendecompositionConfig` (including `ignored_basis_change_dims`), grafting with SGD / AdaGrad / RMSprop /
     Adam or none, every `WeightDecayType`, `ClassicMomentumConfig`, `inverse_exponent_override`,
     `SingleDeviceDistributedConfig`, fp32 state with packed factor matrices, blocks of order 1 to 3 (order 3: what is left of
     convolution weights).
@@ -831,6 +901,8 @@ def _restore_state(self: _NativeGroup, optimizer: DistributedShampoo) -> None:
         optimizer.state[p][STEP] = self.step_tensor
     if self.plan:
         native.check(self.lib.sa_plan_invalidate_inverse_cache(self.plan), "sa_plan_invalidate_inverse_cache")
+    # eigendecomposed Shampoo: the inverse roots are a function of the restored (Q, lambda)
+    self.inverse_roots_stale = self.eigendecomposed
 
 
 _NativeGroup.restore_state = _restore_state  # type: ignore[attr-defined]

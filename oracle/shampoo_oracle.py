@@ -288,6 +288,19 @@ def eigh_inverse_root(a: Tensor, root: float, eps: float = 0.0) -> Tensor:
     return q * lam.pow(-1.0 / root).unsqueeze(0) @ q.T
 
 
+def inverse_root_from_eigendecomposition(lam: Tensor, q: Tensor, root: float, eps: float = 0.0) -> Tensor:
+    """matrix_functions.py:179-279 with the default PerturbationConfig(perturb_before_computation=True):
+    the eigenvalues are used as they are unless their minimum is below eps, in which case they are
+    shifted to start at eps (two rounded additions); X = Q diag(lam^(-1/root)) Q^T.
+    Pinned by the same identity as eigh_inverse_root (which is this function applied to torch.linalg.eigh)
+    and by the eigendecomposed-Shampoo fixtures written from the reference."""
+    lmin = torch.min(lam).item()
+    if lmin < eps:
+        lam = lam + (-lmin)
+        lam = lam + eps
+    return q * lam.pow(-1.0 / root).unsqueeze(0) @ q.T
+
+
 def eigh_pseudo_inverse_root(
     a: Tensor, root: float, rank_rtol: float | None = None, rank_atol: float = 0.0
 ) -> Tensor:
@@ -341,7 +354,8 @@ class OracleConfig:
 
     preconditioner: "newton" | "higher_order" | "eigh" (RootInvShampooPreconditionerConfig with
     CoupledNewtonConfig / CoupledHigherOrderConfig / EigenConfig) or "soap_qr" | "soap_eigh"
-    (EigenvalueCorrectedShampooPreconditionerConfig).
+    (EigenvalueCorrectedShampooPreconditionerConfig) or "eigendecomposed_eigh" | "eigendecomposed_qr"
+    (EigendecomposedShampooPreconditionerConfig).
     grafting: None | "adam" | "rmsprop" | "adagrad" | "sgd".
     """
 
@@ -401,6 +415,7 @@ class ShampooOracle:
             raise ValueError("start_preconditioning_step must be >= precondition_frequency")
         self.step_t = torch.tensor(0, dtype=torch.int64)
         self.soap = cfg.preconditioner.startswith("soap")
+        self.eigendecomposed = cfg.preconditioner.startswith("eigendecomposed")
         self.blocks: list[Tensor] = []
         self.block_ids: list[tuple[int, str]] = []
         self.num_blocks_per_param: list[int] = []
@@ -447,6 +462,10 @@ class ShampooOracle:
         if self.soap:
             st["eigvecs"] = [torch.eye(d, dtype=dt, device=dev) for d in dims]
             st["corrected"] = torch.zeros(b.shape, dtype=dt, device=dev)
+        elif self.eigendecomposed:
+            # shampoo_preconditioner_list.py:730-750: identity eigenvectors, unit eigenvalues
+            st["eigvecs"] = [torch.eye(d, dtype=dt, device=dev) for d in dims]
+            st["eigvals"] = [torch.ones(d, dtype=dt, device=dev) for d in dims]
         else:
             if cfg.use_symmetric_packing:
                 st["inv"] = [packed_eye(d, dt, dev) for d in dims]
@@ -517,7 +536,15 @@ class ShampooOracle:
                     f"Encountered nan/inf values in factor matrix {name}! "
                 )
             try:
-                if self.soap:
+                if self.eigendecomposed:
+                    # shampoo_preconditioner_list.py:868-940: matrix_eigendecomposition started from the stored basis
+                    if cfg.preconditioner == "eigendecomposed_qr":
+                        vals, res = qr_refresh(a, st["eigvecs"][k], cfg.epsilon, cfg.qr_max_iterations, cfg.qr_tolerance)
+                    else:
+                        vals, res = torch.linalg.eigh(ridge(a, cfg.epsilon))
+                    eigenvalues = vals
+                    key, packed = "eigvecs", res
+                elif self.soap:
                     if cfg.preconditioner == "soap_qr":
                         _, res = qr_refresh(
                             a, st["eigvecs"][k], cfg.epsilon, cfg.qr_max_iterations, cfg.qr_tolerance
@@ -548,9 +575,15 @@ class ShampooOracle:
             except Exception as exc:  # keep the previous result, count the failure
                 last_exc = exc
                 continue
+            if self.eigendecomposed:  # both computed quantities are checked, eigenvalues first (:401-426)
+                if not torch.isfinite(eigenvalues).all():
+                    raise OraclePreconditionerValueError(
+                        f"Encountered nan or inf values in eigenvalues of factor matrix {name}! "
+                    )
+                st["eigvals"][k].copy_(eigenvalues)
             if not torch.isfinite(packed).all():
                 raise OraclePreconditionerValueError(
-                    f"Encountered nan or inf values in {'eigenvectors' if self.soap else 'matrices'} of factor matrix {name}! "
+                    f"Encountered nan or inf values in {'eigenvectors' if (self.soap or self.eigendecomposed) else 'matrices'} of factor matrix {name}! "
                 )
             st[key][k].copy_(packed)
         if last_exc is None:
@@ -573,6 +606,13 @@ class ShampooOracle:
     def _shampoo_direction(self, st: dict[str, Any], ghat: Tensor) -> Tensor:
         cfg = self.cfg
         sel = st["selector"]
+        if self.eigendecomposed:
+            # shampoo_preconditioner_list.py:1800-1832: the inverse roots are formed from (lambda, Q) in every step
+            mats = [
+                inverse_root_from_eigendecomposition(lam, q, Fraction(r), cfg.epsilon)
+                for lam, q, r in zip(st["eigvals"], st["eigvecs"], st["roots"])
+            ]
+            return self._contract(ghat, sel, mats)
         if not self.soap:
             mats = [self._unpack(p) for p in st["inv"]]
             return self._contract(ghat, sel, mats)

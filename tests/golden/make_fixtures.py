@@ -43,7 +43,9 @@ from distributed_shampoo import (  # noqa: E402
     DefaultSOAPConfig,
     DistributedShampoo,
     EigenConfig,
+    EigendecomposedShampooPreconditionerConfig,
     EigenvalueCorrectedShampooPreconditionerConfig,
+    EighEigendecompositionConfig,
     QREigendecompositionConfig,
     RootInvShampooPreconditionerConfig,
     WeightDecayType,
@@ -152,6 +154,22 @@ CASES = {
         max_preconditioner_dim=16, precondition_frequency=2, start_preconditioning_step=2,
         preconditioner="soap_eigh", override_1d=False, grafting="adam", grafting_beta2=0.99, grafting_epsilon=1e-8,
     ),
+    # EigendecomposedShampooPreconditionerConfig, default eigh, 1-D blocks preconditioned too (their rank-deficient
+    # factors are well posed only with an epsilon above the fp32 resolution of the spectrum)
+    "eigendecomposed_eigh": dict(
+        shapes=[[24, 20], [20]], seed=14, grad_scale=1.0, steps=8,
+        lr=1e-2, betas=[0.9, 0.99], epsilon=1e-4, weight_decay=1e-3, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=16, precondition_frequency=2, start_preconditioning_step=4,
+        preconditioner="eigendecomposed_eigh", override_1d=False, grafting="adam", grafting_beta2=0.99, grafting_epsilon=1e-8,
+    ),
+    # the same family with the QR algorithm started from the stored eigenvectors; the first refresh comes when the
+    # order-16 factor of the 16 x 4 block has seen five gradients (rank 20), so no null space makes the basis arbitrary
+    "eigendecomposed_qr": dict(
+        shapes=[[24, 20], [20]], seed=15, grad_scale=1.0, steps=10,
+        lr=1e-2, betas=[0.9, 0.99], epsilon=1e-6, weight_decay=0.0, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=16, precondition_frequency=1, start_preconditioning_step=5,
+        preconditioner="eigendecomposed_qr", override_1d=True, grafting="adagrad", grafting_epsilon=1e-8,
+    ),
     "cfg1_override": dict(  # benchmark configuration 1 with 1-D blocks left to grafting
         shapes=[[512, 512], [512]], seed=0, grad_scale=1.0, steps=10, zero_init=True, torch_seed_grads=True,
         lr=1e-3, betas=[0.9, 0.999], epsilon=1e-12, weight_decay=0.0, weight_decay_type="DECOUPLED",
@@ -189,6 +207,13 @@ def build_reference(c, params):
         assert pc == DefaultSOAPConfig
     elif c["preconditioner"] == "soap_eigh":
         pc = EigenvalueCorrectedShampooPreconditionerConfig()
+    elif c["preconditioner"] in ("eigendecomposed_eigh", "eigendecomposed_qr"):
+        pc = EigendecomposedShampooPreconditionerConfig(
+            amortized_computation_config=(
+                QREigendecompositionConfig() if c["preconditioner"].endswith("qr") else EighEigendecompositionConfig()
+            ),
+            inverse_exponent_override={1: {0: 0.0}} if c["override_1d"] else {},
+        )
     else:
         raise ValueError(c["preconditioner"])
     graft = {
@@ -278,7 +303,8 @@ def run_case(name, c):
                     if isinstance(sv, torch.Tensor):
                         out[f"state_p{pi}_{key}_{sk}"] = sv.numpy().copy()
                     elif sk == "shampoo":
-                        for fname in ("factor_matrices", "inv_factor_matrices", "factor_matrices_eigenvectors"):
+                        for fname in ("factor_matrices", "inv_factor_matrices", "factor_matrices_eigenvectors",
+                                      "factor_matrices_eigenvalues"):
                             for k, t in enumerate(getattr(sv, fname, ())):
                                 out[f"state_p{pi}_{key}_{fname}_{k}"] = t.numpy().copy()
                         if hasattr(sv, "corrected_eigenvalues"):

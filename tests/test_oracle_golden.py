@@ -44,6 +44,8 @@ def test_multi_step_matches_reference(name):
                 assert rel_err(f, z[pre + f"inv_factor_matrices_{j}"]) < 2e-5
             for j, f in enumerate(st.get("eigvecs", [])):
                 assert rel_err(f, z[pre + f"factor_matrices_eigenvectors_{j}"]) < 2e-5
+            for j, f in enumerate(st.get("eigvals", [])):
+                assert rel_err(f, z[pre + f"factor_matrices_eigenvalues_{j}"]) < 2e-5
             if "corrected" in st:
                 assert rel_err(st["corrected"], z[pre + "corrected_eigenvalues"]) < 2e-5
             if "adagrad" in st:
