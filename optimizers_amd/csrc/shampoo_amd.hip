@@ -2268,6 +2268,7 @@ int32_t sa_compute_root_inverses_eigh(sa_plan* p, float bias_correction2, float 
 int32_t sa_refresh_eigenbases_eigh(sa_plan* p, float bias_correction2, float epsilon, float tolerance, int32_t max_sweeps,
                                    int32_t* sweeps_out, int32_t* status_out, void* stream) {
   if (!p || !sweeps_out || !status_out) return fail(SA_ERR_INVALID, "sa_refresh_eigenbases_eigh: NULL argument");
+  if (p->factors.empty()) return SA_OK;  // nothing is preconditioned
   if (!p->has_eigvec) return fail(SA_ERR_STATE, "plan has no eigenvector state");
   if (!(bias_correction2 != 0.0f) || max_sweeps < 1) return fail(SA_ERR_INVALID, "bad bias correction or max_sweeps");
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -2442,6 +2443,7 @@ int32_t sa_compute_root_inverses_from_eigendecomposition(sa_plan* p, const float
                                                          int32_t* status_out, void* stream) {
   if (!p || !eigenvalues || !roots || !status_out)
     return fail(SA_ERR_INVALID, "sa_compute_root_inverses_from_eigendecomposition: NULL argument");
+  if (p->factors.empty()) return SA_OK;  // nothing is preconditioned
   if (!p->has_eigvec || p->eigenvalue_corrected) return fail(SA_ERR_STATE, "plan is not an eigendecomposed-Shampoo plan");
   if (stability < 0 || stability > 2) return fail(SA_ERR_INVALID, "stability must be 0, 1 or 2");
   if (stability == 2 && epsilon != 0.0f)
@@ -2655,6 +2657,7 @@ static int qr_accumulate(sa_plan* p, const std::vector<int>& ids, hipStream_t s)
 int32_t sa_refresh_eigenbases_qr(sa_plan* p, float bias_correction2, float epsilon, int32_t max_iterations, float tolerance,
                                  int32_t* iterations_out, int32_t* status_out, void* stream) {
   if (!p || !iterations_out || !status_out) return fail(SA_ERR_INVALID, "sa_refresh_eigenbases_qr: NULL argument");
+  if (p->factors.empty()) return SA_OK;  // nothing is preconditioned
   if (!p->has_eigvec) return fail(SA_ERR_STATE, "plan has no eigenvector state");
   if (!(bias_correction2 != 0.0f) || max_iterations < 0) return fail(SA_ERR_INVALID, "bad bias correction or max_iterations");
   hipStream_t s = static_cast<hipStream_t>(stream);
