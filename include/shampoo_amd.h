@@ -303,6 +303,13 @@ int32_t sa_set_symmetric_newton(int32_t policy);
  * Process wide.  No counterpart in the reference. */
 int32_t sa_set_eigh_solver(int32_t solver);
 
+/* KL-Shampoo (RootInvKLShampooPreconditionerConfig / EigendecomposedKLShampooPreconditionerConfig,
+ * shampoo_preconditioner_list.py:1945-2046): with `enabled`, sa_update_factor_matrices takes the Gram matrices of a
+ * block with two Kronecker factors from the gradient preconditioned along the other dim with the stored inverse
+ * root, L <- beta2 L + w (G X_R)(G X_R)^T and R <- beta2 R + w (X_L G)^T (X_L G); blocks with one factor are
+ * unchanged.  Order-3 blocks with more than one factor are rejected. */
+int32_t sa_plan_set_kl_shampoo(sa_plan* plan, int32_t enabled);
+
 /* Trace scaling (use_trace_scaling / trace_scaling_exponent, shampoo_preconditioner_list.py:366-371): when
  * enabled, every root-inverse and eigenbasis computation of this plan works on
  *   (factor / bias_correction2) * max(trace(factor / bias_correction2), floor) ^ (-exponent)

@@ -239,6 +239,9 @@ struct sa_plan {
   Table<ChunkRef> t_chunks;
   Table<int> t_active_blocks;
   GemmTable syrk0, syrk1, g1_store, g1_norm, g2_norm, g2g_norm;
+  // KL-Shampoo: the Gram matrices of a two-sided block are taken of the gradient preconditioned along the other dim
+  bool kl = false;
+  GemmTable kl_right, kl_left;  // G X_R -> T buffer, X_L G -> P buffer
   // Newton, [0] full products / [1] symmetric products: X*M_p with M_p^2 per parity, power chain, M update per parity
   GemmTable nt_a[2][2], nt_pow[2][8], nt_m[2][2];
   GemmTable nt_h[8];      // Horner products of the higher-order iteration
@@ -417,9 +420,44 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
   // factor-update tables
   p->syrk0.clear();
   p->syrk1.clear();
+  p->kl_right.clear();
+  p->kl_left.clear();
   for (int b : active) {
     const sa_block_desc& d = p->blocks[b];
     const float* G = p->grads[b];
+    if (p->kl && d.mid == 0 && d.factor[0] && d.factor[1]) {
+      // KL-Shampoo (shampoo_preconditioner_list.py:1945-1987): L from G X_R, R from X_L G, X the stored inverse roots
+      const Factor& fl = p->factors[p->block_factor[0][b]];
+      const Factor& fr = p->factors[p->block_factor[1][b]];
+      const float* XL = p->f(p->off_inv_dense) + fl.dense_off;
+      const float* XR = p->f(p->off_inv_dense) + fr.dense_off;
+      const long long eo = p->elem_off[b];
+      float* TR = tbuf(p) + eo;
+      float* TL = pbuf(p) + eo;
+      GemmProblem r{};
+      r.A = G; r.lda = d.ld; r.a_vec = vec_ok(G, d.ld);
+      r.B = XR; r.ldb = fr.dpad; r.b_vec = vec_ok(XR, fr.dpad);
+      r.C = TR; r.ldc = d.cols; r.M = d.rows; r.N = d.cols; r.K = d.cols;
+      p->kl_right.add(r, false);
+      GemmProblem l{};
+      l.A = XL; l.lda = fl.dpad; l.a_vec = vec_ok(XL, fl.dpad);
+      l.B = G; l.ldb = d.ld; l.b_vec = vec_ok(G, d.ld);
+      l.C = TL; l.ldc = d.cols; l.M = d.rows; l.N = d.cols; l.K = d.rows;
+      p->kl_left.add(l, false);
+      GemmProblem q{};
+      q.A = TR; q.B = TR; q.C = d.factor[0];
+      q.lda = d.cols; q.ldb = d.cols; q.ldc = 0;
+      q.M = d.rows; q.N = d.rows; q.K = d.cols;
+      q.a_vec = q.b_vec = vec_ok(TR, d.cols);
+      p->syrk0.add(q, true);
+      GemmProblem w{};
+      w.A = TL; w.B = TL; w.C = d.factor[1];
+      w.lda = d.cols; w.ldb = d.cols; w.ldc = 0;
+      w.M = d.cols; w.N = d.cols; w.K = d.rows;
+      w.a_vec = w.b_vec = vec_ok(TL, d.cols);
+      p->syrk1.add(w, true);
+      continue;
+    }
     if (d.mid > 0) {
       // order 3, from the dense copies: factor k = unfolding_k unfolding_k^T
       const BlockDev& B = p->t_blocks.host[b];
@@ -456,6 +494,8 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
   }
   SACHECK(p->syrk0.commit(s));
   SACHECK(p->syrk1.commit(s));
+  SACHECK(p->kl_right.commit(s));
+  SACHECK(p->kl_left.commit(s));
 
   // eigenvalue-corrected tables
   for (GemmTable* g : {&p->ec_stat1, &p->ec_stat2, &p->ec_stat_l, &p->ec_stat_r, &p->ec_p1, &p->ec_p1d, &p->ec_p2, &p->ec_p2d,
@@ -796,6 +836,21 @@ double sa_phase_executed_flops(const char* phase) {
   auto it = g_phases.find(phase ? phase : "");
   return it == g_phases.end() ? -1.0 : it->second.executed;
 }
+int32_t sa_plan_set_kl_shampoo(sa_plan* p, int32_t enabled) {
+  if (!p) return fail(SA_ERR_INVALID, "NULL plan");
+  if (enabled) {
+    if (p->eigenvalue_corrected) return fail(SA_ERR_STATE, "KL-Shampoo needs inverse roots: not an eigenvalue-corrected plan");
+    for (int b = 0; b < p->n_blocks; ++b) {
+      const sa_block_desc& d = p->blocks[b];
+      if (d.mid > 0 && (d.factor[0] != nullptr) + (d.factor[1] != nullptr) + (d.factor[2] != nullptr) > 1)
+        return fail(SA_ERR_UNSUPPORTED, "KL-Shampoo is built for blocks of order 1 and 2");
+    }
+  }
+  p->kl = enabled != 0;
+  p->tables_valid = false;
+  return SA_OK;
+}
+
 int32_t sa_plan_set_trace_scaling(sa_plan* p, int32_t enabled, float exponent, float floor) {
   if (!p) return fail(SA_ERR_INVALID, "sa_plan_set_trace_scaling: null plan");
   if (enabled && !(exponent > 0.0f && exponent <= 1.0f))
@@ -930,6 +985,7 @@ int32_t sa_plan_create(const sa_block_desc* blocks, int32_t n_blocks, sa_plan** 
 void sa_plan_destroy(sa_plan* p) {
   if (!p) return;
   p->t_blocks.destroy(); p->t_chunks.destroy(); p->t_active_blocks.destroy();
+  for (GemmTable* g : {&p->kl_right, &p->kl_left}) g->t.destroy();
   for (GemmTable* g : {&p->syrk0, &p->syrk1, &p->g1_store, &p->g1_norm, &p->g2_norm, &p->g2g_norm, &p->nt_a[0][0],
                        &p->nt_a[0][1], &p->nt_m[0][0], &p->nt_m[0][1], &p->nt_a[1][0], &p->nt_a[1][1], &p->nt_m[1][0],
                        &p->nt_m[1][1]})
@@ -1014,6 +1070,11 @@ int32_t sa_update_factor_matrices(sa_plan* p, float beta2, float weighting_facto
   if (p->has_order3 && p->t_chunks.n) {
     hipLaunchKernelGGL(gather3_kernel, dim3((unsigned)p->t_chunks.n), dim3(EW_THREADS), 0, s, p->t_blocks.dev, p->t_chunks.dev, 0);
     HIPCHECK(hipGetLastError());
+  }
+  if (p->kl && (p->kl_right.total_tiles || p->kl_left.total_tiles)) {
+    SACHECK(refresh_inverse_cache(p, s));
+    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE>(p->kl_right, unit_scalars(), s)));
+    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE>(p->kl_left, unit_scalars(), s)));
   }
   Span span("syrk", s, flops, launches, true);
   SACHECK((launch_gemm_auto<A_MK, B_NK, EPI_SYRK_EMA>(p->syrk0, sc, s)));

@@ -35,7 +35,7 @@ EXPORTS = (
     "sa_apply_update", "sa_grafting_only_step", "sa_plan_read_norms", "sa_plan_read_preconditioned",
     "sa_gemm_f32", "sa_copy_f32", "sa_set_profiling", "sa_phase_ms", "sa_phase_flops", "sa_phase_launches", "sa_phase_executed_flops", "sa_set_symmetric_newton", "sa_set_eigh_solver",
     "sa_plan_set_trace_scaling", "sa_compute_root_inverses_higher_order", "sa_plan_read_eigenvalues", "sa_add_to_views",
-    "sa_compute_root_inverses_from_eigendecomposition",
+    "sa_compute_root_inverses_from_eigendecomposition", "sa_plan_set_kl_shampoo",
 )
 
 
@@ -159,6 +159,7 @@ def load() -> ctypes.CDLL:
     lib.sa_compute_root_inverses_from_eigendecomposition.argtypes = [
         c_void_p, POINTER(c_void_p), c_float, POINTER(c_float), c_int32, c_float, c_float, POINTER(c_int32), c_void_p,
     ]
+    lib.sa_plan_set_kl_shampoo.argtypes = [c_void_p, c_int32]
     lib.sa_add_to_views.argtypes = [POINTER(View), POINTER(View), c_int32, c_void_p]
     lib.sa_set_profiling.argtypes = [c_int32]
     lib.sa_phase_ms.argtypes = [c_char_p]

@@ -32,8 +32,10 @@ from optimizers_amd.matrix_functions_types import (
 )
 from optimizers_amd.shampoo_types import (
     EPSILON,
+    EigendecomposedKLShampooPreconditionerConfig,
     EigendecomposedShampooPreconditionerConfig,
     EigenvalueCorrectedShampooPreconditionerConfig,
+    RootInvKLShampooPreconditionerConfig,
     RootInvShampooPreconditionerConfig,
 )
 
@@ -126,6 +128,7 @@ class EigendecomposedShampooKroneckerFactorsState:
 class _NativeShampooPreconditionerList(PreconditionerList, _AmortizedComputation):
     soap = False
     eigendecomposed = False
+    kl = False
 
     def __init__(
         self,
@@ -316,6 +319,8 @@ class _NativeShampooPreconditionerList(PreconditionerList, _AmortizedComputation
         pc = self.preconditioner_config
         if pc.use_trace_scaling:
             native.check(self.lib.sa_plan_set_trace_scaling(self.plan, 1, pc.trace_scaling_exponent, self._epsilon), "sa_plan_set_trace_scaling")
+        if self.kl:
+            native.check(self.lib.sa_plan_set_kl_shampoo(self.plan, 1), "sa_plan_set_kl_shampoo")
         self._plan_strides = strides
 
     def _bind(self, masked_grad_list: tuple[Tensor, ...]) -> int:
@@ -447,6 +452,28 @@ class EigendecomposedShampooPreconditionerList(_NativeShampooPreconditionerList)
         _NativeGroup._check_supported({"distributed_config": _single_device(), "iterate_averaging_config": None}, self.preconditioner_config)
 
     _get_inverse_exponent = RootInvShampooPreconditionerList._get_inverse_exponent
+
+
+class RootInvKLShampooPreconditionerList(RootInvShampooPreconditionerList):
+    """Root-inverse KL-Shampoo (shampoo_preconditioner_list.py:1945-1987)."""
+
+    kl = True
+
+    def _check_config(self) -> None:
+        if not isinstance(self.preconditioner_config, RootInvKLShampooPreconditionerConfig):
+            raise NotImplementedError(f"{self.preconditioner_config=} not supported!")
+        super()._check_config()
+
+
+class EigendecomposedKLShampooPreconditionerList(EigendecomposedShampooPreconditionerList):
+    """Eigendecomposed KL-Shampoo (shampoo_preconditioner_list.py:1989-2046)."""
+
+    kl = True
+
+    def _check_config(self) -> None:
+        if not isinstance(self.preconditioner_config, EigendecomposedKLShampooPreconditionerConfig):
+            raise NotImplementedError(f"{self.preconditioner_config=} not supported!")
+        super()._check_config()
 
 
 def _single_device():

@@ -389,6 +389,7 @@ class OracleConfig:
     use_nesterov: bool = False
     use_symmetric_packing: bool = True
     num_tolerated_failed_amortized_computations: int = 3
+    kl: bool = False  # RootInvKLShampooPreconditionerConfig / EigendecomposedKLShampooPreconditionerConfig
     use_trace_scaling: bool = False  # shampoo_types.py:187-188
     trace_scaling_exponent: float = 0.5
 
@@ -512,9 +513,17 @@ class ShampooOracle:
             order = g.dim()
             ks = [k for k in range(order) if st["selector"][k]]
             outer = []
-            for k in ks:
+            mats = self._inverse_roots(st) if cfg.kl else None
+            for idx_of_k, k in enumerate(ks):
                 rest = [d for d in range(order) if d != k]
-                outer.append(self._pack(torch.tensordot(g, g, dims=[rest, rest])))
+                src = g
+                if cfg.kl:
+                    # shampoo_preconditioner_list.py:1945-2046: the gradient preconditioned along every other
+                    # preconditioned dim with the stored inverse roots
+                    local = list(st["selector"])
+                    local[k] = False
+                    src = self._contract(g, local, [m for i, m in enumerate(mats) if i != idx_of_k])
+                outer.append(self._pack(torch.tensordot(src, src, dims=[rest, rest])))
             for f, o in zip(st["factors"], outer):
                 if beta2 != 1.0:
                     f.mul_(beta2)
@@ -603,19 +612,20 @@ class ShampooOracle:
         den = (st["adagrad"] / self.bc2_graft).sqrt_().add_(self.cfg.grafting_epsilon)
         return ghat / den
 
+    def _inverse_roots(self, st: dict[str, Any]) -> list[Tensor]:
+        if self.eigendecomposed:
+            # shampoo_preconditioner_list.py:1800-1832: the inverse roots are formed from (lambda, Q) in every step
+            return [
+                inverse_root_from_eigendecomposition(lam, q, Fraction(r), self.cfg.epsilon)
+                for lam, q, r in zip(st["eigvals"], st["eigvecs"], st["roots"])
+            ]
+        return [self._unpack(p) for p in st["inv"]]
+
     def _shampoo_direction(self, st: dict[str, Any], ghat: Tensor) -> Tensor:
         cfg = self.cfg
         sel = st["selector"]
-        if self.eigendecomposed:
-            # shampoo_preconditioner_list.py:1800-1832: the inverse roots are formed from (lambda, Q) in every step
-            mats = [
-                inverse_root_from_eigendecomposition(lam, q, Fraction(r), cfg.epsilon)
-                for lam, q, r in zip(st["eigvals"], st["eigvecs"], st["roots"])
-            ]
-            return self._contract(ghat, sel, mats)
         if not self.soap:
-            mats = [self._unpack(p) for p in st["inv"]]
-            return self._contract(ghat, sel, mats)
+            return self._contract(ghat, sel, self._inverse_roots(st))
         # shampoo_preconditioner_list.py:1914-1942
         rot = self._contract(ghat.clone(), sel, st["eigvecs"])
         rot.div_((st["corrected"] / self.bc2_shampoo).pow_(1 / st["roots"][0]).add_(cfg.epsilon))

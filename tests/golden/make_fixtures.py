@@ -43,10 +43,12 @@ from distributed_shampoo import (  # noqa: E402
     DefaultSOAPConfig,
     DistributedShampoo,
     EigenConfig,
+    EigendecomposedKLShampooPreconditionerConfig,
     EigendecomposedShampooPreconditionerConfig,
     EigenvalueCorrectedShampooPreconditionerConfig,
     EighEigendecompositionConfig,
     QREigendecompositionConfig,
+    RootInvKLShampooPreconditionerConfig,
     RootInvShampooPreconditionerConfig,
     WeightDecayType,
 )
@@ -170,6 +172,25 @@ CASES = {
         max_preconditioner_dim=16, precondition_frequency=1, start_preconditioning_step=5,
         preconditioner="eigendecomposed_qr", override_1d=True, grafting="adagrad", grafting_epsilon=1e-8,
     ),
+    "kl_rootinv_eigh": dict(  # RootInvKLShampooPreconditionerConfig, default eigh root inverse
+        shapes=[[24, 20], [20]], seed=16, grad_scale=1.0, steps=8,
+        lr=1e-2, betas=[0.9, 0.99], epsilon=1e-6, weight_decay=0.0, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=16, precondition_frequency=1, start_preconditioning_step=5,
+        preconditioner="eigh", kl=True, override_1d=True, grafting="adam", grafting_beta2=0.99, grafting_epsilon=1e-8,
+    ),
+    "kl_rootinv_newton": dict(  # the same with the coupled Newton iteration, amortized every second step
+        shapes=[[24, 20], [20]], seed=17, grad_scale=1.0, steps=9,
+        lr=1e-2, betas=[0.9, 0.99], epsilon=1e-6, weight_decay=0.0, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=16, precondition_frequency=2, start_preconditioning_step=5,
+        preconditioner="newton", kl=True, override_1d=True, grafting="adagrad", grafting_epsilon=1e-8,
+    ),
+    "kl_eigendecomposed_eigh": dict(  # EigendecomposedKLShampooPreconditionerConfig
+        shapes=[[24, 20], [20]], seed=18, grad_scale=1.0, steps=8,
+        lr=1e-2, betas=[0.9, 0.99], epsilon=1e-6, weight_decay=0.0, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=16, precondition_frequency=1, start_preconditioning_step=5,
+        preconditioner="eigendecomposed_eigh", kl=True, override_1d=True, grafting="adam", grafting_beta2=0.99,
+        grafting_epsilon=1e-8,
+    ),
     "cfg1_override": dict(  # benchmark configuration 1 with 1-D blocks left to grafting
         shapes=[[512, 512], [512]], seed=0, grad_scale=1.0, steps=10, zero_init=True, torch_seed_grads=True,
         lr=1e-3, betas=[0.9, 0.999], epsilon=1e-12, weight_decay=0.0, weight_decay_type="DECOUPLED",
@@ -183,20 +204,22 @@ def build_reference(c, params):
     trace = dict(
         use_trace_scaling=c.get("use_trace_scaling", False), trace_scaling_exponent=c.get("trace_scaling_exponent", 0.5)
     )
+    RootInv = RootInvKLShampooPreconditionerConfig if c.get("kl") else RootInvShampooPreconditionerConfig
+    Eigendecomposed = EigendecomposedKLShampooPreconditionerConfig if c.get("kl") else EigendecomposedShampooPreconditionerConfig
     if c["preconditioner"] == "newton":
-        pc = RootInvShampooPreconditionerConfig(
+        pc = RootInv(
             amortized_computation_config=CoupledNewtonConfig(),
             inverse_exponent_override={1: {0: 0.0}} if c["override_1d"] else {}, **trace,
         )
     elif c["preconditioner"] == "higher_order":
-        pc = RootInvShampooPreconditionerConfig(
+        pc = RootInv(
             amortized_computation_config=CoupledHigherOrderConfig(
                 rel_epsilon=c["ho_rel_epsilon"], abs_epsilon=c["ho_abs_epsilon"], order=c["ho_order"]
             ),
             inverse_exponent_override={1: {0: 0.0}} if c["override_1d"] else {}, **trace,
         )
     elif c["preconditioner"] == "eigh":
-        pc = RootInvShampooPreconditionerConfig(
+        pc = RootInv(
             amortized_computation_config=EigenConfig(),
             inverse_exponent_override={1: {0: 0.0}} if c["override_1d"] else {}, **trace,
         )
@@ -208,7 +231,7 @@ def build_reference(c, params):
     elif c["preconditioner"] == "soap_eigh":
         pc = EigenvalueCorrectedShampooPreconditionerConfig()
     elif c["preconditioner"] in ("eigendecomposed_eigh", "eigendecomposed_qr"):
-        pc = EigendecomposedShampooPreconditionerConfig(
+        pc = Eigendecomposed(
             amortized_computation_config=(
                 QREigendecompositionConfig() if c["preconditioner"].endswith("qr") else EighEigendecompositionConfig()
             ),

@@ -11,12 +11,18 @@ import torch
 
 pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda:0")
-SOLVERS = ("eigh", "newton", "higher_order", "eigendecomposed_eigh", "eigendecomposed_qr")
+SOLVERS = ("eigh", "newton", "higher_order", "eigendecomposed_eigh", "eigendecomposed_qr", "kl_eigh", "kl_eigendecomposed_qr")
 
 
 def _config(solver):
     import optimizers_amd as oa
 
+    if solver.startswith("kl_"):
+        # RootInvKLShampooPreconditionerListTest / EigendecomposedKLShampooPreconditionerListTest (:1514-1554) inherit the
+        # abstract tests: the inverse roots are the identity until the one amortized computation at the last step
+        base = _config(solver[3:])
+        kl = oa.EigendecomposedKLShampooPreconditionerConfig if "eigendecomposed" in solver else oa.RootInvKLShampooPreconditionerConfig
+        return kl(amortized_computation_config=base.amortized_computation_config)
     if solver.startswith("eigendecomposed"):
         # EigendecomposedShampooPreconditionerList: the same abstract tests apply (shampoo_preconditioner_list_test.py:1185-1262)
         acc = oa.QREigendecompositionConfig() if solver.endswith("qr") else oa.EighEigendecompositionConfig()
@@ -58,8 +64,16 @@ class Harness:
         import optimizers_amd as oa
         from optimizers_amd.preconditioner_list import EigendecomposedShampooPreconditionerList, RootInvShampooPreconditionerList
 
-        if factory is None and isinstance(kwargs.get("preconditioner_config"), oa.EigendecomposedShampooPreconditionerConfig):
-            factory = EigendecomposedShampooPreconditionerList
+        from optimizers_amd.preconditioner_list import EigendecomposedKLShampooPreconditionerList, RootInvKLShampooPreconditionerList
+
+        cfg = kwargs.get("preconditioner_config")
+        if factory is None:
+            for cls, lst in ((oa.EigendecomposedKLShampooPreconditionerConfig, EigendecomposedKLShampooPreconditionerList),
+                             (oa.RootInvKLShampooPreconditionerConfig, RootInvKLShampooPreconditionerList),
+                             (oa.EigendecomposedShampooPreconditionerConfig, EigendecomposedShampooPreconditionerList)):
+                if isinstance(cfg, cls):
+                    factory = lst
+                    break
         return (factory or RootInvShampooPreconditionerList)(
             block_list=self.block_list, state=self.state, block_info_list=self.block_info_list, **kwargs)
 

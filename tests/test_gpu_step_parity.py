@@ -18,6 +18,7 @@ CASES = load_cases()
 NEWTON_CASES = [
     n for n, c in CASES.items()
     if c["preconditioner"] in ("newton", "higher_order") or c.get("use_trace_scaling") or (n.startswith("conv_like") and "soap" not in n)
+    or n == "kl_rootinv_eigh"
 ]
 
 
@@ -25,7 +26,7 @@ def native_optimizer(c, params):
     import optimizers_amd as oa
 
     if c["preconditioner"].startswith("eigendecomposed"):
-        pc = oa.EigendecomposedShampooPreconditionerConfig(
+        pc = (oa.EigendecomposedKLShampooPreconditionerConfig if c.get("kl") else oa.EigendecomposedShampooPreconditionerConfig)(
             amortized_computation_config=(
                 oa.QREigendecompositionConfig() if c["preconditioner"].endswith("qr") else oa.EighEigendecompositionConfig()
             ),
@@ -58,7 +59,7 @@ def _root_inverse_config(oa, c):
             rel_epsilon=c.get("ho_rel_epsilon", 0.0), abs_epsilon=c.get("ho_abs_epsilon", 0.0), order=c.get("ho_order", 3)
         ),
     }[c["preconditioner"]]
-    return oa.RootInvShampooPreconditionerConfig(
+    return (oa.RootInvKLShampooPreconditionerConfig if c.get("kl") else oa.RootInvShampooPreconditionerConfig)(
         amortized_computation_config=solver,
         inverse_exponent_override={1: {0: 0.0}} if c.get("override_1d") else {},
         use_trace_scaling=c.get("use_trace_scaling", False), trace_scaling_exponent=c.get("trace_scaling_exponent", 0.5),
@@ -203,7 +204,7 @@ def test_twenty_steps_at_moderate_size(kind):
             assert rel_err(st["shampoo"]["inv_factor_matrices"][j].cpu(), f) < 1e-3, (k, j)
 
 
-@pytest.mark.parametrize("name", ["eigendecomposed_eigh", "eigendecomposed_qr"])
+@pytest.mark.parametrize("name", ["eigendecomposed_eigh", "eigendecomposed_qr", "kl_eigendecomposed_eigh"])
 def test_eigendecomposed_shampoo_matches_oracle_and_reference_fixture(name):
     """EigendecomposedShampooPreconditionerConfig: the state keeps (Q, lambda) of every factor; parameters within
     1e-3 of the fixture written by the reference, eigenvalues within 1e-3, eigenvectors up to the sign of a column
