@@ -143,6 +143,30 @@ int32_t sa_compute_root_inverses_newton(sa_plan* plan, float bias_correction2, f
                                         int32_t max_iterations, float tolerance,
                                         int32_t* iterations_out, int32_t* status_out, void* stream);
 
+/* Factor matrices in fp64 (`factor_matrix_dtype=torch.float64`, shampoo_types.py:184 of the reference): with 64,
+ * every `factor[]` pointer of the plan's descriptors addresses a packed triangle of doubles, the Gram matrices (fp32
+ * products, like the reference's tensordot of fp32 gradients) are averaged in double, and the root inverse runs in
+ * double precision; `inv_factor[]` stays fp32 (`inv_factor_matrix_dtype`).  Root-inverse Shampoo only.  Must be
+ * called before sa_plan_workspace_bytes / sa_plan_bind_workspace (the Newton scratch doubles). */
+int32_t sa_plan_set_factor_dtype(sa_plan* plan, int32_t bits);
+
+/* sa_update_factor_matrices for an fp64 plan: L <- beta2 L + w G G^T with beta2 and w in double, as
+ * `factor.mul_(beta2)`, `factor.add_(outer_product, alpha=w)` act on a float64 factor
+ * (shampoo_preconditioner_list.py:1524-1539). */
+int32_t sa_update_factor_matrices_f64(sa_plan* plan, double beta2, double weighting_factor, void* stream);
+
+/* sa_compute_root_inverses_newton for an fp64 plan: the coupled Newton iteration of matrix_functions.py:368-437 on
+ * A = unpack(factor / bias_correction2) + epsilon I in double precision (fp64 MFMA GEMMs), the result cast to the fp32
+ * inverse-root state (shampoo_preconditioner_list.py:672-678).  bias_correction2 is the reference's fp32 scalar, widened
+ * exactly.  iterations_out / status_out as in the fp32 call.  widen_ridge_on_failure = 0 is the reference's CoupledNewtonConfig
+ * on a float64 factor.  With 1 the call stands in for the reference's float64 eigendecomposition root inverse
+ * (EigenConfig, matrix_functions.py:306-366): a factor on which the iteration does not converge (not positive
+ * definite above epsilon) is solved again with the ridge epsilon + 2^-21 ||A||_F, where the eigendecomposition would
+ * shift the spectrum by its smallest eigenvalue. */
+int32_t sa_compute_root_inverses_newton_f64(sa_plan* plan, float bias_correction2, double epsilon, int32_t max_iterations,
+                                            double tolerance, int32_t widen_ridge_on_failure, int32_t* iterations_out,
+                                            int32_t* status_out, void* stream);
+
 /* Batched coupled higher-order iteration on every factor (CoupledHigherOrderConfig; matrix_functions.py:439-661 via
  * :682-689): A = unpack(factor / bias_correction2), A_r = A + max(rel_epsilon * |A|_inf, abs_epsilon) I,
  * z = 1 / trace(A_r); one plain Newton step, then steps with M_p = sum_{i < order} b_i (I - M)^i until the error

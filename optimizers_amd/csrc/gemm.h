@@ -45,6 +45,7 @@ enum Epilogue {
   EPI_DIVPOW = 5,       // C = acc / ((C2 / div)^pow_exp + eps)   (C2 has the layout of C)
   EPI_SUB = 6,          // C -= acc                         (block-reflector updates of the QR refresh)
   EPI_HORNER = 7,       // C = alpha*acc + beta*C2 + mp_diag*I over d x d (C2 read only; Horner step of a matrix polynomial)
+  EPI_SYRK_EMA64 = 8,   // EPI_SYRK_EMA on a packed triangle of doubles: C = beta64*C + alpha64*acc (fp32 product, fp64 average)
 };
 
 struct GemmProblem {
@@ -68,6 +69,7 @@ struct GemmScalars {
   float alpha, beta;       // EPI_SYRK_EMA: C = beta*C + alpha*acc.  EPI_HORNER: C = alpha*acc + beta*C2 + mp_diag*I
   float mp_scale, mp_diag; // EPI_NEWTON_M: M_p = M*mp_scale + mp_diag*I
   float div, pow_exp, eps; // EPI_DIVPOW
+  double alpha64, beta64;  // EPI_SYRK_EMA64
 };
 
 __device__ __forceinline__ float4 load4_guarded(const float* p, bool vec, int valid) {
@@ -154,7 +156,7 @@ __device__ __forceinline__ float wave_max_nan(float v) {
 // same matrix).  Only tiles on or above the diagonal are computed; everything above the diagonal is stored
 // twice, as computed and transposed, which halves the MFMA work of a square product and leaves an exactly
 // mirrored matrix (so a later product may read it through its transpose).
-template <int AL, int BL, int EPI, bool EDGE, bool TRI = (EPI == EPI_SYRK_EMA)>
+template <int AL, int BL, int EPI, bool EDGE, bool TRI = (EPI == EPI_SYRK_EMA || EPI == EPI_SYRK_EMA64)>
 __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(
     const GemmProblem* __restrict__ problems, int n_problems, int total_tiles, GemmScalars sc) {
   __shared__ __attribute__((aligned(16))) float As[2][BK * LDS_STRIDE];
@@ -317,6 +319,13 @@ __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(
             const long long off = (long long)row * N - ((long long)row * (row - 1)) / 2 + (col - row);
             const float old = C[off];
             C[off] = __fadd_rn(__fmul_rn(old, sc.beta), __fmul_rn(v, sc.alpha));
+          }
+        } else if (EPI == EPI_SYRK_EMA64) {
+          // the factor matrix is kept in fp64: the fp32 Gram matrix entry is widened, then averaged in double
+          if (row < M && col < N && col >= row) {
+            const long long off = (long long)row * N - ((long long)row * (row - 1)) / 2 + (col - row);
+            double* C64 = reinterpret_cast<double*>(C);
+            C64[off] = C64[off] * sc.beta64 + (double)v * sc.alpha64;
           }
         } else if (EPI == EPI_SQ_EMA) {
           if (!EDGE || (row < M && col < N)) {

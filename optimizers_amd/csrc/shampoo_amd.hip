@@ -16,6 +16,7 @@
 #include "eigh.h"
 #include "elementwise.h"
 #include "gemm.h"
+#include "gemm64.h"
 #include "qr.h"
 #include "tridiag.h"
 
@@ -130,7 +131,7 @@ struct GemmTable {
 
 inline int vec_ok(const void* p, long long ld) { return ((reinterpret_cast<uintptr_t>(p) & 15) == 0 && (ld % 4) == 0) ? 1 : 0; }
 
-template <int AL, int BL, int EPI, bool EDGE, bool TRI = (EPI == EPI_SYRK_EMA)>
+template <int AL, int BL, int EPI, bool EDGE, bool TRI = (EPI == EPI_SYRK_EMA || EPI == EPI_SYRK_EMA64)>
 int launch_gemm(const GemmTable& g, GemmScalars sc, hipStream_t s) {
   if (g.total_tiles == 0) return SA_OK;
   const int per = (g.total_tiles + NUM_XCD - 1) / NUM_XCD;
@@ -154,7 +155,7 @@ int launch_gemm_auto(const GemmTable& g, GemmScalars sc, hipStream_t s) {
   return g.aligned ? launch_gemm<AL, BL, EPI, false>(g, sc, s) : launch_gemm<AL, BL, EPI, true>(g, sc, s);
 }
 
-GemmScalars unit_scalars() { return GemmScalars{1.0f, 1.0f, 1.0f, 0.0f, 0.0f, 0.0f, 1.0f, 1.0f, 0.0f}; }
+GemmScalars unit_scalars() { return GemmScalars{1.0f, 1.0f, 1.0f, 0.0f, 0.0f, 0.0f, 1.0f, 1.0f, 0.0f, 1.0, 0.0}; }
 
 // ---- phase timing -------------------------------------------------------------------------
 struct Phase {
@@ -239,6 +240,24 @@ struct sa_plan {
   Table<ChunkRef> t_chunks;
   Table<int> t_active_blocks;
   GemmTable syrk0, syrk1, g1_store, g1_norm, g2_norm, g2g_norm;
+  // factor matrices kept in fp64 (factor_matrix_dtype = float64): fp64 averages in the SYRK epilogue, fp64 coupled
+  // Newton root inverse on a scratch region twice the size; the inverse roots stay fp32
+  bool factor_f64 = false;
+  Table<Factor64> t_f64;
+  double* d_norm64 = nullptr;  // one squared norm per factor
+  struct GemmTable64 {
+    Table<GemmProblem64> t;
+    int total_tiles = 0;
+    std::vector<GemmProblem64> build;
+    void clear() { build.clear(); total_tiles = 0; }
+    void add(GemmProblem64 q) {
+      q.tiles = q.n / BM64;
+      q.tile_begin = total_tiles;
+      total_tiles += q.tiles * q.tiles;
+      build.push_back(q);
+    }
+  };
+  GemmTable64 n64_a[2], n64_pow[8], n64_m[2];
   // KL-Shampoo: the Gram matrices of a two-sided block are taken of the gradient preconditioned along the other dim
   bool kl = false;
   GemmTable kl_right, kl_left;  // G X_R -> T buffer, X_L G -> P buffer
@@ -318,7 +337,7 @@ void compute_layout(sa_plan* p) {
   p->off_ghat_partial = take(p->total_chunks_all);
   p->off_ptile_partial = take(p->total_ptiles_all);
   p->off_norm_partial = take(p->norm_partials_total);
-  p->scratch_floats = std::max(8LL * p->dense_total, 4LL * round_up(p->total_elems, 64) + 256);
+  p->scratch_floats = std::max((p->factor_f64 ? 16LL : 8LL) * p->dense_total, 4LL * round_up(p->total_elems, 64) + 256);
   p->off_scratch = take(p->scratch_floats);
   p->ws_needed = o * (long long)sizeof(float);
 }
@@ -805,6 +824,16 @@ static int launch_e3_chain(sa_plan* p, int chain, const GemmScalars& mid, const 
   return SA_OK;
 }
 
+template <int EPI>
+static int launch_gemm64(sa_plan::GemmTable64& g, double mp_scale, double mp_diag, hipStream_t s) {
+  if (g.total_tiles == 0) return SA_OK;
+  const int per = (g.total_tiles + NUM_XCD - 1) / NUM_XCD;
+  hipLaunchKernelGGL((grouped_gemm64_kernel<EPI>), dim3(per * NUM_XCD), dim3(GEMM_THREADS), 0, s, g.t.dev, (int)g.t.n,
+                     g.total_tiles, mp_scale, mp_diag);
+  HIPCHECK(hipGetLastError());
+  return SA_OK;
+}
+
 extern "C" {
 
 const char* sa_last_error(void) { return g_err.c_str(); }
@@ -994,6 +1023,10 @@ void sa_plan_destroy(sa_plan* p) {
   for (auto& g : p->nt_h) g.t.destroy();
   for (auto& a : p->g3) for (auto& b2 : a) for (auto& g : b2) g.t.destroy();
   for (auto& a : p->e3) for (auto& b2 : a) for (auto& c2 : b2) for (auto& g : c2) g.t.destroy();
+  p->t_f64.destroy();
+  for (auto* g : {&p->n64_a[0], &p->n64_a[1], &p->n64_m[0], &p->n64_m[1]}) g->t.destroy();
+  for (auto& g : p->n64_pow) g.t.destroy();
+  if (p->d_norm64) (void)hipFree(p->d_norm64);
   p->t_ho.destroy();
   p->t_sym.destroy(); p->t_normjobs.destroy(); p->t_ids.destroy();
   p->t_jacobi.destroy(); p->t_sched.destroy(); p->t_eiginit.destroy(); p->t_eigfinal.destroy(); p->eig_gemm.t.destroy();
@@ -1056,13 +1089,27 @@ int32_t sa_add_l2_regularization(sa_plan* p, float weight_decay, void* stream) {
   return SA_OK;
 }
 
+static int update_factor_matrices(sa_plan* p, double beta2, double weighting_factor, hipStream_t s);
+
 int32_t sa_update_factor_matrices(sa_plan* p, float beta2, float weighting_factor, void* stream) {
   if (!p) return fail(SA_ERR_INVALID, "NULL plan");
-  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (p->factor_f64) return fail(SA_ERR_STATE, "the factor matrices of this plan are fp64: use sa_update_factor_matrices_f64");
+  return update_factor_matrices(p, beta2, weighting_factor, static_cast<hipStream_t>(stream));
+}
+
+int32_t sa_update_factor_matrices_f64(sa_plan* p, double beta2, double weighting_factor, void* stream) {
+  if (!p) return fail(SA_ERR_INVALID, "NULL plan");
+  if (!p->factor_f64) return fail(SA_ERR_STATE, "the factor matrices of this plan are fp32: use sa_update_factor_matrices");
+  return update_factor_matrices(p, beta2, weighting_factor, static_cast<hipStream_t>(stream));
+}
+
+static int update_factor_matrices(sa_plan* p, double beta2, double weighting_factor, hipStream_t s) {
   SACHECK(ensure_tables(p, nullptr, s));
   GemmScalars sc = unit_scalars();
-  sc.alpha = weighting_factor;
-  sc.beta = beta2;
+  sc.alpha = (float)weighting_factor;
+  sc.beta = (float)beta2;
+  sc.alpha64 = weighting_factor;
+  sc.beta64 = beta2;
   double flops = 0.0;
   for (const GemmTable* g : {&p->syrk0, &p->syrk1})
     for (const GemmProblem& q : g->build) flops += (double)q.N * q.N * q.K;  // symmetric half: d^2 k
@@ -1077,8 +1124,13 @@ int32_t sa_update_factor_matrices(sa_plan* p, float beta2, float weighting_facto
     SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE>(p->kl_left, unit_scalars(), s)));
   }
   Span span("syrk", s, flops, launches, true);
-  SACHECK((launch_gemm_auto<A_MK, B_NK, EPI_SYRK_EMA>(p->syrk0, sc, s)));
-  SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_SYRK_EMA>(p->syrk1, sc, s)));
+  if (p->factor_f64) {
+    SACHECK((launch_gemm_auto<A_MK, B_NK, EPI_SYRK_EMA64>(p->syrk0, sc, s)));
+    SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_SYRK_EMA64>(p->syrk1, sc, s)));
+  } else {
+    SACHECK((launch_gemm_auto<A_MK, B_NK, EPI_SYRK_EMA>(p->syrk0, sc, s)));
+    SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_SYRK_EMA>(p->syrk1, sc, s)));
+  }
   return SA_OK;
 }
 
@@ -1576,6 +1628,270 @@ int32_t sa_compute_root_inverses_newton(sa_plan* p, float bias_correction2, floa
     const int fi = todo[i];
     iterations_out[fi] = iters[fi];
     if (i < ok) status_out[fi] = (errs[fi] <= tolerance) ? SA_FACTOR_OK : SA_FACTOR_NOT_CONVERGED;
+  }
+  return SA_OK;
+}
+
+// --------------------------------------------------------------------------------------------
+// Factor matrices in fp64: coupled Newton in double precision (reference: the same matrix_inverse_root_newton,
+// matrix_functions.py:368-437, on a torch.float64 factor; the result is cast to the fp32 inverse-root state,
+// shampoo_preconditioner_list.py:672-678)
+// --------------------------------------------------------------------------------------------
+
+int32_t sa_plan_set_factor_dtype(sa_plan* p, int32_t bits) {
+  if (!p) return fail(SA_ERR_INVALID, "NULL plan");
+  if (bits != 32 && bits != 64) return fail(SA_ERR_INVALID, "factor dtype must be 32 or 64 bits");
+  if (p->ws) return fail(SA_ERR_STATE, "sa_plan_set_factor_dtype must be called before the workspace is bound");
+  if (bits == 64) {
+    if (p->has_eigvec) return fail(SA_ERR_UNSUPPORTED, "fp64 factor matrices are built for root-inverse Shampoo only");
+    for (const Factor& f : p->factors)
+      if (!f.inv) return fail(SA_ERR_STATE, "fp64 factor matrices need inverse-root storage");
+    if (!p->d_norm64 && !p->factors.empty())
+      HIPCHECK(hipMalloc(reinterpret_cast<void**>(&p->d_norm64), p->factors.size() * sizeof(double)));
+  }
+  p->factor_f64 = bits == 64;
+  compute_layout(p);
+  return SA_OK;
+}
+
+static inline double* newton_buf64(const sa_plan* p, int k, const Factor& F) {
+  return reinterpret_cast<double*>(p->f(p->off_scratch)) + (long long)k * p->dense_total + F.dense_off;
+}
+
+static int commit64(sa_plan::GemmTable64& g, hipStream_t s) {
+  SACHECK(g.t.begin(g.build.size()));
+  if (!g.build.empty()) std::memcpy(g.t.host, g.build.data(), g.build.size() * sizeof(GemmProblem64));
+  return g.t.upload(s);
+}
+
+static int newton_batch64(sa_plan* p, const std::vector<int>& ids, int root, const std::vector<double>& ridge, double bc2,
+                          int max_iter, float tol, hipStream_t s) {
+  const int n = (int)ids.size();
+  if (n == 0) return SA_OK;
+  std::vector<char> ops;
+  SACHECK(power_ops(root, &ops));
+  const double alpha = -1.0 / root, one_minus_alpha = 1.0 - alpha;
+  SACHECK(p->t_ids.begin(n));
+  std::memcpy(p->t_ids.host, ids.data(), n * sizeof(int));
+  SACHECK(p->t_ids.upload(s));
+  SACHECK(p->t_f64.begin(n));
+  int nmax = 0;
+  for (int i = 0; i < n; ++i) {
+    const Factor& f = p->factors[ids[i]];
+    Factor64& J = p->t_f64.host[i];
+    std::memset(&J, 0, sizeof(J));
+    J.packed = reinterpret_cast<const double*>(f.factor);
+    J.M = newton_buf64(p, NB_M0, f); J.Mp = newton_buf64(p, NB_MP0, f); J.X = newton_buf64(p, NB_X0, f);
+    J.norm_sq = p->d_norm64 + ids[i];
+    J.nonfinite = p->d_flags + ids[i];
+    J.ridge = ridge[ids[i]];
+    J.d = f.d; J.n = f.dpad;
+    nmax = std::max(nmax, f.dpad);
+  }
+  SACHECK(p->t_f64.upload(s));
+  const unsigned gx = (unsigned)std::min<long long>(((long long)nmax * nmax + 255) / 256, 2048);
+  hipLaunchKernelGGL(f64_newton_start_kernel, dim3(gx, n), dim3(256), 0, s, p->t_f64.dev, bc2, root, alpha, one_minus_alpha);
+  HIPCHECK(hipGetLastError());
+
+  for (int par = 0; par < 2; ++par) { p->n64_a[par].clear(); p->n64_m[par].clear(); }
+  for (auto& g : p->n64_pow) g.clear();
+  auto prob = [&](const Factor& f, const double* A, const double* B, double* C) {
+    GemmProblem64 q{};
+    q.A = A; q.B = B; q.C = C;
+    q.n = f.dpad; q.d = f.d;
+    q.active = p->d_active + (&f - p->factors.data());
+    return q;
+  };
+  for (int i = 0; i < n; ++i) {
+    const Factor& f = p->factors[ids[i]];
+    for (int par = 0; par < 2; ++par) {
+      const double* X = newton_buf64(p, par ? NB_X1 : NB_X0, f);
+      double* Xn = newton_buf64(p, par ? NB_X0 : NB_X1, f);
+      const double* Mp = newton_buf64(p, par ? NB_MP1 : NB_MP0, f);
+      double* Mpn = newton_buf64(p, par ? NB_MP0 : NB_MP1, f);
+      const double* M = newton_buf64(p, par ? NB_M1 : NB_M0, f);
+      double* Mn = newton_buf64(p, par ? NB_M0 : NB_M1, f);
+      double* S1 = newton_buf64(p, NB_S1, f);
+      double* S2 = newton_buf64(p, NB_S2, f);
+      p->n64_a[par].add(prob(f, X, Mp, Xn));
+      if (!ops.empty()) p->n64_a[par].add(prob(f, Mp, Mp, S1));
+      const double* cur = ops.empty() ? Mp : S1;
+      int slot = par * 4;
+      double* pong[2] = {S2, S1};
+      int which = 0;
+      for (size_t q = 1; q < ops.size(); ++q) {
+        p->n64_pow[slot++].add(prob(f, cur, ops[q] == 'S' ? cur : Mp, pong[which]));
+        cur = pong[which];
+        which ^= 1;
+      }
+      GemmProblem64 m = prob(f, cur, M, Mn);
+      m.C2 = Mpn;
+      m.err_bits = p->d_err + ids[i];
+      p->n64_m[par].add(m);
+    }
+  }
+  for (int par = 0; par < 2; ++par) { SACHECK(commit64(p->n64_a[par], s)); SACHECK(commit64(p->n64_m[par], s)); }
+  for (auto& g : p->n64_pow) SACHECK(commit64(g, s));
+
+  // the start error is 1 (M = z A is far from I): one control pass with err = +inf activates every factor
+  NewtonCtl ctl{p->d_err, p->d_active, p->d_iters, p->d_final_parity, p->d_final_err};
+  int parity = 0;
+  const int Fall = (int)p->factors.size();
+  {
+    std::vector<unsigned int> inf_bits(Fall, 0x7f800000u);
+    HIPCHECK(hipMemcpyAsync(p->d_err, inf_bits.data(), Fall * sizeof(unsigned int), hipMemcpyHostToDevice, s));
+    HIPCHECK(hipStreamSynchronize(s));
+  }
+  hipLaunchKernelGGL(newton_control_kernel, dim3(1), dim3(256), 0, s, ctl, p->t_ids.dev, n, tol, max_iter, parity, p->d_nactive);
+  HIPCHECK(hipGetLastError());
+  int* h_active = p->h_pinned;
+  HIPCHECK(hipMemcpyAsync(h_active, p->d_active, Fall * sizeof(int), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipStreamSynchronize(s));
+  for (int it = 0; it < max_iter; ++it) {
+    int live = 0;
+    double flops = 0.0;
+    for (int i = 0; i < n; ++i)
+      if (h_active[ids[i]]) { ++live; const double d = p->factors[ids[i]].d; flops += 2.0 * d * d * d * (2.0 + ops.size()); }
+    if (!live) break;
+    {
+      Span span("newton_gemm_f64", s, flops, 2 + (int)ops.size() - 1, it == 0);
+      SACHECK(launch_gemm64<EPI64_STORE>(p->n64_a[parity], 0.0, 0.0, s));
+      for (int k = 0; k < 4; ++k) SACHECK(launch_gemm64<EPI64_STORE>(p->n64_pow[parity * 4 + k], 0.0, 0.0, s));
+      SACHECK(launch_gemm64<EPI64_NEWTON_M>(p->n64_m[parity], alpha, one_minus_alpha, s));
+    }
+    parity ^= 1;
+    hipLaunchKernelGGL(newton_control_kernel, dim3(1), dim3(256), 0, s, ctl, p->t_ids.dev, n, tol, max_iter, parity, p->d_nactive);
+    HIPCHECK(hipGetLastError());
+    HIPCHECK(hipMemcpyAsync(h_active, p->d_active, Fall * sizeof(int), hipMemcpyDeviceToHost, s));
+    HIPCHECK(hipStreamSynchronize(s));
+  }
+  return SA_OK;
+}
+
+int32_t sa_compute_root_inverses_newton_f64(sa_plan* p, float bias_correction2, double epsilon, int32_t max_iterations,
+                                            double tolerance, int32_t widen_ridge_on_failure, int32_t* iterations_out,
+                                            int32_t* status_out, void* stream) {
+  if (!p || !iterations_out || !status_out) return fail(SA_ERR_INVALID, "sa_compute_root_inverses_newton_f64: NULL argument");
+  if (!p->factor_f64) return fail(SA_ERR_STATE, "the factor matrices of this plan are fp32");
+  if (!(bias_correction2 != 0.0f) || max_iterations < 0) return fail(SA_ERR_INVALID, "bad bias correction or max_iterations");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SACHECK(ensure_tables(p, nullptr, s));
+  const int F = (int)p->factors.size();
+  if (F == 0) return SA_OK;
+  std::vector<int> todo;
+  for (int i = 0; i < F; ++i) {
+    iterations_out[i] = 0;
+    status_out[i] = SA_FACTOR_SKIPPED;
+    if (block_active(p, p->factors[i].block)) todo.push_back(i);
+  }
+  if (todo.empty()) return SA_OK;
+  SACHECK(refresh_inverse_cache(p, s));  // factors that are not recomputed keep a valid dense copy
+  const double bc2 = (double)bias_correction2;
+  int* h_bad = p->h_pinned + 3 * F;
+  std::vector<double> ridge(F, epsilon);
+
+  auto jobs = [&](const std::vector<int>& ids) -> int {
+    SACHECK(p->t_f64.begin(ids.size()));
+    for (size_t i = 0; i < ids.size(); ++i) {
+      const Factor& f = p->factors[ids[i]];
+      Factor64& J = p->t_f64.host[i];
+      std::memset(&J, 0, sizeof(J));
+      J.packed = reinterpret_cast<const double*>(f.factor);
+      J.norm_sq = p->d_norm64 + ids[i];
+      J.nonfinite = p->d_flags + ids[i];
+      J.inv_packed = f.inv;
+      J.inv_dense = p->f(p->off_inv_dense) + f.dense_off;
+      J.ridge = ridge[ids[i]];
+      J.d = f.d; J.n = f.dpad;
+    }
+    return p->t_f64.upload(s);
+  };
+  // norm and finiteness of the bias-corrected factors; the reference raises at the first non-finite one
+  auto norms = [&](const std::vector<int>& ids) -> int {
+    SACHECK(jobs(ids));
+    hipLaunchKernelGGL(f64_norm_kernel, dim3((unsigned)ids.size()), dim3(256), 0, s, p->t_f64.dev, bc2);
+    HIPCHECK(hipGetLastError());
+    return SA_OK;
+  };
+  HIPCHECK(hipMemsetAsync(p->d_flags, 0, F * sizeof(int), s));
+  SACHECK(norms(todo));
+  HIPCHECK(hipMemcpyAsync(h_bad, p->d_flags, F * sizeof(int), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipStreamSynchronize(s));
+  for (size_t i = 0; i < todo.size(); ++i)
+    if (h_bad[todo[i]]) { status_out[todo[i]] = SA_FACTOR_INPUT_NONFINITE; todo.resize(i); break; }
+  if (todo.empty()) return SA_OK;
+
+  std::vector<int> par(F, 0);
+  std::vector<float> errs(F, 0.0f);
+  if (g_profiling) { Phase& ph = g_phases["newton_gemm_f64"]; ph.used = 0; ph.work = 0.0; ph.executed = 0.0; ph.launches = 0; }
+  auto solve = [&](const std::vector<int>& subset) -> int {
+    std::vector<int> ones(F, 0);
+    for (int i : subset) ones[i] = 1;
+    HIPCHECK(hipMemsetAsync(p->d_iters, 0, F * sizeof(int), s));
+    HIPCHECK(hipMemsetAsync(p->d_final_parity, 0, F * sizeof(int), s));
+    HIPCHECK(hipMemcpyAsync(p->d_active, ones.data(), F * sizeof(int), hipMemcpyHostToDevice, s));
+    HIPCHECK(hipStreamSynchronize(s));
+    std::map<int, std::vector<int>> by_root;
+    for (int i : subset) by_root[p->factors[i].root].push_back(i);
+    for (auto& kv : by_root)
+      SACHECK(newton_batch64(p, kv.second, kv.first, ridge, bc2, max_iterations, (float)tolerance, s));
+    HIPCHECK(hipMemcpyAsync(p->h_pinned, p->d_iters, F * sizeof(int), hipMemcpyDeviceToHost, s));
+    HIPCHECK(hipMemcpyAsync(p->h_pinned + F, p->d_final_parity, F * sizeof(int), hipMemcpyDeviceToHost, s));
+    HIPCHECK(hipMemcpyAsync(p->h_pinned + 2 * F, p->d_final_err, F * sizeof(float), hipMemcpyDeviceToHost, s));
+    HIPCHECK(hipStreamSynchronize(s));
+    for (int i : subset) {
+      iterations_out[i] = p->h_pinned[i];
+      par[i] = p->h_pinned[F + i];
+      std::memcpy(&errs[i], p->h_pinned + 2 * F + i, sizeof(float));
+    }
+    return SA_OK;
+  };
+  SACHECK(solve(todo));
+  if (widen_ridge_on_failure) {
+    // A factor that is not positive definite above epsilon (Gram matrices are fp32 products: a rank-deficient factor has
+    // eigenvalues of either sign of the order 1e-7 ||A||) makes the iteration diverge.  The eigendecomposition the
+    // caller stands in for shifts such a spectrum by its smallest eigenvalue; here the ridge grows to 2^-21 ||A||_F.
+    std::vector<int> redo;
+    for (int i : todo)
+      if (!(errs[i] <= (float)tolerance)) redo.push_back(i);
+    if (!redo.empty()) {
+      std::vector<double> norm_sq(F, 0.0);
+      HIPCHECK(hipMemcpy(norm_sq.data(), p->d_norm64, F * sizeof(double), hipMemcpyDeviceToHost));
+      for (int i : redo) ridge[i] = epsilon + std::ldexp(std::sqrt(norm_sq[i]), -21);
+      HIPCHECK(hipMemsetAsync(p->d_flags, 0, F * sizeof(int), s));
+      SACHECK(norms(redo));
+      SACHECK(solve(redo));
+    }
+  }
+
+  // finiteness of the fp32 results first; the factors that precede the first bad one are stored
+  auto run_commit = [&](const std::vector<int>& ids, int check_only) -> int {
+    SACHECK(jobs(ids));
+    int nmax = 0;
+    for (size_t i = 0; i < ids.size(); ++i) {
+      const Factor& f = p->factors[ids[i]];
+      p->t_f64.host[i].result = newton_buf64(p, par[ids[i]] ? NB_X1 : NB_X0, f);
+      nmax = std::max(nmax, f.dpad);
+    }
+    SACHECK(p->t_f64.upload(s));
+    const unsigned gx = (unsigned)std::min<long long>(((long long)nmax * nmax + 255) / 256, 2048);
+    hipLaunchKernelGGL(f64_commit_kernel, dim3(gx, (unsigned)ids.size()), dim3(256), 0, s, p->t_f64.dev, check_only);
+    HIPCHECK(hipGetLastError());
+    return SA_OK;
+  };
+  HIPCHECK(hipMemsetAsync(p->d_flags, 0, F * sizeof(int), s));
+  SACHECK(run_commit(todo, 1));
+  HIPCHECK(hipMemcpyAsync(h_bad, p->d_flags, F * sizeof(int), hipMemcpyDeviceToHost, s));
+  HIPCHECK(hipStreamSynchronize(s));
+  std::vector<int> good;
+  for (int i : todo) {
+    if (h_bad[i]) { status_out[i] = SA_FACTOR_RESULT_NONFINITE; break; }
+    good.push_back(i);
+    status_out[i] = (errs[i] <= (float)tolerance) ? SA_FACTOR_OK : SA_FACTOR_NOT_CONVERGED;
+  }
+  if (!good.empty()) {
+    SACHECK(run_commit(good, 0));
+    HIPCHECK(hipStreamSynchronize(s));
   }
   return SA_OK;
 }

@@ -90,16 +90,16 @@ def _round_up(x: int, a: int) -> int:
 
 
 class _Arena:
-    """One flat fp32 device buffer handing out aligned views (state tensors stay ordinary torch
+    """One flat device buffer (fp32 unless stated) handing out aligned views (state tensors stay ordinary torch
     tensors, so checkpoints see the same objects the kernels update)."""
 
-    def __init__(self, sizes: list[int], device: torch.device) -> None:
+    def __init__(self, sizes: list[int], device: torch.device, dtype: torch.dtype = torch.float32) -> None:
         self.offsets = []
         total = 0
         for n in sizes:
             self.offsets.append(total)
             total += _round_up(max(n, 1), _ALIGN)
-        self.buffer = torch.zeros(max(total, _ALIGN), dtype=torch.float32, device=device)
+        self.buffer = torch.zeros(max(total, _ALIGN), dtype=dtype, device=device)
 
     def view(self, i: int, shape: tuple[int, ...]) -> torch.Tensor:
         n = math.prod(shape)
@@ -117,7 +117,24 @@ class _AmortizedComputation:
         pc = self.preconditioner_config
         cfg = pc.amortized_computation_config
         refreshes_basis = self.soap or getattr(self, "eigendecomposed", False)
-        if refreshes_basis and isinstance(cfg, EighEigendecompositionConfig):
+        if getattr(self, "factor_f64", False):
+            # float64 factor matrices: the root inverse is the coupled Newton iteration in double precision.  With
+            # CoupledNewtonConfig that is the reference's own algorithm on a float64 matrix; with EigenConfig (the
+            # reference runs torch.linalg.eigh in float64) the same inverse root is reached by iterating to 1e-10, far
+            # below the fp32 resolution of the inverse-root state it is cast to.
+            if isinstance(cfg, CoupledNewtonConfig):
+                max_iterations, tolerance, widen = cfg.max_iterations, cfg.tolerance, 0
+            else:
+                # where the eigendecomposition would shift an indefinite spectrum by its smallest eigenvalue, the
+                # iteration is repeated with a ridge of 2^-21 ||A||_F
+                max_iterations, tolerance, widen = 100, 1e-10, 1
+            native.check(
+                self.lib.sa_compute_root_inverses_newton_f64(
+                    self.plan, bc2, group[EPSILON], max_iterations, tolerance, widen, self.iterations, self.status, stream
+                ),
+                "sa_compute_root_inverses_newton_f64",
+            )
+        elif refreshes_basis and isinstance(cfg, EighEigendecompositionConfig):
             # epsilon * I is added only when the config perturbs before the computation (matrix_functions.py:869-882)
             ridge = group[EPSILON] * float(cfg.rank_deficient_stability_config.perturb_before_computation)
             native.check(
@@ -332,7 +349,8 @@ class _NativeGroup(_AmortizedComputation):
             s = self.block_specs[i]
             fdims.extend(s.shape[d] for d in range(s.order) if self.selectors[k][d])
         packed = [d * (d + 1) // 2 for d in fdims]
-        self.factor_arena = _Arena(packed, self.device)
+        self.factor_f64 = pc.factor_matrix_dtype == torch.float64
+        self.factor_arena = _Arena(packed, self.device, pc.factor_matrix_dtype)
         self.inv_arena = _Arena(packed, self.device) if not self.soap else None
         self.eigvec_arena = _Arena([d * d for d in fdims], self.device) if (self.soap or self.eigendecomposed) else None
         self.eigenvalue_arena = _Arena(list(fdims), self.device) if self.eigendecomposed else None
@@ -415,7 +433,11 @@ class _NativeGroup(_AmortizedComputation):
                         self._slots.append((p, s.block_key, (SHAMPOO, "inv_factor_matrices", slot), inv))
                 root = Fraction(self.roots[k][slot])
                 self.factor_roots.append(float(self.roots[k][slot]))
-                if self.use_eigh or self.soap:
+                if self.factor_f64 and root.denominator != 1:
+                    raise NotImplementedError(
+                        f"factor_matrix_dtype=float64 with a fractional root ({root}) is not built natively"
+                    )
+                if (self.use_eigh or self.soap) and not self.factor_f64:
                     d.root[dim] = max(int(round(self.roots[k][slot])), 1)  # unused by the eigh path
                 elif root.denominator != 1 and self.use_higher_order:
                     raise NotImplementedError(
@@ -461,6 +483,8 @@ class _NativeGroup(_AmortizedComputation):
         self.workspace = None
         if nb:
             native.check(self.lib.sa_plan_create(descs, nb, ctypes.byref(self.plan)), "sa_plan_create")
+            if self.factor_f64:
+                native.check(self.lib.sa_plan_set_factor_dtype(self.plan, 64), "sa_plan_set_factor_dtype")
             need = int(self.lib.sa_plan_workspace_bytes(self.plan))
             self.workspace = torch.empty(need, dtype=torch.uint8, device=self.device)
             native.check(
@@ -553,8 +577,21 @@ class _NativeGroup(_AmortizedComputation):
             )
         if not pc.use_symmetric_packing:
             raise NotImplementedError("use_symmetric_packing=False: the native step keeps factors packed")
-        if pc.factor_matrix_dtype != torch.float32 or getattr(pc, "inv_factor_matrix_dtype", torch.float32) != torch.float32:
-            raise NotImplementedError("factor matrices are fp32 in the native step")
+        if getattr(pc, "inv_factor_matrix_dtype", torch.float32) != torch.float32:
+            raise NotImplementedError("inverse factor matrices are fp32 in the native step")
+        if pc.factor_matrix_dtype == torch.float64:
+            plain_root_inverse = type(pc) is RootInvShampooPreconditionerConfig and (
+                isinstance(acc, CoupledNewtonConfig)
+                or (isinstance(acc, EigenConfig) and isinstance(acc.rank_deficient_stability_config, PerturbationConfig)
+                    and acc.rank_deficient_stability_config.perturb_before_computation)
+            )
+            if not plain_root_inverse or pc.use_trace_scaling:
+                raise NotImplementedError(
+                    "factor_matrix_dtype=float64 is built for RootInvShampooPreconditionerConfig with CoupledNewtonConfig or "
+                    "EigenConfig (PerturbationConfig, perturb_before_computation=True), without trace scaling"
+                )
+        elif pc.factor_matrix_dtype != torch.float32:
+            raise NotImplementedError(f"factor matrices are fp32 or fp64 in the native step, got {pc.factor_matrix_dtype}")
         if group[ITERATE_AVERAGING_CONFIG] is not None and not isinstance(
             group[ITERATE_AVERAGING_CONFIG], ClassicMomentumConfig
         ):
@@ -653,7 +690,10 @@ class _NativeGroup(_AmortizedComputation):
             self.inverse_roots_stale = False
         drop = pc.drop_weighting_factor_on_gsquare
         weighting = 1.0 if (drop or beta2 == 1.0) else 1 - beta2
-        native.check(lib.sa_update_factor_matrices(self.plan, beta2, weighting, stream), "sa_update_factor_matrices")
+        if self.factor_f64:
+            native.check(lib.sa_update_factor_matrices_f64(self.plan, beta2, weighting, stream), "sa_update_factor_matrices_f64")
+        else:
+            native.check(lib.sa_update_factor_matrices(self.plan, beta2, weighting, stream), "sa_update_factor_matrices")
 
         # fp32 scalars evaluated with the very torch expressions the reference uses
         bc2 = 1.0
@@ -727,7 +767,8 @@ class DistributedShampoo(torch.optim.Optimizer):
     `EigenvalueCorrectedShampooPreconditionerConfig` and `EigendecomposedShampooPreconditionerConfig` with
     `QREigendecompositionConfig` or `EighEigendecompositionConfig` (including `ignored_basis_change_dims`), grafting with SGD / AdaGrad / RMSprop /
     Adam or none, every `WeightDecayType`, `ClassicMomentumConfig`, `inverse_exponent_override`,
-    `SingleDeviceDistributedConfig`, fp32 state with packed factor matrices, blocks of order 1 to 3 (order 3: what is left of
+    `SingleDeviceDistributedConfig`, fp32 state with packed factor matrices (`factor_matrix_dtype=torch.float64` for
+    root-inverse Shampoo: fp64 factor averages and an fp64 coupled Newton root inverse), blocks of order 1 to 3 (order 3: what is left of
     convolution weights).
     Anything else raises NotImplementedError at construction.
     """

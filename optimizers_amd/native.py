@@ -36,6 +36,7 @@ EXPORTS = (
     "sa_gemm_f32", "sa_copy_f32", "sa_set_profiling", "sa_phase_ms", "sa_phase_flops", "sa_phase_launches", "sa_phase_executed_flops", "sa_set_symmetric_newton", "sa_set_eigh_solver",
     "sa_plan_set_trace_scaling", "sa_compute_root_inverses_higher_order", "sa_plan_read_eigenvalues", "sa_add_to_views",
     "sa_compute_root_inverses_from_eigendecomposition", "sa_plan_set_kl_shampoo",
+    "sa_plan_set_factor_dtype", "sa_update_factor_matrices_f64", "sa_compute_root_inverses_newton_f64",
 )
 
 
@@ -160,6 +161,11 @@ def load() -> ctypes.CDLL:
         c_void_p, POINTER(c_void_p), c_float, POINTER(c_float), c_int32, c_float, c_float, POINTER(c_int32), c_void_p,
     ]
     lib.sa_plan_set_kl_shampoo.argtypes = [c_void_p, c_int32]
+    lib.sa_plan_set_factor_dtype.argtypes = [c_void_p, c_int32]
+    lib.sa_update_factor_matrices_f64.argtypes = [c_void_p, c_double, c_double, c_void_p]
+    lib.sa_compute_root_inverses_newton_f64.argtypes = [
+        c_void_p, c_float, c_double, c_int32, c_double, c_int32, POINTER(c_int32), POINTER(c_int32), c_void_p,
+    ]
     lib.sa_add_to_views.argtypes = [POINTER(View), POINTER(View), c_int32, c_void_p]
     lib.sa_set_profiling.argtypes = [c_int32]
     lib.sa_phase_ms.argtypes = [c_char_p]

@@ -389,6 +389,7 @@ class OracleConfig:
     use_nesterov: bool = False
     use_symmetric_packing: bool = True
     num_tolerated_failed_amortized_computations: int = 3
+    factor_matrix_dtype: str = "float32"  # "float64": factor matrices and their root inverse in double (shampoo_types.py:184)
     kl: bool = False  # RootInvKLShampooPreconditionerConfig / EigendecomposedKLShampooPreconditionerConfig
     use_trace_scaling: bool = False  # shampoo_types.py:187-188
     trace_scaling_exponent: float = 0.5
@@ -456,10 +457,11 @@ class ShampooOracle:
         st["selector"] = sel
         dims = [b.shape[d] for d in range(order) if sel[d]]
         st["dims"] = dims
+        fdt = torch.float64 if cfg.factor_matrix_dtype == "float64" else dt
         if cfg.use_symmetric_packing:
-            st["factors"] = [torch.zeros(d * (d + 1) // 2, dtype=dt, device=dev) for d in dims]
+            st["factors"] = [torch.zeros(d * (d + 1) // 2, dtype=fdt, device=dev) for d in dims]
         else:
-            st["factors"] = [torch.zeros(d, d, dtype=dt, device=dev) for d in dims]
+            st["factors"] = [torch.zeros(d, d, dtype=fdt, device=dev) for d in dims]
         if self.soap:
             st["eigvecs"] = [torch.eye(d, dtype=dt, device=dev) for d in dims]
             st["corrected"] = torch.zeros(b.shape, dtype=dt, device=dev)

@@ -191,6 +191,23 @@ CASES = {
         preconditioner="eigendecomposed_eigh", kl=True, override_1d=True, grafting="adam", grafting_beta2=0.99,
         grafting_epsilon=1e-8,
     ),
+    # factor_matrix_dtype=float64: factors averaged and inverted in double, inverse roots stored in fp32; epsilon small
+    # enough that fp32 factors would not resolve it; the first root inverse comes when every factor has full rank (the
+    # Gram matrices are fp32 products, so a rank-deficient factor is indefinite at the 1e-7 level and its root inverse
+    # is decided by rounding noise)
+    "f64_factors_eigh": dict(
+        shapes=[[24, 20], [20]], seed=19, grad_scale=1.0, steps=8,
+        lr=1e-2, betas=[0.9, 0.99], epsilon=1e-10, weight_decay=0.0, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=16, precondition_frequency=2, start_preconditioning_step=6,
+        preconditioner="eigh", factor_matrix_dtype="float64", override_1d=True, grafting="adam", grafting_beta2=0.99,
+        grafting_epsilon=1e-8,
+    ),
+    "f64_factors_newton": dict(
+        shapes=[[24, 20], [20]], seed=20, grad_scale=1.0, steps=8,
+        lr=1e-2, betas=[0.9, 0.99], epsilon=1e-10, weight_decay=0.0, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=16, precondition_frequency=2, start_preconditioning_step=4,
+        preconditioner="newton", factor_matrix_dtype="float64", override_1d=True, grafting="adagrad", grafting_epsilon=1e-8,
+    ),
     "cfg1_override": dict(  # benchmark configuration 1 with 1-D blocks left to grafting
         shapes=[[512, 512], [512]], seed=0, grad_scale=1.0, steps=10, zero_init=True, torch_seed_grads=True,
         lr=1e-3, betas=[0.9, 0.999], epsilon=1e-12, weight_decay=0.0, weight_decay_type="DECOUPLED",
@@ -204,6 +221,8 @@ def build_reference(c, params):
     trace = dict(
         use_trace_scaling=c.get("use_trace_scaling", False), trace_scaling_exponent=c.get("trace_scaling_exponent", 0.5)
     )
+    if c.get("factor_matrix_dtype") == "float64":
+        trace["factor_matrix_dtype"] = torch.float64
     RootInv = RootInvKLShampooPreconditionerConfig if c.get("kl") else RootInvShampooPreconditionerConfig
     Eigendecomposed = EigendecomposedKLShampooPreconditionerConfig if c.get("kl") else EigendecomposedShampooPreconditionerConfig
     if c["preconditioner"] == "newton":

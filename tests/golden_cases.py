@@ -66,7 +66,7 @@ def oracle_config(c):
         grafting_epsilon=c.get("grafting_epsilon", 1e-10),
         momentum=c.get("momentum", 0.0), dampening=c.get("dampening", 0.0),
         use_nesterov=c.get("use_nesterov", False),
-        kl=c.get("kl", False),
+        kl=c.get("kl", False), factor_matrix_dtype=c.get("factor_matrix_dtype", "float32"),
         use_trace_scaling=c.get("use_trace_scaling", False),
         trace_scaling_exponent=c.get("trace_scaling_exponent", 0.5),
         higher_order=c.get("ho_order", 3), higher_order_rel_epsilon=c.get("ho_rel_epsilon", 0.0),

@@ -59,8 +59,9 @@ def _root_inverse_config(oa, c):
             rel_epsilon=c.get("ho_rel_epsilon", 0.0), abs_epsilon=c.get("ho_abs_epsilon", 0.0), order=c.get("ho_order", 3)
         ),
     }[c["preconditioner"]]
+    extra = {"factor_matrix_dtype": torch.float64} if c.get("factor_matrix_dtype") == "float64" else {}
     return (oa.RootInvKLShampooPreconditionerConfig if c.get("kl") else oa.RootInvShampooPreconditionerConfig)(
-        amortized_computation_config=solver,
+        amortized_computation_config=solver, **extra,
         inverse_exponent_override={1: {0: 0.0}} if c.get("override_1d") else {},
         use_trace_scaling=c.get("use_trace_scaling", False), trace_scaling_exponent=c.get("trace_scaling_exponent", 0.5),
     )
@@ -292,3 +293,89 @@ def test_eigendecomposed_qr_first_refreshes_match_the_oracle():
             got_q = st["factor_matrices_eigenvectors"][j].cpu()
             assert rel_err(got_lam, lam) < 1e-4, (k, j)
             assert float(((got_q.T @ q).abs() - torch.eye(q.shape[0])).abs().max()) < 1e-3, (k, j)
+
+
+@pytest.mark.parametrize("name", ["f64_factors_eigh", "f64_factors_newton"])
+def test_float64_factor_matrices_match_oracle_and_reference_fixture(name):
+    """factor_matrix_dtype=torch.float64: the state keeps float64 factor matrices (fp32 Gram matrices averaged in
+    double), the root inverse runs in double precision and lands in the fp32 inverse-root state.  Parameters within
+    1e-3 of the fixture written by the reference, factors within 1e-6, inverse roots within 1e-3."""
+    print(f"case {name}", flush=True)
+    c = CASES[name]
+    z = load_npz(name)
+    opt, params, ref, ref_params, worst = run_both(c)
+    assert worst < 0.0, worst
+    for i, p in enumerate(params):
+        assert rel_err(p.detach().cpu().reshape(-1), z[f"final_p{i}"]) < 1e-3
+    ng = opt._groups[0]
+    for k, bi in enumerate(ng.native_index):
+        spec = ng.block_specs[bi]
+        st = opt.state[params[spec.param_index]][spec.block_key]["shampoo"]
+        ost = ref.state[bi]
+        for j, f in enumerate(ost["factors"]):
+            got = st["factor_matrices"][j]
+            assert got.dtype == torch.float64 and f.dtype == torch.float64
+            assert rel_err(got.cpu(), f) < 1e-6, (k, j)
+        for j, f in enumerate(ost["inv"]):
+            got = st["inv_factor_matrices"][j]
+            assert got.dtype == torch.float32
+            assert rel_err(got.cpu(), f) < 1e-3, (k, j)
+    if name.endswith("newton"):
+        want = [int(v) for v in z["newton_iterations"][-1] if v >= 0]
+        got = ng.last_newton_iterations
+        assert len(got) == len(want) and max(abs(a - b) for a, b in zip(got, want)) <= 1, (got, want)
+
+
+def test_float64_factors_with_a_rank_deficient_factor_stay_finite():
+    """EigenConfig on float64 factors: a 16 x 4 block gives, after two steps, an order-16 factor of rank 8 whose fp32
+    Gram entries make it indefinite at the 1e-7 level.  The reference's eigendecomposition shifts such a spectrum by
+    its smallest eigenvalue; the native double-precision iteration widens its ridge to epsilon + 2^-21 ||A||_F.  The
+    step must go through and the stored inverse root must be (A + ridge I)^(-1/4) of the stored float64 factor."""
+    import optimizers_amd as oa
+    from oracle.shampoo_oracle import unpack_triu
+
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    p = torch.nn.Parameter(torch.zeros(16, 4, device=dev))
+    pc = oa.RootInvShampooPreconditionerConfig(factor_matrix_dtype=torch.float64, inverse_exponent_override={2: {1: 0.0}})
+    opt = oa.DistributedShampoo([p], lr=1e-3, betas=(0.0, 1.0), epsilon=1e-10, max_preconditioner_dim=16,
+                                precondition_frequency=1, start_preconditioning_step=2, preconditioner_config=pc,
+                                grafting_config=oa.SGDPreconditionerConfig())
+    for _ in range(2):
+        p.grad = torch.randn(16, 4, device=dev)
+        opt.step()
+    st = opt.state[p]["block_0"]["shampoo"]
+    a = unpack_triu(st["factor_matrices"][0].cpu(), 16)
+    assert a.dtype == torch.float64
+    x = unpack_triu(st["inv_factor_matrices"][0].cpu(), 16).double()
+    assert bool(torch.isfinite(x).all()) and bool(torch.isfinite(p).all())
+    eye = torch.eye(16, dtype=torch.float64)
+    lam = torch.linalg.eigvalsh(a)
+    assert float(lam[0]) < 0.0 < 1e-10 < float(-lam[0]), "the case must be indefinite beyond epsilon"
+    ridge = 1e-10 + float(torch.linalg.norm(a + 1e-10 * eye)) * 2.0**-21
+    lam, q = torch.linalg.eigh(a + ridge * eye)
+    assert rel_err(x, (q * lam.pow(-0.25)) @ q.T) < 1e-4
+
+
+@pytest.mark.parametrize("kind", ["newton", "eigh"])
+def test_float64_factors_at_moderate_size(kind):
+    """The fp64 GEMM path over several 128 x 128 tiles per factor (orders 1100 -> 9 x 9 tiles, 400, 300, 200) against the
+    oracle with float64 factor matrices."""
+    c = dict(
+        shapes=[[1100, 400], [300, 200]], seed=91, grad_scale=0.05, steps=6,
+        lr=1e-3, betas=[0.9, 0.999], epsilon=1e-12, weight_decay=0.0, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=2048, precondition_frequency=1, start_preconditioning_step=4,
+        preconditioner=kind, factor_matrix_dtype="float64", override_1d=True, grafting="adam", grafting_beta2=0.999,
+        grafting_epsilon=1e-8,
+    )
+    opt, params, ref, ref_params, worst = run_both(c)
+    assert worst < 0.0, worst
+    ng = opt._groups[0]
+    for k, bi in enumerate(ng.native_index):
+        spec = ng.block_specs[bi]
+        st = opt.state[params[spec.param_index]][spec.block_key]["shampoo"]
+        ost = ref.state[bi]
+        for j, f in enumerate(ost["factors"]):
+            assert rel_err(st["factor_matrices"][j].cpu(), f) < 1e-6, (k, j)
+        for j, f in enumerate(ost["inv"]):
+            assert rel_err(st["inv_factor_matrices"][j].cpu(), f) < 1e-3, (k, j)
