@@ -82,6 +82,7 @@ typedef struct sa_block_desc {
   float* corrected_eigenvalues;
   int32_t mid;            /* d1 of an order-3 block, else 0 */
   int64_t ld_outer;       /* stride of dim 0 of an order-3 block */
+  float* weight_buffer;   /* the "z" sequence of generalized primal averaging / Schedule-Free (rows * cols, contiguous), or NULL */
 } sa_block_desc;
 
 /* Scalars of one step, already evaluated by the host exactly as the reference evaluates
@@ -101,6 +102,12 @@ typedef struct sa_step_scalars {
   float momentum;           /* 0 = classic momentum off */
   float dampening;
   int32_t use_nesterov;
+  /* Generalized primal averaging / Schedule-Free (distributed_shampoo.py:1343-1382), applied to the scaled direction
+   * D = -lr P: T = Z - W; Z += D; D <- D * averaging_direction_coeff + averaging_buffer_coeff * T; W += D, with
+   * averaging_direction_coeff = 1 - mu_y mu_x and averaging_buffer_coeff = 1 - mu_x evaluated by the host in fp32. */
+  int32_t use_primal_averaging;
+  float averaging_direction_coeff;
+  float averaging_buffer_coeff;
 } sa_step_scalars;
 
 const char* sa_last_error(void);
@@ -250,6 +257,11 @@ int32_t sa_precondition(sa_plan* plan, const sa_step_scalars* s, void* stream);
 /* Grafting rescale, weight decay, momentum, learning rate and W += P
  * (distributed_shampoo.py:1115-1122, 1202-1293, 1484; shampoo_distributor.py:335-365). */
 int32_t sa_apply_update(sa_plan* plan, const sa_step_scalars* s, void* stream);
+
+/* W += coeff * (Z - W) for every block that has a weight buffer, masked or not: the switch between the training
+ * sequence y and the evaluation sequence x of generalized primal averaging / Schedule-Free,
+ * `DistributedShampoo.train()` (coeff = 1 - mu_y) and `eval()` (coeff = 1 - 1 / mu_y), distributed_shampoo.py:1729-1793. */
+int32_t sa_move_params_towards_weight_buffer(sa_plan* plan, float coeff, void* stream);
 
 /* Whole step before preconditioning starts: the grafted direction is the update
  * (distributed_shampoo.py:1093-1098 followed by :1202-1293, 1484). */

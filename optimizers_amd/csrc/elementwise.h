@@ -46,6 +46,7 @@ struct BlockDev {
   float* g3_perm;         // order 3: the same permuted to d1 x d0 x d2, or nullptr
   float* g3_ghat;         // order 3, beta1 == 0: dense copy of the gradient for the mode products, or nullptr
   float* g3_stat;         // order 3, eigenvalue-corrected: dense copy of the gradient for the rotated second moment
+  float* weight_buffer;    // z sequence of primal averaging, or null
 };
 
 // offset of element e (block's own row-major order) inside the strided param / grad view
@@ -128,9 +129,14 @@ __device__ __forceinline__ PreOut pre_element(float g, float& m, float& v, float
 }
 
 __device__ __forceinline__ float apply_element(float p, float& w, float& mom, const sa_step_scalars& s,
-                                               float scale, bool has_mom) {
+                                               float scale, bool has_mom, float& z, bool has_avg) {
   p = p * scale;
-  if (s.weight_decay_alpha != 0.0f) p = p + s.weight_decay_alpha * w;
+  if (s.weight_decay_alpha != 0.0f) {
+    // with primal averaging the decay shrinks the z sequence instead of entering the direction, which the averaging
+    // reuses (distributed_shampoo.py:1202-1254)
+    if (has_avg) z = z * (1.0f - s.lr * s.weight_decay_alpha);
+    else p = p + s.weight_decay_alpha * w;
+  }
   if (has_mom) {
     float mb = mom * s.momentum;
     mb = mb + (1.0f - s.dampening) * p;
@@ -138,6 +144,12 @@ __device__ __forceinline__ float apply_element(float p, float& w, float& mom, co
     p = s.use_nesterov ? (p * (1.0f - s.dampening)) + s.momentum * mb : mb;
   }
   p = p * (-s.lr);
+  if (has_avg) {
+    const float t = z - w;
+    z = z + p;
+    p = p * s.averaging_direction_coeff;
+    p = p + s.averaging_buffer_coeff * t;
+  }
   w = w + p;
   return p;
 }
@@ -156,6 +168,10 @@ __global__ __launch_bounds__(EW_THREADS) void grafting_kernel(const BlockDev* __
   const int n_el = B.rows * B.cols;
   const bool has_m = B.filtered_grad != nullptr, has_v = B.adagrad != nullptr;
   const bool has_mom = B.momentum != nullptr && s.momentum != 0.0f;
+  // classic momentum and primal averaging exclude each other: one auxiliary state buffer per block
+  const bool has_avg = B.weight_buffer != nullptr && s.use_primal_averaging != 0;
+  const bool has_aux = has_mom || has_avg;
+  float* __restrict__ aux = has_avg ? B.weight_buffer : B.momentum;
   const bool b3 = B.ghat_tmp != nullptr;
   float gsum = 0.f, hsum = 0.f;
   constexpr int NIT = EW_CHUNK / (EW_THREADS * 4);
@@ -178,7 +194,7 @@ __global__ __launch_bounds__(EW_THREADS) void grafting_kernel(const BlockDev* __
       v[it] = has_v ? nt_load4(B.adagrad + e) : make_float4(0, 0, 0, 0);
       if (MODE == 1) {
         w[it] = nt_load4(B.param + gi[it]);
-        mo[it] = has_mom ? nt_load4(B.momentum + e) : make_float4(0, 0, 0, 0);
+        mo[it] = has_aux ? nt_load4(aux + e) : make_float4(0, 0, 0, 0);
       }
     }
 #pragma unroll
@@ -196,12 +212,12 @@ __global__ __launch_bounds__(EW_THREADS) void grafting_kernel(const BlockDev* __
         gsum += (o0.graft * o0.graft + o1.graft * o1.graft) + (o2.graft * o2.graft + o3.graft * o3.graft);
         hsum += (o0.ghat * o0.ghat + o1.ghat * o1.ghat) + (o2.ghat * o2.ghat + o3.ghat * o3.ghat);
       } else {
-        apply_element(o0.graft, w[it].x, mo[it].x, s, 1.0f, has_mom);
-        apply_element(o1.graft, w[it].y, mo[it].y, s, 1.0f, has_mom);
-        apply_element(o2.graft, w[it].z, mo[it].z, s, 1.0f, has_mom);
-        apply_element(o3.graft, w[it].w, mo[it].w, s, 1.0f, has_mom);
+        apply_element(o0.graft, w[it].x, mo[it].x, s, 1.0f, has_mom, mo[it].x, has_avg);
+        apply_element(o1.graft, w[it].y, mo[it].y, s, 1.0f, has_mom, mo[it].y, has_avg);
+        apply_element(o2.graft, w[it].z, mo[it].z, s, 1.0f, has_mom, mo[it].z, has_avg);
+        apply_element(o3.graft, w[it].w, mo[it].w, s, 1.0f, has_mom, mo[it].w, has_avg);
         *reinterpret_cast<float4*>(B.param + gi[it]) = w[it];
-        if (has_mom) nt_store4(mo[it], B.momentum + e);
+        if (has_aux) nt_store4(mo[it], aux + e);
       }
     }
   } else
@@ -228,13 +244,13 @@ __global__ __launch_bounds__(EW_THREADS) void grafting_kernel(const BlockDev* __
         hsum += (o0.ghat * o0.ghat + o1.ghat * o1.ghat) + (o2.ghat * o2.ghat + o3.ghat * o3.ghat);
       } else {
         float4 w = *reinterpret_cast<const float4*>(B.param + gi);
-        float4 mo = has_mom ? *reinterpret_cast<const float4*>(B.momentum + e) : make_float4(0, 0, 0, 0);
-        apply_element(o0.graft, w.x, mo.x, s, 1.0f, has_mom);
-        apply_element(o1.graft, w.y, mo.y, s, 1.0f, has_mom);
-        apply_element(o2.graft, w.z, mo.z, s, 1.0f, has_mom);
-        apply_element(o3.graft, w.w, mo.w, s, 1.0f, has_mom);
+        float4 mo = has_aux ? *reinterpret_cast<const float4*>(aux + e) : make_float4(0, 0, 0, 0);
+        apply_element(o0.graft, w.x, mo.x, s, 1.0f, has_mom, mo.x, has_avg);
+        apply_element(o1.graft, w.y, mo.y, s, 1.0f, has_mom, mo.y, has_avg);
+        apply_element(o2.graft, w.z, mo.z, s, 1.0f, has_mom, mo.z, has_avg);
+        apply_element(o3.graft, w.w, mo.w, s, 1.0f, has_mom, mo.w, has_avg);
         *reinterpret_cast<float4*>(B.param + gi) = w;
-        if (has_mom) *reinterpret_cast<float4*>(B.momentum + e) = mo;
+        if (has_aux) *reinterpret_cast<float4*>(aux + e) = mo;
       }
     } else {
       for (int k = 0; k < 4 && e + k < n_el; ++k) {
@@ -253,10 +269,10 @@ __global__ __launch_bounds__(EW_THREADS) void grafting_kernel(const BlockDev* __
           hsum += o.ghat * o.ghat;
         } else {
           float w = B.param[gk];
-          float mo = has_mom ? B.momentum[ee] : 0.f;
-          apply_element(o.graft, w, mo, s, 1.0f, has_mom);
+          float mo = has_aux ? aux[ee] : 0.f;
+          apply_element(o.graft, w, mo, s, 1.0f, has_mom, mo, has_avg);
           B.param[gk] = w;
-          if (has_mom) B.momentum[ee] = mo;
+          if (has_aux) aux[ee] = mo;
         }
       }
     }
@@ -309,6 +325,10 @@ __global__ __launch_bounds__(EW_THREADS) void apply_kernel(const BlockDev* __res
   const BlockDev& B = blocks[cr.block];
   const int n_el = B.rows * B.cols;
   const bool has_mom = B.momentum != nullptr && s.momentum != 0.0f;
+  // classic momentum and primal averaging exclude each other: one auxiliary state buffer per block
+  const bool has_avg = B.weight_buffer != nullptr && s.use_primal_averaging != 0;
+  const bool has_aux = has_mom || has_avg;
+  float* __restrict__ aux = has_avg ? B.weight_buffer : B.momentum;
   const float p_div = B.p_is_ghat ? s.bias_correction1 : 1.0f;
   float scale = 1.0f;
   if (s.graft_type != SA_GRAFT_NONE) {
@@ -328,17 +348,17 @@ __global__ __launch_bounds__(EW_THREADS) void apply_kernel(const BlockDev* __res
       const long long pi = direction_offset(B, e);
       p[it] = nt_load4(B.p_src + pi);
       w[it] = nt_load4(B.param + wi[it]);
-      mo[it] = has_mom ? nt_load4(B.momentum + e) : make_float4(0, 0, 0, 0);
+      mo[it] = has_aux ? nt_load4(aux + e) : make_float4(0, 0, 0, 0);
     }
 #pragma unroll
     for (int it = 0; it < NIT; ++it) {
       const int e = cr.start + (it * EW_THREADS + threadIdx.x) * 4;
-      apply_element(p[it].x / p_div, w[it].x, mo[it].x, s, scale, has_mom);
-      apply_element(p[it].y / p_div, w[it].y, mo[it].y, s, scale, has_mom);
-      apply_element(p[it].z / p_div, w[it].z, mo[it].z, s, scale, has_mom);
-      apply_element(p[it].w / p_div, w[it].w, mo[it].w, s, scale, has_mom);
+      apply_element(p[it].x / p_div, w[it].x, mo[it].x, s, scale, has_mom, mo[it].x, has_avg);
+      apply_element(p[it].y / p_div, w[it].y, mo[it].y, s, scale, has_mom, mo[it].y, has_avg);
+      apply_element(p[it].z / p_div, w[it].z, mo[it].z, s, scale, has_mom, mo[it].z, has_avg);
+      apply_element(p[it].w / p_div, w[it].w, mo[it].w, s, scale, has_mom, mo[it].w, has_avg);
       *reinterpret_cast<float4*>(B.param + wi[it]) = w[it];
-      if (has_mom) nt_store4(mo[it], B.momentum + e);
+      if (has_aux) nt_store4(mo[it], aux + e);
     }
   } else
 #pragma unroll
@@ -351,24 +371,44 @@ __global__ __launch_bounds__(EW_THREADS) void apply_kernel(const BlockDev* __res
     if (vec) {
       float4 p = *reinterpret_cast<const float4*>(B.p_src + pi);
       float4 w = *reinterpret_cast<const float4*>(B.param + wi);
-      float4 mo = has_mom ? *reinterpret_cast<const float4*>(B.momentum + e) : make_float4(0, 0, 0, 0);
-      apply_element(p.x / p_div, w.x, mo.x, s, scale, has_mom);
-      apply_element(p.y / p_div, w.y, mo.y, s, scale, has_mom);
-      apply_element(p.z / p_div, w.z, mo.z, s, scale, has_mom);
-      apply_element(p.w / p_div, w.w, mo.w, s, scale, has_mom);
+      float4 mo = has_aux ? *reinterpret_cast<const float4*>(aux + e) : make_float4(0, 0, 0, 0);
+      apply_element(p.x / p_div, w.x, mo.x, s, scale, has_mom, mo.x, has_avg);
+      apply_element(p.y / p_div, w.y, mo.y, s, scale, has_mom, mo.y, has_avg);
+      apply_element(p.z / p_div, w.z, mo.z, s, scale, has_mom, mo.z, has_avg);
+      apply_element(p.w / p_div, w.w, mo.w, s, scale, has_mom, mo.w, has_avg);
       *reinterpret_cast<float4*>(B.param + wi) = w;
-      if (has_mom) *reinterpret_cast<float4*>(B.momentum + e) = mo;
+      if (has_aux) *reinterpret_cast<float4*>(aux + e) = mo;
     } else {
       for (int k = 0; k < 4 && e + k < n_el; ++k) {
         const int ee = e + k;
         const long long wk = view_offset(B, ee);
         const long long pk = direction_offset(B, ee);
         float w = B.param[wk];
-        float mo = has_mom ? B.momentum[ee] : 0.f;
-        apply_element(B.p_src[pk] / p_div, w, mo, s, scale, has_mom);
+        float mo = has_aux ? aux[ee] : 0.f;
+        apply_element(B.p_src[pk] / p_div, w, mo, s, scale, has_mom, mo, has_avg);
         B.param[wk] = w;
-        if (has_mom) B.momentum[ee] = mo;
+        if (has_aux) aux[ee] = mo;
       }
+    }
+  }
+}
+
+// W += coeff * (Z - W) over the chunks of every block with a weight buffer (train / eval switch of primal averaging).
+__global__ __launch_bounds__(EW_THREADS) void move_params_kernel(const BlockDev* __restrict__ blocks,
+                                                                const ChunkRef* __restrict__ chunks, float coeff) {
+  const ChunkRef cr = chunks[blockIdx.x];
+  const BlockDev& B = blocks[cr.block];
+  if (B.weight_buffer == nullptr) return;
+  const int n_el = B.rows * B.cols;
+  constexpr int NIT = EW_CHUNK / (EW_THREADS * 4);
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int e0 = cr.start + (it * EW_THREADS + threadIdx.x) * 4;
+    for (int k = 0; k < 4 && e0 + k < n_el; ++k) {
+      const long long wi = view_offset(B, e0 + k);
+      const float w = B.param[wi];
+      const float t = B.weight_buffer[e0 + k] - w;
+      B.param[wi] = w + t * coeff;
     }
   }
 }

@@ -258,6 +258,7 @@ struct sa_plan {
     }
   };
   GemmTable64 n64_a[2], n64_pow[8], n64_m[2];
+  Table<ChunkRef> t_all_chunks;  // chunks of every block, masked or not (train / eval switch of primal averaging)
   // KL-Shampoo: the Gram matrices of a two-sided block are taken of the gradient preconditioned along the other dim
   bool kl = false;
   GemmTable kl_right, kl_left;  // G X_R -> T buffer, X_L G -> P buffer
@@ -377,6 +378,7 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
     B.filtered_grad = d.filtered_grad;
     B.adagrad = d.adagrad;
     B.momentum = d.momentum_buffer;
+    B.weight_buffer = d.weight_buffer;
     B.ld = d.ld;
     B.rows = d.rows;
     B.cols = d.cols;
@@ -412,7 +414,7 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
     B.contig = contig ? 1 : 0;
     auto al = [](const void* q) { return q == nullptr || (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
     const bool shape_ok = contig || (d.cols % 4 == 0 && d.ld % 4 == 0 && (d.mid == 0 || d.ld_outer % 4 == 0));
-    B.vec = (shape_ok && al(B.param) && al(B.grad) && al(B.filtered_grad) && al(B.adagrad) && al(B.momentum) &&
+    B.vec = (shape_ok && al(B.param) && al(B.grad) && al(B.filtered_grad) && al(B.adagrad) && al(B.momentum) && al(B.weight_buffer) &&
              al(B.ghat_tmp)) ? 1 : 0;
     const bool p_contig = (B.p_ld == d.cols);
     B.p_vec = ((p_contig || (d.cols % 4 == 0 && B.p_ld % 4 == 0)) && al(B.p_src)) ? 1 : 0;
@@ -755,6 +757,8 @@ int validate_scalars(const sa_plan* p, const sa_step_scalars* s) {
     if (s->beta1 != 0.0f && !d.filtered_grad) return fail(SA_ERR_INVALID, "beta1 != 0 needs filtered_grad state in every block");
     if (s->graft_type == SA_GRAFT_ADAGRAD && !d.adagrad) return fail(SA_ERR_INVALID, "adagrad-family grafting needs adagrad state in every block");
     if (s->momentum != 0.0f && !d.momentum_buffer) return fail(SA_ERR_INVALID, "momentum != 0 needs momentum_buffer state in every block");
+    if (s->use_primal_averaging && !d.weight_buffer) return fail(SA_ERR_INVALID, "primal averaging needs weight_buffer state in every block");
+    if (s->use_primal_averaging && s->momentum != 0.0f) return fail(SA_ERR_INVALID, "classic momentum and primal averaging exclude each other");
   }
   if (!(s->bias_correction1 != 0.0f) || !(s->graft_bias_correction2 != 0.0f)) return fail(SA_ERR_INVALID, "bias corrections must be non-zero divisors");
   return SA_OK;
@@ -837,8 +841,8 @@ static int launch_gemm64(sa_plan::GemmTable64& g, double mp_scale, double mp_dia
 extern "C" {
 
 const char* sa_last_error(void) { return g_err.c_str(); }
-int32_t sa_abi_version(void) { return 2; }
-static_assert(sizeof(sa_block_desc) == 160, "sa_block_desc layout changed: bump sa_abi_version and the ctypes mirror");
+int32_t sa_abi_version(void) { return 3; }
+static_assert(sizeof(sa_block_desc) == 168, "sa_block_desc layout changed: bump sa_abi_version and the ctypes mirror");
 
 int32_t sa_set_profiling(int32_t enabled) {
   g_profiling = enabled != 0;
@@ -1023,6 +1027,7 @@ void sa_plan_destroy(sa_plan* p) {
   for (auto& g : p->nt_h) g.t.destroy();
   for (auto& a : p->g3) for (auto& b2 : a) for (auto& g : b2) g.t.destroy();
   for (auto& a : p->e3) for (auto& b2 : a) for (auto& c2 : b2) for (auto& g : c2) g.t.destroy();
+  p->t_all_chunks.destroy();
   p->t_f64.destroy();
   for (auto* g : {&p->n64_a[0], &p->n64_a[1], &p->n64_m[0], &p->n64_m[1]}) g->t.destroy();
   for (auto& g : p->n64_pow) g.t.destroy();
@@ -1227,11 +1232,37 @@ int32_t sa_apply_update(sa_plan* p, const sa_step_scalars* sc, void* stream) {
   for (int b = 0; b < p->n_blocks; ++b)
     if (block_active(p, b)) {
       const sa_block_desc& d = p->blocks[b];
-      bytes += 4.0 * (double)d.rows * d.cols * (3 + (d.momentum_buffer && sc->momentum != 0.0f ? 2 : 0));
+      bytes += 4.0 * (double)d.rows * d.cols *
+               (3 + ((d.momentum_buffer && sc->momentum != 0.0f) || (d.weight_buffer && sc->use_primal_averaging) ? 2 : 0));
     }
   Span span("apply", s, bytes, 1, true);
   hipLaunchKernelGGL(apply_kernel, dim3((unsigned)p->t_chunks.n), dim3(EW_THREADS), 0, s, p->t_blocks.dev,
                      p->t_chunks.dev, *sc, p->n_blocks, p->f(p->off_norms));
+  HIPCHECK(hipGetLastError());
+  return SA_OK;
+}
+
+int32_t sa_move_params_towards_weight_buffer(sa_plan* p, float coeff, void* stream) {
+  if (!p) return fail(SA_ERR_INVALID, "NULL plan");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // the block table must exist; gradients need not be bound for this call
+  if (!p->tables_valid) {
+    if (!p->grads_bound) { p->grads.assign(p->n_blocks, nullptr); }
+    SACHECK(rebuild_tables(p, p->table_mode < 0 ? 0 : p->table_mode, s));
+    p->tables_valid = p->grads_bound;
+  }
+  std::vector<ChunkRef> chunks;
+  for (int b = 0; b < p->n_blocks; ++b) {
+    const sa_block_desc& d = p->blocks[b];
+    if (!d.weight_buffer) continue;
+    const long long n_el = (long long)d.rows * d.cols;
+    for (long long e = 0; e < n_el; e += EW_CHUNK) chunks.push_back(ChunkRef{b, (int)e});
+  }
+  if (chunks.empty()) return SA_OK;
+  SACHECK(p->t_all_chunks.begin(chunks.size()));
+  std::memcpy(p->t_all_chunks.host, chunks.data(), chunks.size() * sizeof(ChunkRef));
+  SACHECK(p->t_all_chunks.upload(s));
+  hipLaunchKernelGGL(move_params_kernel, dim3((unsigned)chunks.size()), dim3(EW_THREADS), 0, s, p->t_blocks.dev, p->t_all_chunks.dev, coeff);
   HIPCHECK(hipGetLastError());
   return SA_OK;
 }

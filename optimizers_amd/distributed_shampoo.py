@@ -59,6 +59,11 @@ from optimizers_amd.shampoo_types import (
     AdamPreconditionerConfig,
     BaseShampooPreconditionerConfig,
     ClassicMomentumConfig,
+    GeneralizedPrimalAveragingConfig,
+    LR_SUM,
+    ScheduleFreeConfig,
+    TRAIN_MODE,
+    WEIGHT_BUFFER,
     ConcurrencyConfig,
     DefaultConcurrencyConfig,
     DefaultShampooConfig,
@@ -359,6 +364,8 @@ class _NativeGroup(_AmortizedComputation):
         self.filtered_arena = _Arena(numels, self.device) if beta1 != 0.0 else None
         self.adagrad_arena = _Arena(numels, self.device) if self.graft_type == native.SA_GRAFT_ADAGRAD else None
         self.momentum_arena = _Arena(numels, self.device) if isinstance(momentum_cfg, ClassicMomentumConfig) else None
+        self.primal_averaging = isinstance(momentum_cfg, (GeneralizedPrimalAveragingConfig, ScheduleFreeConfig))
+        self.weight_arena = _Arena(numels, self.device) if self.primal_averaging else None
 
         # optimizer.state layout (reference golden: tests/distributed_shampoo_test.py:516-622)
         descs = (native.BlockDesc * max(nb, 1))()
@@ -469,6 +476,13 @@ class _NativeGroup(_AmortizedComputation):
                 block_state[MOMENTUM_BUFFER] = self.momentum_arena.view(k, s.shape)
                 d.momentum_buffer = block_state[MOMENTUM_BUFFER].data_ptr()
                 self._slots.append((p, s.block_key, (MOMENTUM_BUFFER,), block_state[MOMENTUM_BUFFER]))
+            if self.weight_arena is not None:
+                # the "z" sequence starts at the current parameters (distributed_shampoo.py:909-922)
+                z = self.weight_arena.view(k, s.shape)
+                z.copy_(torch.as_strided(p.detach(), s.shape, s.strides, p.storage_offset() + s.offset))
+                block_state[WEIGHT_BUFFER] = z
+                d.weight_buffer = z.data_ptr()
+                self._slots.append((p, s.block_key, (WEIGHT_BUFFER,), z))
             logger.info(
                 f"Instantiated Shampoo Preconditioner {s.param_index}.{s.block_key} for Parameter {s.param_index} "
                 f"({tuple(p.shape)}), Block {s.block_key} ({s.shape})."
@@ -516,6 +530,13 @@ class _NativeGroup(_AmortizedComputation):
         self.step_tensor = torch.tensor(0, dtype=torch.int64, device="cpu")
         for p in params:
             optimizer.state[p][STEP] = self.step_tensor
+        if self.primal_averaging:
+            # per-group scalars aliased under every parameter (distributed_shampoo.py:924-937)
+            self.lr_sum = torch.tensor(0.0, dtype=torch.float, device=self.device)
+            self.train_mode = torch.tensor(True, dtype=torch.bool, device="cpu")
+            for p in params:
+                optimizer.state[p][TRAIN_MODE] = self.train_mode
+                optimizer.state[p][LR_SUM] = self.lr_sum
         self.stream: torch.cuda.Stream | None = None
 
     def _identity(self, n: int) -> torch.Tensor:
@@ -593,10 +614,11 @@ class _NativeGroup(_AmortizedComputation):
         elif pc.factor_matrix_dtype != torch.float32:
             raise NotImplementedError(f"factor matrices are fp32 or fp64 in the native step, got {pc.factor_matrix_dtype}")
         if group[ITERATE_AVERAGING_CONFIG] is not None and not isinstance(
-            group[ITERATE_AVERAGING_CONFIG], ClassicMomentumConfig
+            group[ITERATE_AVERAGING_CONFIG], (ClassicMomentumConfig, GeneralizedPrimalAveragingConfig, ScheduleFreeConfig)
         ):
             raise NotImplementedError(
-                f"{group[ITERATE_AVERAGING_CONFIG]=} is not supported! Supported configs: ClassicMomentumConfig."
+                f"{group[ITERATE_AVERAGING_CONFIG]=} is not supported! "
+                "Supported configs: ClassicMomentumConfig, GeneralizedPrimalAveragingConfig, ScheduleFreeConfig."
             )
 
     @staticmethod
@@ -656,6 +678,35 @@ class _NativeGroup(_AmortizedComputation):
                 active += 1
         self._grads_alive = grads  # keep the tensors alive until the step has been enqueued
         return active
+
+    def _interp_coeffs(self, cfg: Any, lr: torch.Tensor | None) -> tuple[torch.Tensor, torch.Tensor]:
+        """(mu_y, mu_x) as fp32 tensors, distributed_shampoo.py:1296-1340.  Schedule-Free accumulates lr^power in
+        `lr_sum` (state) and uses mu_x = 1 - lr^power / lr_sum; without an lr (train / eval switch) mu_x is 0."""
+        train = torch.tensor(cfg.train_interp_coeff, dtype=torch.float32)
+        if isinstance(cfg, GeneralizedPrimalAveragingConfig):
+            return train, torch.tensor(cfg.eval_interp_coeff, dtype=torch.float32)
+        if lr is None:
+            logger.warning("lr or lr_sum not provided to _get_train_and_eval_interp_coeffs; returning eval_interp_coeff = 0.0!")
+            return train, torch.tensor(0.0, dtype=torch.float32)
+        lr_power = torch.pow(lr, cfg.eval_coeff_lr_power)
+        lr_sum = self.lr_sum.cpu() + lr_power
+        self.lr_sum.copy_(lr_sum)
+        return train, 1.0 - lr_power / lr_sum
+
+    def switch_mode(self, group: dict[str, Any], train: bool) -> None:
+        """train(): y = x + (1 - mu_y)(z - x); eval(): x = y + (1 - 1/mu_y)(z - y), on every block
+        (distributed_shampoo.py:1729-1797)."""
+        if not self.primal_averaging or bool(self.train_mode) == train:
+            return
+        mu_y, _ = self._interp_coeffs(group[ITERATE_AVERAGING_CONFIG], None)
+        coeff = float(1 - mu_y) if train else float(1 - torch.reciprocal(mu_y))
+        if self.n_native:
+            with torch.cuda.device(self.device):
+                native.check(
+                    self.lib.sa_move_params_towards_weight_buffer(self.plan, coeff, native.current_stream_ptr(self.device)),
+                    "sa_move_params_towards_weight_buffer",
+                )
+        self.train_mode.fill_(train)
 
     def step(self, group: dict[str, Any], runtime: ShampooRuntimeConfig) -> None:
         lib = self.lib
@@ -735,6 +786,15 @@ class _NativeGroup(_AmortizedComputation):
             s.momentum, s.dampening, s.use_nesterov = mom.momentum, mom.dampening, int(mom.use_nesterov)
         else:
             s.momentum, s.dampening, s.use_nesterov = 0.0, 0.0, 0
+        if self.primal_averaging:
+            if not bool(self.train_mode):
+                raise RuntimeError(
+                    "Called _apply_in_place_primal_averaging when not in train mode. Call optimizer.train() before calling optimizer.step()!"
+                )
+            train_coeff, eval_coeff = self._interp_coeffs(mom, torch.tensor(group[LR], dtype=torch.float32))
+            s.use_primal_averaging = 1
+            s.averaging_direction_coeff = float(1 - train_coeff * eval_coeff)
+            s.averaging_buffer_coeff = float(1 - eval_coeff)
 
         ref = ctypes.byref(s)
         if graft_only:
@@ -766,7 +826,7 @@ class DistributedShampoo(torch.optim.Optimizer):
     `RootInvKLShampooPreconditionerConfig` / `EigendecomposedKLShampooPreconditionerConfig` (blocks of order 1 and 2),
     `EigenvalueCorrectedShampooPreconditionerConfig` and `EigendecomposedShampooPreconditionerConfig` with
     `QREigendecompositionConfig` or `EighEigendecompositionConfig` (including `ignored_basis_change_dims`), grafting with SGD / AdaGrad / RMSprop /
-    Adam or none, every `WeightDecayType`, `ClassicMomentumConfig`, `inverse_exponent_override`,
+    Adam or none, every `WeightDecayType`, `ClassicMomentumConfig`, `GeneralizedPrimalAveragingConfig`, `ScheduleFreeConfig`, `inverse_exponent_override`,
     `SingleDeviceDistributedConfig`, fp32 state with packed factor matrices (`factor_matrix_dtype=torch.float64` for
     root-inverse Shampoo: fp64 factor averages and an fp64 coupled Newton root inverse), blocks of order 1 to 3 (order 3: what is left of
     convolution weights).
@@ -890,14 +950,19 @@ class DistributedShampoo(torch.optim.Optimizer):
 
     @torch.no_grad()
     def train(self) -> None:
-        """distributed_shampoo.py:1729-1761: switches groups with primal-averaging / schedule-free iterate averaging
-        to the training iterate.  Only `ClassicMomentumConfig` is built here, for which the reference does nothing."""
+        """distributed_shampoo.py:1729-1761: groups with primal averaging / Schedule-Free move back to the training
+        sequence."""
         logger.info("Enabling train mode in Distributed Shampoo!")
+        for ng, group in zip(self._groups, self.param_groups, strict=True):
+            ng.switch_mode(group, train=True)
 
     @torch.no_grad()
     def eval(self) -> None:
-        """distributed_shampoo.py:1763-1795; nothing to do without primal-averaging / schedule-free groups."""
+        """distributed_shampoo.py:1763-1797: groups with primal averaging / Schedule-Free move to the evaluation
+        sequence."""
         logger.info("Enabling eval mode in Distributed Shampoo!")
+        for ng, group in zip(self._groups, self.param_groups, strict=True):
+            ng.switch_mode(group, train=False)
 
     @torch.no_grad()
     def step(self, closure: Callable[[], float] | None = None) -> float | None:
@@ -951,6 +1016,14 @@ def _restore_state(self: _NativeGroup, optimizer: DistributedShampoo) -> None:
         self.step_tensor.fill_(loaded_steps[0])
     for p in self.params:
         optimizer.state[p][STEP] = self.step_tensor
+    if self.primal_averaging:
+        # per-group scalars of primal averaging / Schedule-Free, re-aliased under every parameter
+        for key, mine in ((LR_SUM, self.lr_sum), (TRAIN_MODE, self.train_mode)):
+            loaded = [optimizer.state[p][key] for p in self.params if key in optimizer.state[p]]
+            if loaded:
+                mine.copy_(torch.as_tensor(loaded[0]).to(device=mine.device, dtype=mine.dtype))
+            for p in self.params:
+                optimizer.state[p][key] = mine
     if self.plan:
         native.check(self.lib.sa_plan_invalidate_inverse_cache(self.plan), "sa_plan_invalidate_inverse_cache")
     # eigendecomposed Shampoo: the inverse roots are a function of the restored (Q, lambda)

@@ -36,7 +36,7 @@ EXPORTS = (
     "sa_gemm_f32", "sa_copy_f32", "sa_set_profiling", "sa_phase_ms", "sa_phase_flops", "sa_phase_launches", "sa_phase_executed_flops", "sa_set_symmetric_newton", "sa_set_eigh_solver",
     "sa_plan_set_trace_scaling", "sa_compute_root_inverses_higher_order", "sa_plan_read_eigenvalues", "sa_add_to_views",
     "sa_compute_root_inverses_from_eigendecomposition", "sa_plan_set_kl_shampoo",
-    "sa_plan_set_factor_dtype", "sa_update_factor_matrices_f64", "sa_compute_root_inverses_newton_f64",
+    "sa_move_params_towards_weight_buffer", "sa_plan_set_factor_dtype", "sa_update_factor_matrices_f64", "sa_compute_root_inverses_newton_f64",
 )
 
 
@@ -59,6 +59,7 @@ class BlockDesc(ctypes.Structure):
         ("corrected_eigenvalues", c_void_p),
         ("mid", c_int32),
         ("ld_outer", c_int64),
+        ("weight_buffer", c_void_p),
     ]
 
 
@@ -77,6 +78,9 @@ class StepScalars(ctypes.Structure):
         ("momentum", c_float),
         ("dampening", c_float),
         ("use_nesterov", c_int32),
+        ("use_primal_averaging", c_int32),
+        ("averaging_direction_coeff", c_float),
+        ("averaging_buffer_coeff", c_float),
     ]
 
 
@@ -161,6 +165,7 @@ def load() -> ctypes.CDLL:
         c_void_p, POINTER(c_void_p), c_float, POINTER(c_float), c_int32, c_float, c_float, POINTER(c_int32), c_void_p,
     ]
     lib.sa_plan_set_kl_shampoo.argtypes = [c_void_p, c_int32]
+    lib.sa_move_params_towards_weight_buffer.argtypes = [c_void_p, c_float, c_void_p]
     lib.sa_plan_set_factor_dtype.argtypes = [c_void_p, c_int32]
     lib.sa_update_factor_matrices_f64.argtypes = [c_void_p, c_double, c_double, c_void_p]
     lib.sa_compute_root_inverses_newton_f64.argtypes = [

@@ -384,6 +384,10 @@ class OracleConfig:
     grafting: str | None = None
     grafting_beta2: float = 0.999
     grafting_epsilon: float = 1e-10
+    averaging: str | None = None  # "gpa" (GeneralizedPrimalAveragingConfig) | "schedule_free" (ScheduleFreeConfig)
+    eval_interp_coeff: float = 0.9
+    train_interp_coeff: float = 0.8
+    eval_coeff_lr_power: int = 2
     momentum: float = 0.0  # ClassicMomentumConfig.momentum (0 = disabled)
     dampening: float = 0.0
     use_nesterov: bool = False
@@ -416,6 +420,8 @@ class ShampooOracle:
         if self.start < cfg.precondition_frequency:
             raise ValueError("start_preconditioning_step must be >= precondition_frequency")
         self.step_t = torch.tensor(0, dtype=torch.int64)
+        self.lr_sum = torch.tensor(0.0, dtype=torch.float32)
+        self.train_mode = True
         self.soap = cfg.preconditioner.startswith("soap")
         self.eigendecomposed = cfg.preconditioner.startswith("eigendecomposed")
         self.blocks: list[Tensor] = []
@@ -481,6 +487,8 @@ class ShampooOracle:
             st["filtered_grad"] = torch.zeros(b.shape, dtype=dt, device=dev)
         if cfg.momentum != 0.0:
             st["momentum_buffer"] = torch.zeros(b.shape, dtype=dt, device=dev)
+        if cfg.averaging is not None:  # the z sequence starts at the parameters (distributed_shampoo.py:909-922)
+            st["weight_buffer"] = b.detach().clone()
         return st
 
     # -- helpers ------------------------------------------------------------ #
@@ -727,8 +735,12 @@ class ShampooOracle:
                 a = cfg.weight_decay * torch.tensor(cfg.lr, dtype=torch.float32).item() / self.peak_lr
             else:
                 a = cfg.weight_decay / self.peak_lr
-            for p, w in zip(P, W):
-                p.add_(w, alpha=a)
+            if cfg.averaging is not None:  # the decay shrinks z instead of entering the direction
+                for st in S:
+                    st["weight_buffer"].mul_((1 - lr * a).to(st["weight_buffer"].dtype))
+            else:
+                for p, w in zip(P, W):
+                    p.add_(w, alpha=a)
 
         # 6. classic momentum (:1257-1293)
         if cfg.momentum != 0.0:
@@ -740,7 +752,49 @@ class ShampooOracle:
                 else:
                     p.copy_(mb)
 
-        # 7. learning rate and apply (:1484, shampoo_distributor.py:362-365)
-        for p, w in zip(P, W):
+        # 7. learning rate, primal averaging (:1343-1382) and apply (:1484, shampoo_distributor.py:362-365)
+        if cfg.averaging is not None:
+            if not self.train_mode:
+                raise RuntimeError(
+                    "Called _apply_in_place_primal_averaging when not in train mode. Call optimizer.train() before calling optimizer.step()!"
+                )
+            mu_y, mu_x = self._interp_coeffs(lr)
+        for p, w, st in zip(P, W, S):
             p.mul_(-lr)
+            if cfg.averaging is not None:
+                z = st["weight_buffer"]
+                z_minus_y = z - w
+                z.add_(p)
+                p.mul_((1 - mu_y * mu_x).to(p.dtype))
+                p.add_(z_minus_y, alpha=float(1 - mu_x))
             w.add_(p)
+
+    def _interp_coeffs(self, lr: Tensor | None) -> tuple[Tensor, Tensor]:
+        """distributed_shampoo.py:1296-1340: (mu_y, mu_x) as fp32 tensors; Schedule-Free accumulates lr^power."""
+        cfg = self.cfg
+        mu_y = torch.tensor(cfg.train_interp_coeff, dtype=torch.float32)
+        if cfg.averaging == "gpa":
+            return mu_y, torch.tensor(cfg.eval_interp_coeff, dtype=torch.float32)
+        if lr is None:
+            return mu_y, torch.tensor(0.0, dtype=torch.float32)
+        lr_power = torch.pow(lr.to(torch.float32).cpu(), cfg.eval_coeff_lr_power)
+        self.lr_sum = self.lr_sum + lr_power
+        return mu_y, 1.0 - lr_power / self.lr_sum
+
+    def train(self) -> None:
+        """distributed_shampoo.py:1729-1761: y = x + (1 - mu_y)(z - x) on every block."""
+        if self.cfg.averaging is None or self.train_mode:
+            return
+        mu_y, _ = self._interp_coeffs(None)
+        for w, st in zip(self.blocks, self.state):
+            w.add_((st["weight_buffer"] - w) * float(1 - mu_y))
+        self.train_mode = True
+
+    def eval(self) -> None:
+        """distributed_shampoo.py:1763-1797: x = y + (1 - 1/mu_y)(z - y) on every block."""
+        if self.cfg.averaging is None or not self.train_mode:
+            return
+        mu_y, _ = self._interp_coeffs(None)
+        for w, st in zip(self.blocks, self.state):
+            w.add_((st["weight_buffer"] - w) * float(1 - torch.reciprocal(mu_y)))
+        self.train_mode = False

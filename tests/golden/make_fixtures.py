@@ -56,7 +56,11 @@ from distributed_shampoo.preconditioner.matrix_functions import (  # noqa: E402
     matrix_eigendecomposition,
     matrix_inverse_root,
 )
-from distributed_shampoo.shampoo_types import ClassicMomentumConfig  # noqa: E402
+from distributed_shampoo.shampoo_types import (  # noqa: E402
+    ClassicMomentumConfig,
+    GeneralizedPrimalAveragingConfig,
+    ScheduleFreeConfig,
+)
 
 OUT = os.path.dirname(os.path.abspath(__file__))
 
@@ -208,6 +212,24 @@ CASES = {
         max_preconditioner_dim=16, precondition_frequency=2, start_preconditioning_step=4,
         preconditioner="newton", factor_matrix_dtype="float64", override_1d=True, grafting="adagrad", grafting_epsilon=1e-8,
     ),
+    # iterate averaging: generalized primal averaging, with a round trip through eval() / train() after step 7; the first
+    # root inverse comes when the order-16 factor of the 16 x 4 block has seen six gradients (rank 24)
+    "gpa_newton": dict(
+        shapes=[[24, 20], [20]], seed=21, grad_scale=1.0, steps=9,
+        lr=1e-2, betas=[0.9, 0.99], epsilon=1e-6, weight_decay=1e-3, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=16, precondition_frequency=2, start_preconditioning_step=6,
+        preconditioner="newton", override_1d=True, grafting="adam", grafting_beta2=0.99, grafting_epsilon=1e-8,
+        averaging="gpa", eval_interp_coeff=0.9, train_interp_coeff=0.8, toggle_eval_at=7,
+    ),
+    # Schedule-Free with a learning rate that changes every step (mu_x follows lr^2 / sum of lr^2)
+    "schedule_free_eigh": dict(
+        shapes=[[24, 20], [20]], seed=22, grad_scale=1.0, steps=9,
+        lr=1e-2, betas=[0.9, 0.99], epsilon=1e-6, weight_decay=0.0, weight_decay_type="DECOUPLED",
+        max_preconditioner_dim=16, precondition_frequency=2, start_preconditioning_step=6,
+        preconditioner="eigh", override_1d=True, grafting="adagrad", grafting_epsilon=1e-8,
+        averaging="schedule_free", train_interp_coeff=0.7, eval_coeff_lr_power=2, toggle_eval_at=7,
+        lr_schedule=[1e-2, 2e-2, 3e-2, 3e-2, 2.5e-2, 2e-2, 1e-2, 5e-3, 2e-3],
+    ),
     "cfg1_override": dict(  # benchmark configuration 1 with 1-D blocks left to grafting
         shapes=[[512, 512], [512]], seed=0, grad_scale=1.0, steps=10, zero_init=True, torch_seed_grads=True,
         lr=1e-3, betas=[0.9, 0.999], epsilon=1e-12, weight_decay=0.0, weight_decay_type="DECOUPLED",
@@ -268,6 +290,12 @@ def build_reference(c, params):
         if c.get("momentum", 0.0) != 0.0
         else None
     )
+    if c.get("averaging") == "gpa":
+        mom = GeneralizedPrimalAveragingConfig(
+            eval_interp_coeff=c["eval_interp_coeff"], train_interp_coeff=c["train_interp_coeff"]
+        )
+    elif c.get("averaging") == "schedule_free":
+        mom = ScheduleFreeConfig(train_interp_coeff=c["train_interp_coeff"], eval_coeff_lr_power=c["eval_coeff_lr_power"])
     return DistributedShampoo(
         params, lr=c["lr"], betas=tuple(c["betas"]), beta3=c.get("beta3", -1.0), epsilon=c["epsilon"],
         weight_decay=c["weight_decay"], weight_decay_type=WeightDecayType[c["weight_decay_type"]],
@@ -325,7 +353,15 @@ def run_case(name, c):
             for p, g in zip(params, grads):
                 p.grad = g
             dist_calls.clear()
+            if "lr_schedule" in c:
+                opt.param_groups[0]["lr"] = c["lr_schedule"][s - 1]
             opt.step()
+            if c.get("toggle_eval_at") == s:
+                # the evaluation sequence, then back to the training sequence
+                opt.eval()
+                for i, p in enumerate(params):
+                    out[f"eval_p{i}"] = p.detach().reshape(-1).numpy().copy()
+                opt.train()
             # torch.dist is called once before the loop and once per iteration
             iters_per_step.append([n - (2 if higher else 1) for n in dist_calls])
             for i, p in enumerate(params):

@@ -66,6 +66,8 @@ def oracle_config(c):
         grafting_epsilon=c.get("grafting_epsilon", 1e-10),
         momentum=c.get("momentum", 0.0), dampening=c.get("dampening", 0.0),
         use_nesterov=c.get("use_nesterov", False),
+        averaging=c.get("averaging"), eval_interp_coeff=c.get("eval_interp_coeff", 0.9),
+        train_interp_coeff=c.get("train_interp_coeff", 0.8), eval_coeff_lr_power=c.get("eval_coeff_lr_power", 2),
         kl=c.get("kl", False), factor_matrix_dtype=c.get("factor_matrix_dtype", "float32"),
         use_trace_scaling=c.get("use_trace_scaling", False),
         trace_scaling_exponent=c.get("trace_scaling_exponent", 0.5),

@@ -42,6 +42,10 @@ def native_optimizer(c, params):
     mom = None
     if c.get("momentum", 0.0) != 0.0:
         mom = oa.ClassicMomentumConfig(momentum=c["momentum"], dampening=c["dampening"], use_nesterov=c["use_nesterov"])
+    if c.get("averaging") == "gpa":
+        mom = oa.GeneralizedPrimalAveragingConfig(eval_interp_coeff=c["eval_interp_coeff"], train_interp_coeff=c["train_interp_coeff"])
+    elif c.get("averaging") == "schedule_free":
+        mom = oa.ScheduleFreeConfig(train_interp_coeff=c["train_interp_coeff"], eval_coeff_lr_power=c["eval_coeff_lr_power"])
     return oa.DistributedShampoo(
         params, lr=c["lr"], betas=tuple(c["betas"]), beta3=c.get("beta3", -1.0), epsilon=c["epsilon"],
         weight_decay=c["weight_decay"], weight_decay_type=oa.WeightDecayType[c["weight_decay_type"]],
@@ -379,3 +383,118 @@ def test_float64_factors_at_moderate_size(kind):
             assert rel_err(st["factor_matrices"][j].cpu(), f) < 1e-6, (k, j)
         for j, f in enumerate(ost["inv"]):
             assert rel_err(st["inv_factor_matrices"][j].cpu(), f) < 1e-3, (k, j)
+
+
+@pytest.mark.parametrize("name", ["gpa_newton", "schedule_free_eigh"])
+def test_primal_averaging_matches_oracle_and_reference_fixture(name):
+    """GeneralizedPrimalAveragingConfig / ScheduleFreeConfig: the z sequence (`weight_buffer`), the training sequence
+    in the parameters, a learning rate that changes per step (Schedule-Free: mu_x from lr^2 / sum lr^2, `lr_sum` in the
+    state), decoupled weight decay on z, and a round trip through eval() / train() whose evaluation-sequence parameters
+    are compared with the reference's."""
+    from oracle.shampoo_oracle import ShampooOracle
+
+    c = CASES[name]
+    z = load_npz(name)
+    dev = torch.device("cuda:0")
+    init = initial_params(c)
+    params = [torch.nn.Parameter(t.clone().to(dev)) for t in init]
+    opt = native_optimizer(c, params)
+    ref_params = [t.clone() for t in init]
+    ref = ShampooOracle(ref_params, oracle_config(c))
+    for s, grads in grad_stream(c):
+        if "lr_schedule" in c:
+            opt.param_groups[0]["lr"] = c["lr_schedule"][s - 1]
+            ref.cfg.lr = c["lr_schedule"][s - 1]
+        for p, g in zip(params, grads):
+            p.grad = g.to(dev)
+        opt.step()
+        ref.step([g.clone() for g in grads])
+        for p, r in zip(params, ref_params):
+            assert rel_err(p.detach().cpu(), r) < 1e-3, s
+        if c.get("toggle_eval_at") == s:
+            opt.eval()
+            with pytest.raises(RuntimeError, match="not in train mode"):
+                opt.step()
+            for i, p in enumerate(params):
+                assert rel_err(p.detach().cpu().reshape(-1), z[f"eval_p{i}"]) < 1e-3
+            opt.eval()  # a second call changes nothing
+            opt.train()
+            for p, r in zip(params, ref_params):
+                assert rel_err(p.detach().cpu(), r) < 1e-3
+    for i, p in enumerate(params):
+        assert rel_err(p.detach().cpu().reshape(-1), z[f"final_p{i}"]) < 1e-3
+    ng = opt._groups[0]
+    for k, bi in enumerate(ng.native_index):
+        spec = ng.block_specs[bi]
+        st = opt.state[params[spec.param_index]][spec.block_key]
+        assert rel_err(st["weight_buffer"].cpu(), ref.state[bi]["weight_buffer"]) < 1e-3
+    if name.startswith("schedule_free"):
+        assert float(opt.state[params[0]]["lr_sum"]) == pytest.approx(float(ref.lr_sum), rel=1e-6)
+    assert bool(opt.state[params[0]]["train_mode"])
+
+
+def test_generalized_primal_averaging_is_sgd_with_momentum():
+    """The equivalences the reference documents for GeneralizedPrimalAveragingConfig (shampoo_types.py:813-850):
+    SGD grafting only, lr / (1 - momentum), mu_x = momentum, mu_y = 1 (heavy ball) or momentum (Nesterov) gives, on the
+    evaluation sequence, torch.optim.SGD with that momentum."""
+    import math
+
+    import optimizers_amd as oa
+
+    dev = torch.device("cuda:0")
+    for nesterov in (False, True):
+        torch.manual_seed(4)
+        w0 = torch.randn(12, 10)
+        grads = [torch.randn(12, 10) for _ in range(6)]
+        a = torch.nn.Parameter(w0.clone().to(dev))
+        b = torch.nn.Parameter(w0.clone().to(dev))
+        sgd = torch.optim.SGD([a], lr=0.01, momentum=0.9, nesterov=nesterov)
+        gpa = oa.DistributedShampoo(
+            [b], lr=0.1, betas=(0.0, 1.0), epsilon=1e-10, max_preconditioner_dim=16, start_preconditioning_step=math.inf,
+            grafting_config=oa.SGDPreconditionerConfig(),
+            iterate_averaging_config=oa.GeneralizedPrimalAveragingConfig(
+                eval_interp_coeff=0.9, train_interp_coeff=0.9 if nesterov else 1.0),
+        )
+        for g in grads:
+            a.grad = g.to(dev)
+            b.grad = g.to(dev)
+            sgd.step()
+            gpa.step()
+        if not nesterov:
+            gpa.eval()  # heavy ball: torch's iterate is the evaluation sequence
+        torch.testing.assert_close(b.detach(), a.detach(), rtol=1e-4, atol=1e-5)
+
+
+def test_schedule_free_resumes_from_its_state():
+    """weight_buffer, lr_sum and train_mode travel through state_dict(): an optimizer rebuilt in the middle of the run
+    continues exactly like the original."""
+    c = CASES["schedule_free_eigh"]
+    dev = torch.device("cuda:0")
+
+    def fresh():
+        params = [torch.nn.Parameter(t.clone().to(dev)) for t in initial_params(c)]
+        return params, native_optimizer(c, params)
+
+    params_a, opt_a = fresh()
+    stream = list(grad_stream(c))
+    for s, grads in stream[:5]:
+        opt_a.param_groups[0]["lr"] = c["lr_schedule"][s - 1]
+        for p, g in zip(params_a, grads):
+            p.grad = g.to(dev)
+        opt_a.step()
+    params_b, opt_b = fresh()
+    with torch.no_grad():
+        for pa, pb in zip(params_a, params_b):
+            pb.copy_(pa)
+    opt_b.load_state_dict(opt_a.state_dict())
+    assert float(opt_b.state[params_b[0]]["lr_sum"]) == float(opt_a.state[params_a[0]]["lr_sum"]) > 0.0
+    for s, grads in stream[5:]:
+        for params, opt in ((params_a, opt_a), (params_b, opt_b)):
+            opt.param_groups[0]["lr"] = c["lr_schedule"][s - 1]
+            for p, g in zip(params, grads):
+                p.grad = g.to(dev)
+            opt.step()
+    opt_a.eval()
+    opt_b.eval()
+    for pa, pb in zip(params_a, params_b):
+        assert rel_err(pb.detach().cpu(), pa.detach().cpu()) < 1e-6

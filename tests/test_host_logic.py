@@ -23,20 +23,21 @@ def test_library_loads_and_exports_every_declared_symbol():
     for name in sorted(declared):
         assert hasattr(lib, name), f"{name} declared in include/shampoo_amd.h but not exported"
     assert set(native.EXPORTS) <= declared
-    assert lib.sa_abi_version() == 2
+    assert lib.sa_abi_version() == 3
 
 
 def test_struct_layouts_match_the_header():
     import ctypes
 
-    # sa_block_desc: 2*int32, int64, 4 pointers, 3+3 pointers, 3*int32 (+4 pad), 3+1 pointers, int32 (+4 pad), int64
-    # -> 160 bytes on LP64
-    assert ctypes.sizeof(native.BlockDesc) == 160
+    # sa_block_desc: 2*int32, int64, 4 pointers, 3+3 pointers, 3*int32 (+4 pad), 3+1 pointers, int32 (+4 pad), int64,
+    # 1 pointer -> 168 bytes on LP64
+    assert ctypes.sizeof(native.BlockDesc) == 168
     assert native.BlockDesc.ld.offset == 8 and native.BlockDesc.factor.offset == 48
     assert native.BlockDesc.inv_factor.offset == 72 and native.BlockDesc.root.offset == 96
     assert native.BlockDesc.eigenvectors.offset == 112 and native.BlockDesc.corrected_eigenvalues.offset == 136
     assert native.BlockDesc.mid.offset == 144 and native.BlockDesc.ld_outer.offset == 152
-    assert ctypes.sizeof(native.StepScalars) == 52
+    assert native.BlockDesc.weight_buffer.offset == 160
+    assert ctypes.sizeof(native.StepScalars) == 64 and native.StepScalars.use_primal_averaging.offset == 52
 
 
 def test_no_gpu_means_loud_failure_not_fallback():

@@ -22,7 +22,14 @@ def test_multi_step_matches_reference(name):
     opt = O.ShampooOracle(params, oracle_config(c))
     its = []
     for s, grads in grad_stream(c):
+        if "lr_schedule" in c:
+            opt.cfg.lr = c["lr_schedule"][s - 1]
         opt.step(grads)
+        if c.get("toggle_eval_at") == s:
+            opt.eval()
+            for i, p in enumerate(params):
+                assert rel_err(p.reshape(-1), z[f"eval_p{i}"]) < 5e-6
+            opt.train()
         its.append([i for blk in opt.last_newton_iterations for i in blk])
         for i, p in enumerate(params):
             assert p.double().norm().item() == pytest.approx(float(z[f"norm_s{s}_p{i}"]), rel=2e-6)
@@ -52,6 +59,8 @@ def test_multi_step_matches_reference(name):
                 assert rel_err(st["adagrad"], z[pre + "adagrad"]) < 2e-6
             if "filtered_grad" in st:
                 assert rel_err(st["filtered_grad"], z[pre + "filtered_grad"]) < 2e-6
+            if "weight_buffer" in st:
+                assert rel_err(st["weight_buffer"], z[pre + "weight_buffer"]) < 5e-6
             if "momentum_buffer" in st:
                 assert rel_err(st["momentum_buffer"], z[pre + "momentum_buffer"]) < 2e-5
             bi += 1
