@@ -299,6 +299,18 @@ class _NativeGroup(_AmortizedComputation):
                 raise ValueError("parameters must be contiguous (the reference views them with merged shapes)")
 
         pc = group[PRECONDITIONER_CONFIG]
+        # An element-wise method as the preconditioner itself (SGD / AdaGrad / RMSprop / Adam configs,
+        # distributed_shampoo.py:673-714: the reference then runs its AdagradPreconditionerList, or nothing for SGD, in
+        # place of a Shampoo list): the same arithmetic as grafting with that method before
+        # start_preconditioning_step, so every step takes the fused grafting-only kernel and no block has factors.
+        self.elementwise_only = isinstance(
+            pc, (SGDPreconditionerConfig, AdaGradPreconditionerConfig, RMSpropPreconditionerConfig, AdamPreconditionerConfig)
+        )
+        self.elementwise_config = pc if self.elementwise_only else None
+        if self.elementwise_only:
+            if group[GRAFTING_CONFIG] is not None:
+                raise NotImplementedError("grafting on top of an element-wise preconditioner_config is not built natively")
+            pc = RootInvShampooPreconditionerConfig(inverse_exponent_override={1: 0.0, 2: 0.0, 3: 0.0})
         self._check_supported(group, pc)
         self.preconditioner_config = pc
         dist: DistributedConfig = group[DISTRIBUTED_CONFIG]
@@ -320,7 +332,7 @@ class _NativeGroup(_AmortizedComputation):
         self.native_index = [i for i, s in enumerate(self.block_specs) if s.numel > 0]
         nb = len(self.native_index)
         beta1 = group[BETAS][0]
-        graft = group[GRAFTING_CONFIG]
+        graft = self.elementwise_config if self.elementwise_only else group[GRAFTING_CONFIG]
         self.graft_type, self.graft_beta2, self.graft_weight, self.graft_bias, self.graft_eps = self._graft_setup(graft)
         momentum_cfg = group[ITERATE_AVERAGING_CONFIG]
 
@@ -729,7 +741,7 @@ class _NativeGroup(_AmortizedComputation):
         use_bc = group[USE_BIAS_CORRECTION]
         pc = self.preconditioner_config
         amortize = (step_val % freq == 0 and step_val > start) or step_val == start
-        graft_only = step_val < start and group[GRAFTING_CONFIG] is not None
+        graft_only = (step_val < start and group[GRAFTING_CONFIG] is not None) or self.elementwise_only
 
         if weight_decay != 0.0 and wd_type == WeightDecayType.L2:
             native.check(lib.sa_add_l2_regularization(self.plan, weight_decay, stream), "sa_add_l2_regularization")
@@ -827,6 +839,7 @@ class DistributedShampoo(torch.optim.Optimizer):
     `EigenvalueCorrectedShampooPreconditionerConfig` and `EigendecomposedShampooPreconditionerConfig` with
     `QREigendecompositionConfig` or `EighEigendecompositionConfig` (including `ignored_basis_change_dims`), grafting with SGD / AdaGrad / RMSprop /
     Adam or none, every `WeightDecayType`, `ClassicMomentumConfig`, `GeneralizedPrimalAveragingConfig`, `ScheduleFreeConfig`, `inverse_exponent_override`,
+    an SGD / AdaGrad / RMSprop / Adam config as `preconditioner_config` itself,
     `SingleDeviceDistributedConfig`, fp32 state with packed factor matrices (`factor_matrix_dtype=torch.float64` for
     root-inverse Shampoo: fp64 factor averages and an fp64 coupled Newton root inverse), blocks of order 1 to 3 (order 3: what is left of
     convolution weights).

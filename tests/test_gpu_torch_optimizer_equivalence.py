@@ -135,3 +135,38 @@ def test_sgd_momentum_through_classic_momentum(nesterov):
                      iterate_averaging_config=oa.ClassicMomentumConfig(momentum=0.5, use_nesterov=nesterov),
                      preconditioner_config=oa.DefaultShampooConfig),
              dims=(10, 10))
+
+
+@pytest.mark.parametrize("weight_decay", (0.0, 0.3))
+def test_elementwise_methods_as_the_preconditioner_itself(weight_decay):
+    """`preconditioner_config=AdamPreconditionerConfig(...)` etc. without grafting (distributed_shampoo.py:673-714: the
+    reference then runs its Adagrad list in place of a Shampoo list) is the torch optimizer of that name."""
+    import optimizers_amd as oa
+
+    common = dict(max_preconditioner_dim=10, precondition_frequency=1, start_preconditioning_step=1, weight_decay=weight_decay)
+    _compare(partial(Adam, lr=0.001, betas=(0.9, 0.999), weight_decay=weight_decay, eps=1e-8),
+             lambda ps: oa.DistributedShampoo(ps, lr=0.001, betas=(0.9, 0.999), epsilon=1e-8, weight_decay_type=oa.WeightDecayType.L2,
+                                              preconditioner_config=oa.AdamPreconditionerConfig(beta2=0.999, epsilon=1e-8), **common))
+    _compare(partial(AdamW, lr=0.001, betas=(0.9, 0.999), weight_decay=weight_decay, eps=1e-8),
+             lambda ps: oa.DistributedShampoo(ps, lr=0.001, betas=(0.9, 0.999), epsilon=1e-8, weight_decay_type=oa.WeightDecayType.DECOUPLED,
+                                              preconditioner_config=oa.AdamPreconditionerConfig(beta2=0.999, epsilon=1e-8), **common))
+    _compare(partial(Adagrad, lr=0.01, weight_decay=weight_decay, eps=1e-10),
+             lambda ps: oa.DistributedShampoo(ps, lr=0.01, betas=(0.0, 1.0), epsilon=1e-10, weight_decay_type=oa.WeightDecayType.L2,
+                                              preconditioner_config=oa.AdaGradPreconditionerConfig(epsilon=1e-10), **common))
+    _compare(partial(RMSprop, lr=0.01, weight_decay=weight_decay, alpha=0.99, eps=1e-8),
+             lambda ps: oa.DistributedShampoo(ps, lr=0.01, betas=(0.0, 0.99), epsilon=1e-8, use_bias_correction=False,
+                                              weight_decay_type=oa.WeightDecayType.L2,
+                                              preconditioner_config=oa.RMSpropPreconditionerConfig(beta2=0.99, epsilon=1e-8), **common))
+    _compare(partial(SGD, lr=0.1, weight_decay=weight_decay),
+             lambda ps: oa.DistributedShampoo(ps, lr=0.1, betas=(0.0, 1.0), epsilon=1e-10, weight_decay_type=oa.WeightDecayType.L2,
+                                              preconditioner_config=oa.SGDPreconditionerConfig(), **common),
+             dims=(10, 10))
+
+
+def test_grafting_on_an_elementwise_preconditioner_is_rejected():
+    import optimizers_amd as oa
+
+    p = torch.nn.Parameter(torch.zeros(4, 4, device=DEV))
+    with pytest.raises(NotImplementedError, match="element-wise preconditioner_config"):
+        oa.DistributedShampoo([p], preconditioner_config=oa.AdamPreconditionerConfig(),
+                              grafting_config=oa.SGDPreconditionerConfig())
