@@ -545,6 +545,7 @@ class _NativeGroup(_AmortizedComputation):
         if self.primal_averaging:
             # per-group scalars aliased under every parameter (distributed_shampoo.py:924-937)
             self.lr_sum = torch.tensor(0.0, dtype=torch.float, device=self.device)
+            self._lr_sum_host = torch.tensor(0.0, dtype=torch.float)
             self.train_mode = torch.tensor(True, dtype=torch.bool, device="cpu")
             for p in params:
                 optimizer.state[p][TRAIN_MODE] = self.train_mode
@@ -701,9 +702,10 @@ class _NativeGroup(_AmortizedComputation):
             logger.warning("lr or lr_sum not provided to _get_train_and_eval_interp_coeffs; returning eval_interp_coeff = 0.0!")
             return train, torch.tensor(0.0, dtype=torch.float32)
         lr_power = torch.pow(lr, cfg.eval_coeff_lr_power)
-        lr_sum = self.lr_sum.cpu() + lr_power
-        self.lr_sum.copy_(lr_sum)
-        return train, 1.0 - lr_power / lr_sum
+        # the sum is kept on the host and mirrored into the state tensor, so that no step waits for the device
+        self._lr_sum_host = self._lr_sum_host + lr_power
+        self.lr_sum.copy_(self._lr_sum_host, non_blocking=True)
+        return train, 1.0 - lr_power / self._lr_sum_host
 
     def switch_mode(self, group: dict[str, Any], train: bool) -> None:
         """train(): y = x + (1 - mu_y)(z - x); eval(): x = y + (1 - 1/mu_y)(z - y), on every block
@@ -1037,6 +1039,7 @@ def _restore_state(self: _NativeGroup, optimizer: DistributedShampoo) -> None:
                 mine.copy_(torch.as_tensor(loaded[0]).to(device=mine.device, dtype=mine.dtype))
             for p in self.params:
                 optimizer.state[p][key] = mine
+        self._lr_sum_host = self.lr_sum.detach().cpu().clone()
     if self.plan:
         native.check(self.lib.sa_plan_invalidate_inverse_cache(self.plan), "sa_plan_invalidate_inverse_cache")
     # eigendecomposed Shampoo: the inverse roots are a function of the restored (Q, lambda)
