@@ -247,6 +247,10 @@ def cpu_baseline(workload: dict, name: str, budget_s: float = 25.0) -> dict:
     }
 
 
+def kind_of(workload: dict) -> str:
+    return workload.get("preconditioner", "newton")
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -308,6 +312,21 @@ def main() -> None:
         torch.cuda.synchronize()
         del src, dst
 
+    # what one Newton iteration of each factor costs with the reference's full products: 2 d^3 per product,
+    # 2 + (products of the square-and-multiply chain for M_p^root) products per iteration
+    ng = opt._groups[0]
+    full_product_flops_per_iteration = []
+    for k, i in enumerate(ng.native_index):
+        spec = ng.block_specs[i]
+        slot = 0
+        for dim in range(spec.order):
+            if ng.selectors[k][dim]:
+                root = int(round(ng.roots[k][slot]))
+                chain = (root.bit_length() - 1) + (bin(root).count("1") - 1)
+                full_product_flops_per_iteration.append(2.0 * spec.shape[dim] ** 3 * (2 + chain))
+                slot += 1
+    full_product_flops = 0.0
+
     lib.sa_set_profiling(1)
     phases = ("newton_gemm", "syrk", "precondition_gemm", "grafting", "apply", "jacobi", "qr_refresh", "eigenbasis_rotation",
               "tridiagonalize", "form_q", "tridiagonal_ql")
@@ -326,6 +345,8 @@ def main() -> None:
                 acc[ph][2] += lib.sa_phase_launches(ph.encode())
         executed += max(lib.sa_phase_executed_flops(b"newton_gemm"), 0.0)
         iters.append(list(opt._groups[0].last_newton_iterations))
+        if kind_of(workload) == "newton":
+            full_product_flops += sum(it * w for it, w in zip(iters[-1], full_product_flops_per_iteration))
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     lib.sa_set_profiling(0)
@@ -354,6 +375,11 @@ def main() -> None:
         # d^2 (d + 1) for a symmetric one); `executed_frac` adds the padding and the mirrored halves of
         # diagonal tiles, i.e. what the matrix cores really sustained.
         "symmetric_products_policy": args.symmetric_newton,
+        # the same iterations billed as the reference's full products (2 d^3 each); above `executed_frac` because a
+        # symmetric product computes only the tiles on and above the diagonal
+        "full_product_TFLOP/s": full_product_flops / (ng_ms * 1e-3) / 1e12 if (ng_ms > 0 and dominant == "newton_gemm") else None,
+        "full_product_frac": (full_product_flops / (ng_ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS
+                              if (ng_ms > 0 and dominant == "newton_gemm") else None),
         "executed_TFLOP/s": executed / (ng_ms * 1e-3) / 1e12 if ng_ms > 0 else 0.0,
         "executed_frac": executed / (ng_ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS if ng_ms > 0 else 0.0,
         "avg_launch_ms": ng_ms / max(ng_launches, 1),
@@ -407,7 +433,7 @@ def main() -> None:
     }
     if not args.no_cpu_baseline:
         # the native optimizer's state is released first: the oracle keeps dense factors and inverse roots of its own
-        del opt, params, grads
+        del opt, params, grads, ng
         torch.cuda.empty_cache()
         out["torch_gpu_baseline"] = torch_gpu_baseline(workload, args.workload, device)
         torch.cuda.empty_cache()
