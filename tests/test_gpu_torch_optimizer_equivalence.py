@@ -59,7 +59,8 @@ def _compare(control, experimental, dims=(10, 1, 1)):
 def _configs():
     import optimizers_amd as oa
 
-    return (oa.DefaultShampooConfig, oa.DefaultEigenvalueCorrectedShampooConfig, oa.DefaultSOAPConfig)
+    return (oa.DefaultShampooConfig, oa.DefaultEigenvalueCorrectedShampooConfig, oa.DefaultSOAPConfig,
+            oa.EigendecomposedShampooPreconditionerConfig())
 
 
 def _shampoo(params, **kw):
@@ -70,7 +71,7 @@ def _shampoo(params, **kw):
                                  start_preconditioning_step=math.inf, **kw)
 
 
-@pytest.mark.parametrize("which", range(3))
+@pytest.mark.parametrize("which", range(4))
 @pytest.mark.parametrize("weight_decay", (0.0, 0.3))
 def test_adagrad_grafting(weight_decay, which):
     import optimizers_amd as oa
@@ -80,7 +81,7 @@ def test_adagrad_grafting(weight_decay, which):
                      grafting_config=oa.AdaGradPreconditionerConfig(epsilon=1e-10), preconditioner_config=_configs()[which]))
 
 
-@pytest.mark.parametrize("which", range(3))
+@pytest.mark.parametrize("which", range(4))
 @pytest.mark.parametrize("weight_decay", (0.0, 0.3))
 def test_adam_grafting(weight_decay, which):
     import optimizers_amd as oa
@@ -91,7 +92,7 @@ def test_adam_grafting(weight_decay, which):
                      preconditioner_config=_configs()[which]))
 
 
-@pytest.mark.parametrize("which", range(3))
+@pytest.mark.parametrize("which", range(4))
 @pytest.mark.parametrize("weight_decay", (0.0, 0.3))
 def test_adamw_grafting(weight_decay, which):
     import optimizers_amd as oa
@@ -102,7 +103,7 @@ def test_adamw_grafting(weight_decay, which):
                      preconditioner_config=_configs()[which]))
 
 
-@pytest.mark.parametrize("which", range(3))
+@pytest.mark.parametrize("which", range(4))
 @pytest.mark.parametrize("weight_decay", (0.0, 0.3))
 def test_rmsprop_grafting(weight_decay, which):
     import optimizers_amd as oa
@@ -113,7 +114,7 @@ def test_rmsprop_grafting(weight_decay, which):
                      preconditioner_config=_configs()[which]))
 
 
-@pytest.mark.parametrize("which", range(3))
+@pytest.mark.parametrize("which", range(4))
 @pytest.mark.parametrize("weight_decay", (0.0, 0.3))
 def test_sgd_grafting(weight_decay, which):
     import optimizers_amd as oa
@@ -134,6 +135,65 @@ def test_sgd_momentum_through_classic_momentum(nesterov):
                      grafting_config=oa.SGDPreconditionerConfig(),
                      iterate_averaging_config=oa.ClassicMomentumConfig(momentum=0.5, use_nesterov=nesterov),
                      preconditioner_config=oa.DefaultShampooConfig),
+             dims=(10, 10))
+
+
+@pytest.mark.parametrize("which", range(4))
+@pytest.mark.parametrize("weight_decay", (0.0, 0.3))
+def test_corrected_weight_decay(weight_decay, which):
+    """gpu_tests/weight_decay_test.py:170-217: at a constant learning rate (lr == peak_lr) the corrected decay
+    params *= 1 - lr * (lr / peak_lr) * weight_decay is AdamW's."""
+    import optimizers_amd as oa
+
+    _compare(partial(AdamW, lr=0.001, betas=(0.9, 0.999), weight_decay=weight_decay, eps=1e-8),
+             partial(_shampoo, lr=0.001, betas=(0.9, 0.999), weight_decay=weight_decay, epsilon=1e-8,
+                     weight_decay_type="CORRECTED", grafting_config=oa.AdamPreconditionerConfig(beta2=0.999, epsilon=1e-8),
+                     preconditioner_config=_configs()[which]))
+
+
+@pytest.mark.parametrize("which", range(4))
+@pytest.mark.parametrize("weight_decay", (0.0, 0.3))
+def test_independent_weight_decay(weight_decay, which):
+    """gpu_tests/weight_decay_test.py:219-270: the independent decay params *= 1 - (lr / peak_lr) * weight_decay is,
+    at a constant learning rate, AdamW with weight_decay / lr."""
+    import optimizers_amd as oa
+
+    lr = 0.001
+    _compare(partial(AdamW, lr=lr, betas=(0.9, 0.999), weight_decay=weight_decay / lr, eps=1e-8),
+             partial(_shampoo, lr=lr, betas=(0.9, 0.999), weight_decay=weight_decay, epsilon=1e-8,
+                     weight_decay_type="INDEPENDENT", grafting_config=oa.AdamPreconditionerConfig(beta2=0.999, epsilon=1e-8),
+                     preconditioner_config=_configs()[which]))
+
+
+def test_generalized_primal_averaging_is_heavy_ball_momentum():
+    """gpu_tests/iterate_averaging_test.py:80-144: with the gradient taken at the averaged iterate itself
+    (train_interp_coeff = 1) and eval_interp_coeff = momentum, primal averaging over plain SGD at lr / (1 - momentum)
+    is torch's SGD with heavy-ball momentum."""
+    import optimizers_amd as oa
+
+    lr, momentum = 0.1, 0.9
+    _compare(partial(SGD, lr=lr, momentum=momentum, weight_decay=0.0),
+             lambda ps: oa.DistributedShampoo(
+                 ps, lr=lr / (1 - momentum), betas=(0.0, 1.0), epsilon=1e-10, weight_decay=0.0, max_preconditioner_dim=10,
+                 precondition_frequency=1, start_preconditioning_step=-1, weight_decay_type=oa.WeightDecayType.L2,
+                 preconditioner_config=oa.SGDPreconditionerConfig(), grafting_config=None,
+                 iterate_averaging_config=oa.GeneralizedPrimalAveragingConfig(eval_interp_coeff=momentum,
+                                                                              train_interp_coeff=1.0)),
+             dims=(10, 10))
+
+
+@pytest.mark.parametrize("nesterov", (False, True))
+def test_classic_momentum_over_the_sgd_preconditioner(nesterov):
+    """gpu_tests/iterate_averaging_test.py:265-305: ClassicMomentumConfig with dampening 0 over
+    `preconditioner_config=SGDPreconditionerConfig()` is torch's SGD momentum."""
+    import optimizers_amd as oa
+
+    _compare(partial(SGD, lr=0.01, weight_decay=0.0, momentum=0.9, dampening=0.0, nesterov=nesterov),
+             lambda ps: oa.DistributedShampoo(
+                 ps, lr=0.01, betas=(0.0, 1.0), epsilon=1e-10, weight_decay=0.0, max_preconditioner_dim=10,
+                 precondition_frequency=1, start_preconditioning_step=-1, weight_decay_type=oa.WeightDecayType.L2,
+                 preconditioner_config=oa.SGDPreconditionerConfig(), grafting_config=None,
+                 iterate_averaging_config=oa.ClassicMomentumConfig(momentum=0.9, dampening=0.0, use_nesterov=nesterov)),
              dims=(10, 10))
 
 
