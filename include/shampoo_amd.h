@@ -126,7 +126,8 @@ int32_t sa_plan_bind_workspace(sa_plan* plan, void* workspace, int64_t bytes);
 /* Number of factor matrices, in block order then dim order (the order of every per-factor array). */
 int32_t sa_plan_num_factors(const sa_plan* plan);
 
-/* Marks the dense inverse cache stale (after the caller wrote inv_factor itself, e.g. load_state_dict). */
+/* Marks what the plan derives from the optimizer state stale: the dense inverse cache and the filtered gradient kept
+ * in the eigenbasis (after the caller wrote inv_factor, eigenvectors or filtered_grad itself, e.g. load_state_dict). */
 int32_t sa_plan_invalidate_inverse_cache(sa_plan* plan);
 
 /* Gradients of this step, one device pointer per block (same rows/cols/ld as the block); NULL
@@ -245,6 +246,23 @@ int32_t sa_update_corrected_eigenvalues(sa_plan* plan, float beta2, float weight
  * workspace plus its squared norm per block (shampoo_preconditioner_list.py:1914-1942). */
 int32_t sa_precondition_eigenvalue_corrected(sa_plan* plan, const sa_step_scalars* s, float bias_correction2,
                                              float epsilon, float root, void* stream);
+
+/* sa_update_corrected_eigenvalues followed by sa_precondition_eigenvalue_corrected on the bound gradients, for the
+ * step as the reference runs it (shampoo_preconditioner_list.py:1891-1942 within distributed_shampoo.py:1162-1270:
+ * the eigenbases do not change between the two).  Call it after sa_update_grafting_and_filtered_grad of the same step.
+ * The rotation is linear, so Q_L^T Ghat Q_R need not be formed by two more products: with beta1 = 0 it is the
+ * rotated gradient of the statistic, and otherwise the plan keeps Q_L^T m Q_R and advances it by m's own moving
+ * average inside the statistic's launch (blocks of order 2 with both eigenbases; the copy is rebuilt by the next
+ * full preconditioning after a refresh, a workspace bind, sa_plan_invalidate_inverse_cache or a change of the masked
+ * blocks).  Results equal the two separate calls up to fp32 rounding of the reordered sums.  beta3 != beta1 is
+ * rejected with SA_ERR_UNSUPPORTED: make the two separate calls, the first one before the prologue. */
+int32_t sa_update_and_precondition_eigenvalue_corrected(sa_plan* plan, const sa_step_scalars* s, float beta2,
+                                                        float weighting_factor, float bias_correction2, float epsilon,
+                                                        float root, void* stream);
+
+/* How many calls of sa_update_and_precondition_eigenvalue_corrected shared the rotation (the others fell back to the
+ * two separate routines and rebuilt the rotated copy).  No counterpart in the reference; for tests and tuning. */
+int64_t sa_plan_shared_rotation_steps(const sa_plan* plan);
 
 /* Grafting second moment, filtered gradient and the grafted direction's squared norm per block
  * (adagrad_preconditioner_list.py:122-162, distributed_shampoo.py:1162-1199, 1110-1114). */

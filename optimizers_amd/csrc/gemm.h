@@ -45,6 +45,8 @@ enum Epilogue {
   EPI_DIVPOW = 5,       // C = acc / ((C2 / div)^pow_exp + eps)   (C2 has the layout of C)
   EPI_SUB = 6,          // C -= acc                         (block-reflector updates of the QR refresh)
   EPI_HORNER = 7,       // C = alpha*acc + beta*C2 + mp_diag*I over d x d (C2 read only; Horner step of a matrix polynomial)
+  EPI_EC_FUSED = 9,     // acc = gradient in the eigenbasis: C = beta*C + alpha*acc^2 (second moment), C2 = lerp(C2, acc, mom_w)
+                        // (filtered gradient in the eigenbasis, optional), C3 = (C2 / mom_div) / ((C / div)^pow_exp + eps)
   EPI_SYRK_EMA64 = 8,   // EPI_SYRK_EMA on a packed triangle of doubles: C = beta64*C + alpha64*acc (fp32 product, fp64 average)
 };
 
@@ -53,6 +55,7 @@ struct GemmProblem {
   const float* B;
   float* C;
   float* C2;               // EPI_NEWTON_M: M_p output.  EPI_STORE_SQNORM: per-tile partial sums.  EPI_HORNER: addend (read)
+  float* C3;               // EPI_EC_FUSED: preconditioned output.  EPI_DIVPOW: optional copy of acc * mom_div
   unsigned int* err_bits;  // EPI_NEWTON_M: atomicMax target (bit pattern of a non-negative float)
   const int* active;       // optional: skip the problem when *active == 0
   long long lda, ldb, ldc;
@@ -68,7 +71,8 @@ struct GemmScalars {
   float a_div, b_div;      // operand is divided by this on load (1.0f = as stored)
   float alpha, beta;       // EPI_SYRK_EMA: C = beta*C + alpha*acc.  EPI_HORNER: C = alpha*acc + beta*C2 + mp_diag*I
   float mp_scale, mp_diag; // EPI_NEWTON_M: M_p = M*mp_scale + mp_diag*I
-  float div, pow_exp, eps; // EPI_DIVPOW
+  float div, pow_exp, eps; // EPI_DIVPOW, EPI_EC_FUSED
+  float mom_w, mom_div;    // EPI_EC_FUSED: C2 <- lerp(C2, acc, mom_w), numerator C2 / mom_div.  EPI_DIVPOW: C3 = acc * mom_div
   double alpha64, beta64;  // EPI_SYRK_EMA64
 };
 
@@ -338,6 +342,24 @@ __global__ __launch_bounds__(GEMM_THREADS) void grouped_gemm_kernel(
             const float x = P.C2[o] / sc.div;
             const float r = (sc.pow_exp == 0.5f) ? sqrtf(x) : powf(x, sc.pow_exp);
             C[o] = v / (r + sc.eps);
+            if (P.C3) P.C3[o] = v * sc.mom_div;
+          }
+        } else if (EPI == EPI_EC_FUSED) {
+          if (!EDGE || (row < M && col < N)) {
+            const long long o = (long long)row * ldc + col;
+            const float sq = __fadd_rn(__fmul_rn(C[o], sc.beta), __fmul_rn(__fmul_rn(sc.alpha, v), v));
+            C[o] = sq;
+            float num = v;
+            if (P.C2) {
+              // torch.lerp(m, g, w): m + w (g - m) for w < 0.5, g - (g - m)(1 - w) otherwise
+              const float m0 = P.C2[o];
+              const float m1 = sc.mom_w < 0.5f ? m0 + sc.mom_w * (v - m0) : v - (v - m0) * (1.0f - sc.mom_w);
+              P.C2[o] = m1;
+              num = m1 / sc.mom_div;
+            }
+            const float x = sq / sc.div;
+            const float r = (sc.pow_exp == 0.5f) ? sqrtf(x) : powf(x, sc.pow_exp);
+            P.C3[o] = num / (r + sc.eps);
           }
         } else if (EPI == EPI_SUB) {
           if (!EDGE || (row < M && col < N)) {

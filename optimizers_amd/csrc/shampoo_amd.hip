@@ -155,7 +155,7 @@ int launch_gemm_auto(const GemmTable& g, GemmScalars sc, hipStream_t s) {
   return g.aligned ? launch_gemm<AL, BL, EPI, false>(g, sc, s) : launch_gemm<AL, BL, EPI, true>(g, sc, s);
 }
 
-GemmScalars unit_scalars() { return GemmScalars{1.0f, 1.0f, 1.0f, 0.0f, 0.0f, 0.0f, 1.0f, 1.0f, 0.0f, 1.0, 0.0}; }
+GemmScalars unit_scalars() { return GemmScalars{1.0f, 1.0f, 1.0f, 0.0f, 0.0f, 0.0f, 1.0f, 1.0f, 0.0f, 0.0f, 1.0f, 1.0, 0.0}; }
 
 // ---- phase timing -------------------------------------------------------------------------
 struct Phase {
@@ -297,6 +297,13 @@ struct sa_plan {
   Table<SortJob> t_sort;
   bool eigenvalue_corrected = false;  // blocks carry a second moment in the eigenbasis (corrected_eigenvalues)
   bool has_eigvec = false;            // some factor stores its eigenvectors (eigenvalue-corrected or eigendecomposed Shampoo)
+  // Eigenvalue-corrected blocks of order 2 with both eigenbases keep Q_L^T m Q_R, the filtered gradient in the eigenbasis,
+  // next to m itself.  While the bases stand still it follows m by the same moving average (the rotation is linear), which
+  // saves rotating m on every step.  It belongs to the filtered gradient after `rotm_version` prologues; -1 = not valid.
+  long long off_rotm = 0;
+  long long m_version = 0, rotm_version = -1;
+  long long shared_rotation_steps = 0;  // steps that took the shared-rotation path
+  std::vector<char> rotm_active;        // which blocks were active when the copy was last known to be consistent
   int n_active_blocks = 0;
 
   // Newton control state (device) and pinned readback
@@ -340,6 +347,7 @@ void compute_layout(sa_plan* p) {
   p->off_norm_partial = take(p->norm_partials_total);
   p->scratch_floats = std::max((p->factor_f64 ? 16LL : 8LL) * p->dense_total, 4LL * round_up(p->total_elems, 64) + 256);
   p->off_scratch = take(p->scratch_floats);
+  p->off_rotm = take(p->eigenvalue_corrected ? p->total_elems : 0);
   p->ws_needed = o * (long long)sizeof(float);
 }
 
@@ -619,9 +627,14 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
       float* Pb = pbuf(p) + eo;
       if (f0 >= 0 && f1 >= 0) {
         p->ec_stat1.add(mk(QL, d.rows, G, d.ld, T, nullptr, d.rows), false);                       // T = QL^T G   (A_KM)
-        p->ec_stat2.add(mk(T, d.cols, QR, d.cols, d.corrected_eigenvalues, nullptr, d.cols), false);  // corr <- EMA (T QR)^2
+        // corr <- EMA (T QR)^2; the fused form of the step also advances the rotated filtered gradient and writes T2
+        GemmProblem st2 = mk(T, d.cols, QR, d.cols, d.corrected_eigenvalues, mode == 1 ? p->f(p->off_rotm) + eo : nullptr, d.cols);
+        st2.C3 = T2;
+        p->ec_stat2.add(st2, false);
         p->ec_p1.add(mk(QL, d.rows, B.ghat_src, B.ghat_ld, T, nullptr, d.rows), false);             // T = QL^T Ghat (b_div)
-        p->ec_p2.add(mk(T, d.cols, QR, d.cols, T2, d.corrected_eigenvalues, d.cols), false);         // T2 = (T QR)/den
+        GemmProblem p2 = mk(T, d.cols, QR, d.cols, T2, d.corrected_eigenvalues, d.cols);             // T2 = (T QR)/den
+        if (mode == 1) p2.C3 = p->f(p->off_rotm) + eo;  // and Q_L^T m Q_R itself
+        p->ec_p2.add(p2, false);
         p->ec_p3.add(mk(QL, d.rows, T2, d.cols, T, nullptr, d.rows), false);                         // T = QL T2
         p->ec_p4.add(mk(T, d.cols, QR, d.cols, Pb, part, d.cols), false);                            // P = T QR^T (B_NK)
       } else if (f0 >= 0) {
@@ -734,6 +747,12 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
   for (auto& a : p->g3) for (auto& b2 : a) for (auto& g : b2) SACHECK(g.commit(s));
   if (p->has_order3) SACHECK(p->t_blocks.upload(s));  // ptile ranges of order-3 blocks were set above
   p->tables_valid = true;
+  // new gradient pointers alone leave the rotated filtered gradient valid; a block that joins or leaves does not (its
+  // filtered gradient stood still while the version counter ran on), and neither does another source of Ghat
+  std::vector<char> now(nb, 0);
+  for (int b : active) now[b] = 1;
+  if (now != p->rotm_active || mode != p->table_mode) p->rotm_version = -1;
+  p->rotm_active.swap(now);
   p->table_mode = mode;
   return SA_OK;
 }
@@ -1061,14 +1080,18 @@ int32_t sa_plan_bind_workspace(sa_plan* p, void* workspace, int64_t bytes) {
   p->ws_bytes = bytes;
   p->inv_cache_valid = false;
   p->tables_valid = false;
+  p->rotm_version = -1;
   return SA_OK;
 }
 
 int32_t sa_plan_num_factors(const sa_plan* p) { return p ? (int32_t)p->factors.size() : 0; }
 
+int64_t sa_plan_shared_rotation_steps(const sa_plan* p) { return p ? p->shared_rotation_steps : 0; }
+
 int32_t sa_plan_invalidate_inverse_cache(sa_plan* p) {
   if (!p) return fail(SA_ERR_INVALID, "NULL plan");
   p->inv_cache_valid = false;
+  p->rotm_version = -1;
   return SA_OK;
 }
 
@@ -1156,6 +1179,7 @@ int32_t sa_update_grafting_and_filtered_grad(sa_plan* p, const sa_step_scalars* 
   hipLaunchKernelGGL((grafting_kernel<0>), dim3((unsigned)p->t_chunks.n), dim3(EW_THREADS), 0, s, p->t_blocks.dev,
                      p->t_chunks.dev, *sc, p->f(p->off_graft_partial), p->f(p->off_ghat_partial));
   HIPCHECK(hipGetLastError());
+  ++p->m_version;
   return SA_OK;
 }
 
@@ -1169,6 +1193,7 @@ int32_t sa_grafting_only_step(sa_plan* p, const sa_step_scalars* sc, void* strea
   hipLaunchKernelGGL((grafting_kernel<1>), dim3((unsigned)p->t_chunks.n), dim3(EW_THREADS), 0, s, p->t_blocks.dev,
                      p->t_chunks.dev, *sc, p->f(p->off_graft_partial), p->f(p->off_ghat_partial));
   HIPCHECK(hipGetLastError());
+  ++p->m_version;
   return SA_OK;
 }
 
@@ -2684,6 +2709,7 @@ int32_t sa_refresh_eigenbases_eigh(sa_plan* p, float bias_correction2, float eps
   const int F = (int)p->factors.size();
   if (F == 0) return SA_OK;
   p->eig_source.assign(F, sa_plan::EigSource{});
+  p->rotm_version = -1;  // the eigenbases change
   std::vector<int> todo;
   SACHECK(root_inverse_prologue(p, bias_correction2, epsilon, sweeps_out, status_out, s, &todo));
   if (todo.empty()) return SA_OK;
@@ -2946,27 +2972,29 @@ int32_t sa_update_corrected_eigenvalues(sa_plan* p, float beta2, float weighting
   return SA_OK;
 }
 
-int32_t sa_precondition_eigenvalue_corrected(sa_plan* p, const sa_step_scalars* sc, float bias_correction2, float epsilon,
-                                             float root, void* stream) {
-  if (!p) return fail(SA_ERR_INVALID, "NULL plan");
-  if (!p->eigenvalue_corrected) return fail(SA_ERR_STATE, "plan has no eigenvector state");
-  if (!(root > 0.0f) || !(bias_correction2 != 0.0f)) return fail(SA_ERR_INVALID, "bad root or bias correction");
-  SACHECK(validate_scalars(p, sc));
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  SACHECK(ensure_tables(p, sc, s));
+// Preconditioning of eigenvalue-corrected blocks.  rotated_ready: the blocks with both eigenbases already hold their
+// divided, rotated filtered gradient (the fused statistic launch wrote it), so only the rotation back is left for them.
+static int precondition_eigenvalue_corrected(sa_plan* p, const sa_step_scalars* sc, float bias_correction2, float epsilon,
+                                             float root, bool rotated_ready, hipStream_t s) {
   double flops = 0.0;
-  for (const GemmTable* g : {&p->ec_p1, &p->ec_p1d, &p->ec_p2, &p->ec_p2d, &p->ec_p3, &p->ec_p3n, &p->ec_p4, &p->ec_p4n})
+  for (const GemmTable* g : {&p->ec_p1, &p->ec_p1d, &p->ec_p2, &p->ec_p2d, &p->ec_p3, &p->ec_p3n, &p->ec_p4, &p->ec_p4n}) {
+    if (rotated_ready && (g == &p->ec_p1 || g == &p->ec_p2)) continue;
     for (const GemmProblem& q : g->build) flops += 2.0 * q.M * q.N * q.K;
+  }
   {
-    Span span("precondition_gemm", s, flops, 8, true);
+    Span span("precondition_gemm", s, flops, rotated_ready ? 6 : 8, true);
     GemmScalars u = unit_scalars();
     GemmScalars bdiv = u; bdiv.b_div = sc->bias_correction1;
     GemmScalars den = u; den.div = bias_correction2; den.pow_exp = 1.0f / root; den.eps = epsilon;
     GemmScalars den_b = den; den_b.b_div = sc->bias_correction1;
     GemmScalars den_a = den; den_a.a_div = sc->bias_correction1;
-    SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_STORE>(p->ec_p1, bdiv, s)));
+    GemmScalars den_seed = den; den_seed.mom_div = sc->bias_correction1;  // the product is Q_L^T (m / bc1) Q_R
+    if (!rotated_ready) {
+      SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_STORE>(p->ec_p1, bdiv, s)));
+      SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_DIVPOW>(p->ec_p2, den_seed, s)));
+      if (p->table_mode == 1) p->rotm_version = p->m_version;
+    }
     SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_DIVPOW>(p->ec_p1d, den_b, s)));
-    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_DIVPOW>(p->ec_p2, den, s)));
     SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_DIVPOW>(p->ec_p2d, den_a, s)));
     SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE>(p->ec_p3, u, s)));
     SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE_SQNORM>(p->ec_p3n, u, s)));
@@ -2988,6 +3016,62 @@ int32_t sa_precondition_eigenvalue_corrected(sa_plan* p, const sa_step_scalars* 
     HIPCHECK(hipGetLastError());
   }
   return SA_OK;
+}
+
+int32_t sa_precondition_eigenvalue_corrected(sa_plan* p, const sa_step_scalars* sc, float bias_correction2, float epsilon,
+                                             float root, void* stream) {
+  if (!p) return fail(SA_ERR_INVALID, "NULL plan");
+  if (!p->eigenvalue_corrected) return fail(SA_ERR_STATE, "plan has no eigenvector state");
+  if (!(root > 0.0f) || !(bias_correction2 != 0.0f)) return fail(SA_ERR_INVALID, "bad root or bias correction");
+  SACHECK(validate_scalars(p, sc));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SACHECK(ensure_tables(p, sc, s));
+  return precondition_eigenvalue_corrected(p, sc, bias_correction2, epsilon, root, false, s);
+}
+
+int32_t sa_update_and_precondition_eigenvalue_corrected(sa_plan* p, const sa_step_scalars* sc, float beta2, float weighting_factor,
+                                                        float bias_correction2, float epsilon, float root, void* stream) {
+  if (!p) return fail(SA_ERR_INVALID, "NULL plan");
+  if (!p->eigenvalue_corrected) return fail(SA_ERR_STATE, "plan has no eigenvector state");
+  if (!(root > 0.0f) || !(bias_correction2 != 0.0f)) return fail(SA_ERR_INVALID, "bad root or bias correction");
+  SACHECK(validate_scalars(p, sc));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SACHECK(ensure_tables(p, sc, s));
+  if (p->table_mode == 2)
+    return fail(SA_ERR_UNSUPPORTED, "beta3 != beta1: call sa_update_corrected_eigenvalues before the prologue and "
+                                    "sa_precondition_eigenvalue_corrected after it");
+  // The rotated gradient of the statistic is also what the filtered gradient needs: with beta1 = 0 it is the
+  // numerator itself, otherwise Q_L^T m Q_R follows it by m's own moving average as long as the stored copy belongs to
+  // the filtered gradient of the previous step in these bases.
+  const bool fused = p->table_mode == 0 || (p->table_mode == 1 && p->rotm_version >= 0 && p->rotm_version == p->m_version - 1);
+  if (!fused) {
+    SACHECK(sa_update_corrected_eigenvalues(p, beta2, weighting_factor, stream));
+    return precondition_eigenvalue_corrected(p, sc, bias_correction2, epsilon, root, false, s);
+  }
+  GemmScalars st = unit_scalars();
+  st.alpha = weighting_factor;
+  st.beta = beta2;
+  GemmScalars fu = st;
+  fu.div = bias_correction2; fu.pow_exp = 1.0f / root; fu.eps = epsilon;
+  fu.mom_w = 1.0f - sc->beta1; fu.mom_div = sc->bias_correction1;
+  double flops = 0.0;
+  for (const GemmTable* g : {&p->ec_stat1, &p->ec_stat2, &p->ec_stat_l, &p->ec_stat_r})
+    for (const GemmProblem& q : g->build) flops += 2.0 * q.M * q.N * q.K;
+  {
+    Span span("eigenbasis_rotation", s, flops, 4, true);
+    SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_STORE>(p->ec_stat1, unit_scalars(), s)));
+    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_EC_FUSED>(p->ec_stat2, fu, s)));
+    SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_SQ_EMA>(p->ec_stat_l, st, s)));
+    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_SQ_EMA>(p->ec_stat_r, st, s)));
+    if (p->has_order3 && p->t_chunks.n) {
+      hipLaunchKernelGGL(gather3_kernel, dim3((unsigned)p->t_chunks.n), dim3(EW_THREADS), 0, s, p->t_blocks.dev, p->t_chunks.dev, 2);
+      HIPCHECK(hipGetLastError());
+      SACHECK(launch_e3_chain<EPI_SQ_EMA>(p, 0, unit_scalars(), st, 1.0f, s));
+    }
+  }
+  if (p->table_mode == 1) p->rotm_version = p->m_version;
+  ++p->shared_rotation_steps;
+  return precondition_eigenvalue_corrected(p, sc, bias_correction2, epsilon, root, true, s);
 }
 
 // Blocked Householder QR of B (NB_X0) for the active factors; the reflectors are applied from the right to
@@ -3073,6 +3157,7 @@ int32_t sa_refresh_eigenbases_qr(sa_plan* p, float bias_correction2, float epsil
   const int F = (int)p->factors.size();
   if (F == 0) return SA_OK;
   p->eig_source.assign(F, sa_plan::EigSource{});
+  p->rotm_version = -1;  // the eigenbases change
   std::vector<int> todo;
   SACHECK(root_inverse_prologue(p, bias_correction2, epsilon, iterations_out, status_out, s, &todo));
   if (todo.empty()) return SA_OK;

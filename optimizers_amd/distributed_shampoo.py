@@ -277,6 +277,10 @@ class _NativeGroup(_AmortizedComputation):
     """Native state and schedule of one parameter group (reference: the per-group state lists
     built in distributed_shampoo.py:563-975 plus `_group_step_body` :1562-1667)."""
 
+    # Eigenvalue-corrected Shampoo: one library call updates the second moment in the eigenbasis and preconditions, reusing
+    # the rotated gradient for both.  False = the two separate calls of the reference's order (same results up to rounding).
+    fuse_eigenbasis_rotations = True
+
     def __init__(self, optimizer: "DistributedShampoo", group: dict[str, Any], group_index: int) -> None:
         self.lib = native.load()
         self.group_index = group_index
@@ -767,7 +771,10 @@ class _NativeGroup(_AmortizedComputation):
         if amortize:
             self._amortized_computation(group, bc2, stream)
             self.inverse_roots_stale = False
-        if self.soap:
+        # one call updates the second moment in the eigenbasis and preconditions (the rotated gradient serves both);
+        # with beta3 != beta1, or while only the grafting method steps, the statistic is updated on its own
+        fuse_soap = self.soap and self.fuse_eigenbasis_rotations and not graft_only and (beta1 == 0.0 or beta3 == beta1)
+        if self.soap and not fuse_soap:
             native.check(
                 lib.sa_update_corrected_eigenvalues(self.plan, beta2, weighting, stream), "sa_update_corrected_eigenvalues"
             )
@@ -818,7 +825,13 @@ class _NativeGroup(_AmortizedComputation):
                 lib.sa_update_grafting_and_filtered_grad(self.plan, ref, stream),
                 "sa_update_grafting_and_filtered_grad",
             )
-            if self.soap:
+            if fuse_soap:
+                native.check(
+                    lib.sa_update_and_precondition_eigenvalue_corrected(
+                        self.plan, ref, beta2, weighting, bc2, group[EPSILON], self.soap_root, stream),
+                    "sa_update_and_precondition_eigenvalue_corrected",
+                )
+            elif self.soap:
                 native.check(
                     lib.sa_precondition_eigenvalue_corrected(self.plan, ref, bc2, group[EPSILON], self.soap_root, stream),
                     "sa_precondition_eigenvalue_corrected",

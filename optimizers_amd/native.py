@@ -31,7 +31,7 @@ EXPORTS = (
     "sa_plan_bind_workspace", "sa_plan_num_factors", "sa_plan_invalidate_inverse_cache",
     "sa_plan_bind_gradients", "sa_add_l2_regularization", "sa_update_factor_matrices",
     "sa_compute_root_inverses_newton", "sa_compute_root_inverses_eigh", "sa_refresh_eigenbases_qr", "sa_refresh_eigenbases_eigh", "sa_update_corrected_eigenvalues",
-    "sa_precondition_eigenvalue_corrected", "sa_update_grafting_and_filtered_grad", "sa_precondition",
+    "sa_precondition_eigenvalue_corrected", "sa_update_and_precondition_eigenvalue_corrected", "sa_plan_shared_rotation_steps", "sa_update_grafting_and_filtered_grad", "sa_precondition",
     "sa_apply_update", "sa_grafting_only_step", "sa_plan_read_norms", "sa_plan_read_preconditioned",
     "sa_gemm_f32", "sa_copy_f32", "sa_set_profiling", "sa_phase_ms", "sa_phase_flops", "sa_phase_launches", "sa_phase_executed_flops", "sa_set_symmetric_newton", "sa_set_eigh_solver",
     "sa_plan_set_trace_scaling", "sa_compute_root_inverses_higher_order", "sa_plan_read_eigenvalues", "sa_add_to_views",
@@ -152,6 +152,10 @@ def load() -> ctypes.CDLL:
     ]
     lib.sa_update_corrected_eigenvalues.argtypes = [c_void_p, c_float, c_float, c_void_p]
     lib.sa_precondition_eigenvalue_corrected.argtypes = [c_void_p, POINTER(StepScalars), c_float, c_float, c_float, c_void_p]
+    lib.sa_plan_shared_rotation_steps.argtypes = [c_void_p]
+    lib.sa_plan_shared_rotation_steps.restype = c_int64
+    lib.sa_update_and_precondition_eigenvalue_corrected.argtypes = [
+        c_void_p, POINTER(StepScalars), c_float, c_float, c_float, c_float, c_float, c_void_p]
     for name in ("sa_update_grafting_and_filtered_grad", "sa_precondition", "sa_apply_update", "sa_grafting_only_step"):
         getattr(lib, name).argtypes = [c_void_p, POINTER(StepScalars), c_void_p]
     lib.sa_plan_read_norms.argtypes = [c_void_p, POINTER(c_float), POINTER(c_float), c_void_p]

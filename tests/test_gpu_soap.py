@@ -240,3 +240,60 @@ def test_order_three_blocks_rebuilt_from_the_stored_state(kind):
                 want = -lr * rotate(rot, Q, back=True)
                 delta = (block(after.reshape(48, 40, 9), s) - block(before.reshape(48, 40, 9), s)).double()
                 assert rel_err(delta, want) < 1e-3
+
+
+@pytest.mark.parametrize("beta1, graft", [(0.9, None), (0.0, None), (0.9, "adam")])
+@pytest.mark.parametrize("kind", ["soap_qr", "soap_eigh"])
+def test_shared_rotation_step_equals_the_two_separate_calls(kind, beta1, graft):
+    """The step updates the second moment in the eigenbasis and preconditions in one library call that rotates the gradient
+    once and carries Q_L^T m Q_R along by m's moving average between refreshes.  It must give what
+    sa_update_corrected_eigenvalues + sa_precondition_eigenvalue_corrected give (rotation of m itself on every step), over
+    refreshes, a masked parameter, ragged tiles, one-sided and order-3 blocks and a state reload."""
+    import optimizers_amd as oa
+    from optimizers_amd.distributed_shampoo import _NativeGroup
+
+    shapes = [(200, 136), (64, 300), (520,), (6, 40, 24), (128, 128)]
+    torch.manual_seed(3)
+    init = [0.1 * torch.randn(s) for s in shapes]
+    grads = [[0.05 * torch.randn(s) for s in shapes] for _ in range(13)]
+
+    def run(fused):
+        params = [torch.nn.Parameter(t.clone().to(DEV)) for t in init]
+
+        def make(ps):
+            return oa.DistributedShampoo(
+                ps, lr=0.02, betas=(beta1, 0.95), epsilon=1e-8, weight_decay=0.01, max_preconditioner_dim=128,
+                precondition_frequency=4, start_preconditioning_step=4,
+                grafting_config=oa.AdamPreconditionerConfig(beta2=0.95, epsilon=1e-8) if graft else None,
+                preconditioner_config=oa.DefaultSOAPConfig if kind == "soap_qr" else oa.DefaultEigenvalueCorrectedShampooConfig)
+
+        opt = make(params)
+        shared = 0
+        count = lambda o: o._groups[0].lib.sa_plan_shared_rotation_steps(o._groups[0].plan)
+        old = _NativeGroup.fuse_eigenbasis_rotations
+        _NativeGroup.fuse_eigenbasis_rotations = fused
+        try:
+            for s, gs in enumerate(grads, start=1):
+                for i, (p, g) in enumerate(zip(params, gs)):
+                    p.grad = None if (i == 1 and s in (7, 8)) else g.to(DEV)  # a parameter without gradient for two steps
+                opt.step()
+                if s == 10:  # rebuild from the checkpoint: nothing derived from the old plan may survive
+                    sd = opt.state_dict()
+                    shared += count(opt)
+                    params = [torch.nn.Parameter(p.detach().clone()) for p in params]
+                    opt = make(params)
+                    opt.load_state_dict(sd)
+                if s == 11:  # and a reload into the live optimizer, whose plan holds a rotated copy of the old state
+                    opt.load_state_dict(opt.state_dict())
+        finally:
+            _NativeGroup.fuse_eigenbasis_rotations = old
+        return [p.detach().cpu() for p in params], shared + count(opt)
+
+    (want, n_separate), (got, n_shared) = run(False), run(True)
+    # Without grafting every step preconditions (identity bases before step 4), with it steps 4..13.  With a filtered
+    # gradient the copy is rebuilt on the first step, after the refreshes (4, 8, 12), the mask changes (7, 9) and the
+    # reloads (11, 12): steps 2, 3, 5, 6, 10 and 13 are left, 5, 6, 10 and 13 with grafting.
+    assert n_separate == 0 and n_shared == (13 if beta1 == 0.0 else (4 if graft else 6))
+    for w, g in zip(want, got):
+        assert torch.isfinite(g).all()
+        assert rel_err(g, w) < 2e-5
