@@ -3,8 +3,10 @@
 // One refresh factors B = Q^T A Q (d x d) for every factor at once.  Columns are processed in panels;
 // a panel (all rows below the diagonal x up to 32 columns) is factored by ONE workgroup entirely in LDS
 // (up to 135 KB of the 160 KB a CU has), producing the Householder vectors V (unit lower trapezoid) and
-// the triangular factor T of the compact WY form H_1...H_k = I - V T V^T.  The trailing matrix and the
-// accumulated eigenbasis are then updated with the grouped MFMA GEMM (EPI_SUB).
+// the triangular factor T of the compact WY form H_1...H_k = I - V T V^T.  Panels are gathered into outer
+// blocks of up to QR_OUTER columns: a panel's reflectors are applied at once only to the rest of its outer block,
+// its (V, T) is merged into the block's (T12 = -T1 (V1^T V2) T2), and the trailing matrix and the accumulated
+// eigenbasis are updated once per outer block with the grouped MFMA GEMM (EPI_SUB), k = block width.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -15,16 +17,22 @@
 namespace sa {
 
 constexpr int QR_MAX_PANEL = 32;
+constexpr int QR_OUTER = 128;
 constexpr int QR_THREADS = 256;
 
 struct QrPanel {
   const float* B;   // matrix being factored, row stride ldb
-  float* V;         // rows x pcols, row stride QR_MAX_PANEL: Householder vectors (unit diagonal, zeros above)
-  float* T;         // QR_MAX_PANEL x QR_MAX_PANEL upper triangular
+  float* V;         // this panel's column block of the outer block's V (row stride ldv): `top` rows of zeros, then
+                    // rows x pcols Householder vectors (unit diagonal, zeros above)
+  float* T;         // this panel's column block of the outer block's T (row stride ldt, t_rows rows): the pcols x pcols
+                    // upper triangular factor at rows [top, top + pcols), zeros elsewhere
   long long ldb;
   int d;            // matrix dimension
   int j0;           // first column / row of the panel
   int pcols;        // columns in this panel
+  int ldv, ldt;
+  int top;          // columns of the outer block before this panel
+  int t_rows;       // width of the outer block
   const int* active;
 };
 
@@ -116,13 +124,15 @@ __global__ __launch_bounds__(QR_THREADS) void qr_panel_kernel(const QrPanel* __r
     if (tid == i) Tm[i][i] = tau_s[i];
     __syncthreads();
   }
-  for (int e = tid; e < QR_MAX_PANEL * QR_MAX_PANEL; e += QR_THREADS)
-    J.T[e] = Tm[e / QR_MAX_PANEL][e % QR_MAX_PANEL];
-  for (int e = tid; e < rows * QR_MAX_PANEL; e += QR_THREADS) {
-    const int r = e / QR_MAX_PANEL, c = e % QR_MAX_PANEL;
+  for (int e = tid; e < J.t_rows * pc; e += QR_THREADS) {
+    const int r = e / pc, c = e - r * pc, i = r - J.top;
+    J.T[(long long)r * J.ldt + c] = (i >= 0 && i < pc) ? Tm[i][c] : 0.f;
+  }
+  for (int e = tid; e < (J.top + rows) * pc; e += QR_THREADS) {
+    const int rr = e / pc, c = e - rr * pc, r = rr - J.top;
     float v = 0.f;
-    if (c < pc) v = (r > c) ? P[r * st + c] : (r == c ? 1.0f : 0.0f);
-    J.V[(long long)r * QR_MAX_PANEL + c] = v;
+    if (r >= 0) v = (r > c) ? P[r * st + c] : (r == c ? 1.0f : 0.0f);
+    J.V[(long long)rr * J.ldv + c] = v;
   }
 }
 

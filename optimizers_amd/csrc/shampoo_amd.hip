@@ -282,8 +282,10 @@ struct sa_plan {
   GemmTable eig_gemm;
   GemmTable ec_stat1, ec_stat2, ec_stat_l, ec_stat_r;          // corrected-eigenvalue update
   GemmTable ec_p1, ec_p1d, ec_p2, ec_p2d, ec_p3, ec_p3n, ec_p4, ec_p4n;  // eigenvalue-corrected preconditioning
-  GemmTable qr_g[6], qr_aq, qr_b;
-  Table<QrPanel> t_qrpanel;
+  struct QrInner { Table<QrPanel> panel; GemmTable upd[3], merge[3]; };
+  QrInner qr_in[4];        // rings, so that the host can fill the tables of the next panels while the GPU works
+  GemmTable qr_outer[2][6];
+  GemmTable qr_aq, qr_b;
   Table<TrdJob> t_trd;
   hipStream_t trd_stream = nullptr;  // applies QL rotations concurrently with the next chase
   hipEvent_t trd_ev[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
@@ -1060,8 +1062,9 @@ void sa_plan_destroy(sa_plan* p) {
   for (GemmTable* g : {&p->ec_stat1, &p->ec_stat2, &p->ec_stat_l, &p->ec_stat_r, &p->ec_p1, &p->ec_p1d, &p->ec_p2, &p->ec_p2d,
                        &p->ec_p3, &p->ec_p3n, &p->ec_p4, &p->ec_p4n, &p->qr_aq, &p->qr_b})
     g->t.destroy();
-  for (auto& g : p->qr_g) g.t.destroy();
-  p->t_qrpanel.destroy(); p->t_copy.destroy(); p->t_normpair.destroy(); p->t_sort.destroy();
+  for (auto& r : p->qr_in) { r.panel.destroy(); for (auto& g : r.upd) g.t.destroy(); for (auto& g : r.merge) g.t.destroy(); }
+  for (auto& a : p->qr_outer) for (auto& g : a) g.t.destroy();
+  p->t_copy.destroy(); p->t_normpair.destroy(); p->t_sort.destroy();
   for (void* q : {(void*)p->d_err, (void*)p->d_active, (void*)p->d_iters, (void*)p->d_final_parity,
                   (void*)p->d_final_err, (void*)p->d_flags, (void*)p->d_nactive, (void*)p->d_scale,
                   (void*)p->d_ho, (void*)p->d_kept_err, (void*)p->d_hoflag})
@@ -3075,73 +3078,130 @@ int32_t sa_update_and_precondition_eigenvalue_corrected(sa_plan* p, const sa_ste
 }
 
 // Blocked Householder QR of B (NB_X0) for the active factors; the reflectors are applied from the right to
-// Qacc (NB_X1):  Qacc <- Qacc H_1 H_2 ... H_d.
+// Qacc (NB_X1):  Qacc <- Qacc H_1 H_2 ... H_d.  Two levels of blocking: LDS-resident panels inside outer blocks.
 static int qr_accumulate(sa_plan* p, const std::vector<int>& ids, hipStream_t s) {
   const int n = (int)ids.size();
-  int dmax = 0;
-  for (int i : ids) dmax = std::max(dmax, p->factors[i].d);
+  int dmax = 0, dpad_min = 1 << 30;
+  for (int i : ids) {
+    dmax = std::max(dmax, p->factors[i].d);
+    dpad_min = std::min(dpad_min, p->factors[i].dpad);
+  }
   const int lds_floats = 34816;  // 136 KB for the panel, the rest of the 160 KB holds the small arrays
-  int pc_max = std::min(QR_MAX_PANEL, lds_floats / dmax - 1);
-  if (pc_max < 1) return fail(SA_ERR_UNSUPPORTED, "QR refresh: factor dimension too large for an LDS resident panel");
+  const int ip = std::min(QR_MAX_PANEL, lds_floats / dmax - 1);  // panel width
+  if (ip < 1) return fail(SA_ERR_UNSUPPORTED, "QR refresh: factor dimension too large for an LDS resident panel");
   static bool attr_set = false;
   if (!attr_set) {
     HIPCHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(qr_panel_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                  lds_floats * (int)sizeof(float)));
     attr_set = true;
   }
-  for (int j0 = 0; j0 < dmax; j0 += pc_max) {
-    SACHECK(p->t_qrpanel.begin(n));
-    for (int k = 0; k < 6; ++k) p->qr_g[k].clear();
-    int jobs = 0, max_rows = 0;
+  // Outer blocks pay off where the trailing matrix is large; their scratch (below) needs dpad >= 512.
+  const int OB = dpad_min >= 512 ? QR_OUTER : ip;
+  // scratch of a factor.  NB_S1: V (dpad x OB) | T (OB x OB) | S (OB x 32) | X (OB x 32).
+  //                       NB_S2: W (OB x dpad) | W2 (OB x dpad), later Z (d x OB) | Z2 (d x OB) in the same place.
+  auto mk = [&](int i, const float* A, long long lda, const float* Bm, long long ldb, float* C, long long ldc, int M, int N, int K) {
+    GemmProblem q{};
+    q.A = A; q.lda = lda; q.a_vec = vec_ok(A, lda);
+    q.B = Bm; q.ldb = ldb; q.b_vec = vec_ok(Bm, ldb);
+    q.C = C; q.ldc = ldc; q.M = M; q.N = N; q.K = K;
+    q.active = p->d_active + i;
+    return q;
+  };
+  const GemmScalars u = unit_scalars();
+  GemmScalars neg = u;
+  neg.a_div = -1.0f;
+  int inner_no = 0, outer_no = 0;
+  for (int J0 = 0; J0 < dmax; J0 += OB, ++outer_no) {
+    for (int off = 0; off < OB && J0 + off < dmax; off += ip, ++inner_no) {
+      sa_plan::QrInner& R = p->qr_in[inner_no % 4];
+      const int j0 = J0 + off;
+      SACHECK(R.panel.begin(n));
+      for (int k = 0; k < 3; ++k) { R.upd[k].clear(); R.merge[k].clear(); }
+      int jobs = 0, max_rows = 0;
+      for (int i : ids) {
+        const Factor& f = p->factors[i];
+        if (j0 >= f.d) continue;
+        const int ob = std::min(OB, f.d - J0);  // width of this factor's outer block
+        const int pc = std::min(ip, ob - off), rows = f.d - j0;
+        const int n_in = ob - off - pc;         // columns of the outer block after this panel
+        float* B = newton_buf(p, NB_X0, f);
+        float* V = newton_buf(p, NB_S1, f);
+        float* T = V + (long long)f.dpad * OB;
+        float* S = T + OB * OB;
+        float* X = S + OB * QR_MAX_PANEL;
+        float* W = newton_buf(p, NB_S2, f);
+        float* W2 = W + (long long)OB * f.dpad;
+        float* Vi = V + (long long)off * OB + off;  // this panel's vectors inside V (whose rows start at J0)
+        float* Ti = T + (long long)off * OB + off;
+        QrPanel& J = R.panel.host[jobs++];
+        std::memset(&J, 0, sizeof(J));
+        J.B = B; J.ldb = f.dpad; J.d = f.d; J.j0 = j0; J.pcols = pc; J.active = p->d_active + i;
+        J.V = V + off; J.ldv = OB; J.top = off;
+        J.T = T + off; J.ldt = OB; J.t_rows = ob;
+        max_rows = std::max(max_rows, rows);
+        if (n_in > 0) {
+          float* Bt = B + (long long)j0 * f.dpad + j0 + pc;  // rest of the outer block, B[j0:, j0+pc : J0+ob]
+          R.upd[0].add(mk(i, Vi, OB, Bt, f.dpad, W, f.dpad, pc, n_in, rows), false);   // W = V_i^T Bt    (A_KM)
+          R.upd[1].add(mk(i, Ti, OB, W, f.dpad, W2, f.dpad, pc, n_in, pc), false);     // W2 = T_i^T W    (A_KM)
+          R.upd[2].add(mk(i, Vi, OB, W2, f.dpad, Bt, f.dpad, rows, n_in, pc), false);  // Bt -= V_i W2    (A_MK, SUB)
+        }
+        if (off > 0) {
+          // T[0:off, off:off+pc] = -T[0:off, 0:off] (V[:, 0:off]^T V_i) T_i; V_i is zero above row off
+          R.merge[0].add(mk(i, V + (long long)off * OB, OB, Vi, OB, S, QR_MAX_PANEL, off, pc, rows), false);  // S = V_prev^T V_i (A_KM)
+          R.merge[1].add(mk(i, T, OB, S, QR_MAX_PANEL, X, QR_MAX_PANEL, off, pc, off), false);               // X = T_prev S     (A_MK)
+          R.merge[2].add(mk(i, X, QR_MAX_PANEL, Ti, OB, T + off, OB, off, pc, pc), false);                   // T12 = (-X) T_i   (A_MK)
+        }
+      }
+      if (!jobs) break;
+      R.panel.n = jobs;
+      SACHECK(R.panel.upload(s));
+      for (int k = 0; k < 3; ++k) { SACHECK(R.upd[k].commit(s)); SACHECK(R.merge[k].commit(s)); }
+      const size_t lds_bytes = (size_t)max_rows * (ip + 1) * sizeof(float);
+      hipLaunchKernelGGL(qr_panel_kernel, dim3(jobs), dim3(QR_THREADS), lds_bytes, s, R.panel.dev);
+      HIPCHECK(hipGetLastError());
+      SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, true>(R.upd[0], u, s)));
+      SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, true>(R.upd[1], u, s)));
+      SACHECK((launch_gemm<A_MK, B_KN, EPI_SUB, true>(R.upd[2], u, s)));
+      SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, true>(R.merge[0], u, s)));
+      SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, true>(R.merge[1], u, s)));
+      SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, true>(R.merge[2], neg, s)));
+    }
+    // the outer block's reflectors I - V T V^T on the trailing matrix (from the left, transposed) and on Qacc (from the right)
+    GemmTable* G = p->qr_outer[outer_no % 2];
+    for (int k = 0; k < 6; ++k) G[k].clear();
+    bool any = false;
     for (int i : ids) {
       const Factor& f = p->factors[i];
-      if (j0 >= f.d) continue;
-      const int pc = std::min(pc_max, f.d - j0), rows = f.d - j0, ntrail = f.d - j0 - pc;
+      if (J0 >= f.d) continue;
+      any = true;
+      const int ob = std::min(OB, f.d - J0), rows0 = f.d - J0, ntrail = f.d - J0 - ob;
       float* B = newton_buf(p, NB_X0, f);
       float* Qacc = newton_buf(p, NB_X1, f);
       float* V = newton_buf(p, NB_S1, f);
-      float* T = V + (long long)f.dpad * QR_MAX_PANEL;
-      float* W = T + QR_MAX_PANEL * QR_MAX_PANEL;
-      float* W2 = W + (long long)QR_MAX_PANEL * f.dpad;
-      float* Z = newton_buf(p, NB_S2, f);
-      float* Z2 = Z + (long long)f.dpad * QR_MAX_PANEL;
-      QrPanel& J = p->t_qrpanel.host[jobs++];
-      std::memset(&J, 0, sizeof(J));
-      J.B = B; J.V = V; J.T = T; J.ldb = f.dpad; J.d = f.d; J.j0 = j0; J.pcols = pc; J.active = p->d_active + i;
-      max_rows = std::max(max_rows, rows);
-      auto mk = [&](const float* A, long long lda, const float* Bm, long long ldb, float* C, long long ldc, int M, int N, int K) {
-        GemmProblem q{};
-        q.A = A; q.lda = lda; q.a_vec = vec_ok(A, lda);
-        q.B = Bm; q.ldb = ldb; q.b_vec = vec_ok(Bm, ldb);
-        q.C = C; q.ldc = ldc; q.M = M; q.N = N; q.K = K;
-        q.active = p->d_active + i;
-        return q;
-      };
+      float* T = V + (long long)f.dpad * OB;
+      float* W = newton_buf(p, NB_S2, f);
+      float* W2 = W + (long long)OB * f.dpad;
+      float* Z = W;
+      float* Z2 = W2;
       if (ntrail > 0) {
-        float* Bt = B + (long long)j0 * f.dpad + j0 + pc;  // trailing matrix B[j0:, j0+pc:]
-        p->qr_g[0].add(mk(V, QR_MAX_PANEL, Bt, f.dpad, W, f.dpad, pc, ntrail, rows), false);   // W = V^T Bt      (A_KM)
-        p->qr_g[1].add(mk(T, QR_MAX_PANEL, W, f.dpad, W2, f.dpad, pc, ntrail, pc), false);      // W2 = T^T W     (A_KM)
-        p->qr_g[2].add(mk(V, QR_MAX_PANEL, W2, f.dpad, Bt, f.dpad, rows, ntrail, pc), false);   // Bt -= V W2     (A_MK, SUB)
+        float* Bt = B + (long long)J0 * f.dpad + J0 + ob;  // trailing matrix B[J0:, J0+ob:]
+        G[0].add(mk(i, V, OB, Bt, f.dpad, W, f.dpad, ob, ntrail, rows0), false);   // W = V^T Bt      (A_KM)
+        G[1].add(mk(i, T, OB, W, f.dpad, W2, f.dpad, ob, ntrail, ob), false);      // W2 = T^T W      (A_KM)
+        G[2].add(mk(i, V, OB, W2, f.dpad, Bt, f.dpad, rows0, ntrail, ob), false);  // Bt -= V W2      (A_MK, SUB)
       }
-      float* Qt = Qacc + j0;  // Qacc[:, j0:]
-      p->qr_g[3].add(mk(Qt, f.dpad, V, QR_MAX_PANEL, Z, QR_MAX_PANEL, f.d, pc, rows), false);   // Z = Qt V       (NN)
-      p->qr_g[4].add(mk(Z, QR_MAX_PANEL, T, QR_MAX_PANEL, Z2, QR_MAX_PANEL, f.d, pc, pc), false);  // Z2 = Z T     (NN)
-      p->qr_g[5].add(mk(Z2, QR_MAX_PANEL, V, QR_MAX_PANEL, Qt, f.dpad, f.d, rows, pc), false);  // Qt -= Z2 V^T   (B_NK, SUB)
+      float* Qt = Qacc + J0;  // Qacc[:, J0:]
+      G[3].add(mk(i, Qt, f.dpad, V, OB, Z, OB, f.d, ob, rows0), false);   // Z = Qt V       (NN)
+      G[4].add(mk(i, Z, OB, T, OB, Z2, OB, f.d, ob, ob), false);          // Z2 = Z T       (NN)
+      G[5].add(mk(i, Z2, OB, V, OB, Qt, f.dpad, f.d, rows0, ob), false);  // Qt -= Z2 V^T   (B_NK, SUB)
     }
-    if (!jobs) break;
-    p->t_qrpanel.n = jobs;
-    SACHECK(p->t_qrpanel.upload(s));
-    for (int k = 0; k < 6; ++k) SACHECK(p->qr_g[k].commit(s));
-    const size_t lds_bytes = (size_t)max_rows * (pc_max + 1) * sizeof(float);
-    hipLaunchKernelGGL(qr_panel_kernel, dim3(jobs), dim3(QR_THREADS), lds_bytes, s, p->t_qrpanel.dev);
-    HIPCHECK(hipGetLastError());
-    GemmScalars u = unit_scalars();
-    SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, true>(p->qr_g[0], u, s)));
-    SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, true>(p->qr_g[1], u, s)));
-    SACHECK((launch_gemm<A_MK, B_KN, EPI_SUB, true>(p->qr_g[2], u, s)));
-    SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, true>(p->qr_g[3], u, s)));
-    SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, true>(p->qr_g[4], u, s)));
-    SACHECK((launch_gemm<A_MK, B_NK, EPI_SUB, true>(p->qr_g[5], u, s)));
+    if (!any) break;
+    for (int k = 0; k < 6; ++k) SACHECK(G[k].commit(s));
+    SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, true>(G[0], u, s)));
+    SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, true>(G[1], u, s)));
+    SACHECK((launch_gemm<A_MK, B_KN, EPI_SUB, true>(G[2], u, s)));
+    SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, true>(G[3], u, s)));
+    SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, true>(G[4], u, s)));
+    SACHECK((launch_gemm<A_MK, B_NK, EPI_SUB, true>(G[5], u, s)));
   }
   return SA_OK;
 }

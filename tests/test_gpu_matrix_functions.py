@@ -215,3 +215,27 @@ def test_symmetric_products_converge_like_full_products(d, caplog):
     lam, Q = torch.linalg.eigh(A.double().cpu())
     truth = (Q * lam.pow(-0.25)) @ Q.T
     assert rel_err(results[1].double().cpu(), truth) <= 1e-3
+
+
+@pytest.mark.parametrize("d", (512, 700, 1000))
+def test_qr_refresh_of_large_matrices_against_fp64(d):
+    """One QR iteration from a perturbed eigenbasis at orders where the Householder panels are gathered into outer blocks
+    (block reflectors merged, one trailing update per block; 700 and 1000 end in ragged blocks): the new basis must be
+    the oracle's in fp64 (matrix_functions.py:799-852) up to column signs, and orthonormal to fp32 rounding."""
+    import optimizers_amd as oa
+    from optimizers_amd.matrix_functions import matrix_eigendecomposition
+    from oracle.shampoo_oracle import qr_refresh
+
+    g = torch.Generator().manual_seed(d)
+    a = torch.randn(d, 2 * d, generator=g, dtype=torch.float64)
+    A = a @ a.T / (2 * d) + 0.5 * torch.eye(d, dtype=torch.float64)  # condition number ~ 7: the factorization is well posed
+    q0 = torch.linalg.qr(torch.linalg.eigh(A)[1] + 0.02 * torch.randn(d, d, generator=g, dtype=torch.float64))[0]
+    want_l, want_q = qr_refresh(A, q0, max_iterations=1)
+    L, Q = matrix_eigendecomposition(
+        A=A.float().to(DEV), eigenvectors_estimate=q0.float().to(DEV),
+        eigendecomposition_config=oa.QREigendecompositionConfig(max_iterations=1))
+    Qd = Q.cpu().double()
+    assert (Qd.T @ Qd - torch.eye(d, dtype=torch.float64)).abs().max() < 2e-5
+    signs = torch.sign((Qd * want_q).sum(0))
+    assert rel_err(Qd * signs, want_q) < 1e-4
+    assert rel_err(L.cpu().double(), want_l) < 1e-5

@@ -112,10 +112,12 @@ def test_soap_medium_blocks_match_oracle(shapes, b, graft, kind):
         ref.step([x.clone() for x in grads])
         ref64.step([x.double() for x in grads])
         # After a refresh the stable sort of nearly equal eigenvalue estimates can order two columns
-        # differently under different rounding (the reference's fp32 and fp64 runs differ by ~1e-2 here), so the
-        # bound again carries the reference algorithm's own rounding gap.
+        # differently under different rounding, and the eigenvectors of the noise bulk are decided by rounding (the
+        # reference's fp32 and fp64 runs differ by ~1e-2 here).  Any two fp32 evaluations therefore differ at that level:
+        # what is checked is that the native run stays as close to the fp64 run as an fp32 run of the reference does,
+        # up to a factor of 2.5 (measured 2.1 to 2.3 for the panel-by-panel and the outer-block QR alike).
         for p, r, r64 in zip(params, ref_p, ref64_p):
-            assert rel_err(p.detach().cpu(), r) < 1e-3 + 2.0 * rel_err(r, r64), step
+            assert rel_err(p.detach().cpu().double(), r64) < 1e-3 + 2.5 * rel_err(r, r64), step
     ng = opt._groups[0]
     for k, bi in enumerate(ng.native_index):
         spec = ng.block_specs[bi]
