@@ -18,7 +18,7 @@ namespace sa {
 
 constexpr int QR_MAX_PANEL = 32;
 constexpr int QR_OUTER = 128;
-constexpr int QR_THREADS = 256;
+constexpr int QR_THREADS = 1024;
 
 struct QrPanel {
   const float* B;   // matrix being factored, row stride ldb
@@ -36,10 +36,13 @@ struct QrPanel {
   const int* active;
 };
 
-// dynamic LDS: rows * (pcols + 1) floats for the panel
+// dynamic LDS: rows * (pcols + 1) floats for the panel.  1024 threads: a panel of 1024 rows is one row per thread, and four
+// waves per SIMD hide the LDS latency of the column-by-column sweeps.
 __global__ __launch_bounds__(QR_THREADS) void qr_panel_kernel(const QrPanel* __restrict__ jobs) {
   extern __shared__ float lds[];
-  __shared__ float wred[4][QR_MAX_PANEL];
+  constexpr int NW = QR_THREADS / 64;
+  __shared__ float wred[NW][QR_MAX_PANEL];
+  __shared__ float wfin[QR_MAX_PANEL];
   __shared__ float tau_s[QR_MAX_PANEL];
   __shared__ float S[QR_MAX_PANEL][QR_MAX_PANEL + 1];
   __shared__ float Tm[QR_MAX_PANEL][QR_MAX_PANEL + 1];
@@ -62,7 +65,8 @@ __global__ __launch_bounds__(QR_THREADS) void qr_panel_kernel(const QrPanel* __r
     if (lane == 0) wred[wave][0] = part;
     __syncthreads();
     if (tid == 0) {
-      const float sigma2 = (wred[0][0] + wred[1][0]) + (wred[2][0] + wred[3][0]);
+      float sigma2 = 0.f;
+      for (int w = 0; w < NW; ++w) sigma2 += wred[w][0];
       const float alpha = (c < rows) ? P[c * st + c] : 0.f;
       float tau = 0.f, scale = 0.f, beta = alpha;
       if (sigma2 != 0.f && c < rows) {
@@ -88,16 +92,19 @@ __global__ __launch_bounds__(QR_THREADS) void qr_panel_kernel(const QrPanel* __r
         if (lane == 0) wred[wave][cc] = w;
       }
       __syncthreads();
-      for (int cc = c + 1; cc < pc; ++cc) {
-        const float w = tau * (P[c * st + cc] + (wred[0][cc] + wred[1][cc]) + (wred[2][cc] + wred[3][cc]));
-        for (int r = c + 1 + tid; r < rows; r += QR_THREADS) P[r * st + cc] -= w * P[r * st + c];
+      if (tid < pc - (c + 1)) {
+        // row c itself (v[c] = 1) is this thread's alone
+        const int cc = c + 1 + tid;
+        float w = 0.f;
+        for (int k = 0; k < NW; ++k) w += wred[k][cc];
+        w = tau * (P[c * st + cc] + w);
+        wfin[cc] = w;
+        P[c * st + cc] -= w;
       }
       __syncthreads();
-      if (tid < pc - (c + 1)) {
-        // row c itself (v[c] = 1); row c and the partial sums are still untouched
-        const int cc = c + 1 + tid;
-        const float w = tau * (P[c * st + cc] + (wred[0][cc] + wred[1][cc]) + (wred[2][cc] + wred[3][cc]));
-        P[c * st + cc] -= w;
+      for (int r = c + 1 + tid; r < rows; r += QR_THREADS) {
+        const float v = P[r * st + c];
+        for (int cc = c + 1; cc < pc; ++cc) P[r * st + cc] -= wfin[cc] * v;
       }
       __syncthreads();
     }
