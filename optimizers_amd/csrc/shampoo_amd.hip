@@ -240,6 +240,8 @@ struct sa_plan {
   Table<ChunkRef> t_chunks;
   Table<int> t_active_blocks;
   GemmTable syrk0, syrk1, g1_store, g1_norm, g2_norm, g2g_norm;
+  GemmTable syrk0e, syrk1e;  // Gram problems that need the guarded loader (vectors: k = 1; ragged blocks), launched apart so that
+                             // they do not force it on the rest
   // factor matrices kept in fp64 (factor_matrix_dtype = float64): fp64 averages in the SYRK epilogue, fp64 coupled
   // Newton root inverse on a scratch region twice the size; the inverse roots stay fp32
   bool factor_f64 = false;
@@ -451,6 +453,12 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
   // factor-update tables
   p->syrk0.clear();
   p->syrk1.clear();
+  p->syrk0e.clear();
+  p->syrk1e.clear();
+  auto add_syrk = [&](int which, const GemmProblem& q) {
+    const bool al = q.M % BM == 0 && q.N % BN == 0 && q.K % BK == 0 && q.a_vec && q.b_vec;
+    (which == 0 ? (al ? p->syrk0 : p->syrk0e) : (al ? p->syrk1 : p->syrk1e)).add(q, true);
+  };
   p->kl_right.clear();
   p->kl_left.clear();
   for (int b : active) {
@@ -480,13 +488,13 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
       q.lda = d.cols; q.ldb = d.cols; q.ldc = 0;
       q.M = d.rows; q.N = d.rows; q.K = d.cols;
       q.a_vec = q.b_vec = vec_ok(TR, d.cols);
-      p->syrk0.add(q, true);
+      add_syrk(0, q);
       GemmProblem w{};
       w.A = TL; w.B = TL; w.C = d.factor[1];
       w.lda = d.cols; w.ldb = d.cols; w.ldc = 0;
       w.M = d.cols; w.N = d.cols; w.K = d.rows;
       w.a_vec = w.b_vec = vec_ok(TL, d.cols);
-      p->syrk1.add(w, true);
+      add_syrk(1, w);
       continue;
     }
     if (d.mid > 0) {
@@ -499,7 +507,7 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
         q.lda = ld; q.ldb = ld; q.ldc = 0;
         q.M = dim; q.N = dim; q.K = K;
         q.a_vec = q.b_vec = vec_ok(T, ld);
-        (k_major ? p->syrk1 : p->syrk0).add(q, true);
+        add_syrk(k_major ? 1 : 0, q);
       };
       if (d.factor[0]) gram(B.g3_dense, (long long)d1 * d2, d0, d1 * d2, d.factor[0], false);
       if (d.factor[1]) gram(B.g3_perm, (long long)d0 * d2, d1, d0 * d2, d.factor[1], false);
@@ -512,7 +520,7 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
       q.lda = d.ld; q.ldb = d.ld; q.ldc = 0;
       q.M = d.rows; q.N = d.rows; q.K = d.cols;
       q.a_vec = q.b_vec = vec_ok(G, d.ld);
-      p->syrk0.add(q, true);
+      add_syrk(0, q);
     }
     if (d.factor[1]) {  // R = G^T G  (cols x cols, K = rows)
       GemmProblem q{};
@@ -520,11 +528,13 @@ int rebuild_tables(sa_plan* p, int mode, hipStream_t s) {
       q.lda = d.ld; q.ldb = d.ld; q.ldc = 0;
       q.M = d.cols; q.N = d.cols; q.K = d.rows;
       q.a_vec = q.b_vec = vec_ok(G, d.ld);
-      p->syrk1.add(q, true);
+      add_syrk(1, q);
     }
   }
   SACHECK(p->syrk0.commit(s));
   SACHECK(p->syrk1.commit(s));
+  SACHECK(p->syrk0e.commit(s));
+  SACHECK(p->syrk1e.commit(s));
   SACHECK(p->kl_right.commit(s));
   SACHECK(p->kl_left.commit(s));
 
@@ -1040,7 +1050,7 @@ void sa_plan_destroy(sa_plan* p) {
   if (!p) return;
   p->t_blocks.destroy(); p->t_chunks.destroy(); p->t_active_blocks.destroy();
   for (GemmTable* g : {&p->kl_right, &p->kl_left}) g->t.destroy();
-  for (GemmTable* g : {&p->syrk0, &p->syrk1, &p->g1_store, &p->g1_norm, &p->g2_norm, &p->g2g_norm, &p->nt_a[0][0],
+  for (GemmTable* g : {&p->syrk0, &p->syrk1, &p->syrk0e, &p->syrk1e, &p->g1_store, &p->g1_norm, &p->g2_norm, &p->g2g_norm, &p->nt_a[0][0],
                        &p->nt_a[0][1], &p->nt_m[0][0], &p->nt_m[0][1], &p->nt_a[1][0], &p->nt_a[1][1], &p->nt_m[1][0],
                        &p->nt_m[1][1]})
     g->t.destroy();
@@ -1142,9 +1152,9 @@ static int update_factor_matrices(sa_plan* p, double beta2, double weighting_fac
   sc.alpha64 = weighting_factor;
   sc.beta64 = beta2;
   double flops = 0.0;
-  for (const GemmTable* g : {&p->syrk0, &p->syrk1})
+  for (const GemmTable* g : {&p->syrk0, &p->syrk1, &p->syrk0e, &p->syrk1e})
     for (const GemmProblem& q : g->build) flops += (double)q.N * q.N * q.K;  // symmetric half: d^2 k
-  int launches = (p->syrk0.total_tiles ? 1 : 0) + (p->syrk1.total_tiles ? 1 : 0);
+  int launches = (p->syrk0.total_tiles ? 1 : 0) + (p->syrk1.total_tiles ? 1 : 0) + (p->syrk0e.total_tiles ? 1 : 0) + (p->syrk1e.total_tiles ? 1 : 0);
   if (p->has_order3 && p->t_chunks.n) {
     hipLaunchKernelGGL(gather3_kernel, dim3((unsigned)p->t_chunks.n), dim3(EW_THREADS), 0, s, p->t_blocks.dev, p->t_chunks.dev, 0);
     HIPCHECK(hipGetLastError());
@@ -1158,9 +1168,13 @@ static int update_factor_matrices(sa_plan* p, double beta2, double weighting_fac
   if (p->factor_f64) {
     SACHECK((launch_gemm_auto<A_MK, B_NK, EPI_SYRK_EMA64>(p->syrk0, sc, s)));
     SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_SYRK_EMA64>(p->syrk1, sc, s)));
+    SACHECK((launch_gemm_auto<A_MK, B_NK, EPI_SYRK_EMA64>(p->syrk0e, sc, s)));
+    SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_SYRK_EMA64>(p->syrk1e, sc, s)));
   } else {
     SACHECK((launch_gemm_auto<A_MK, B_NK, EPI_SYRK_EMA>(p->syrk0, sc, s)));
     SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_SYRK_EMA>(p->syrk1, sc, s)));
+    SACHECK((launch_gemm_auto<A_MK, B_NK, EPI_SYRK_EMA>(p->syrk0e, sc, s)));
+    SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_SYRK_EMA>(p->syrk1e, sc, s)));
   }
   return SA_OK;
 }
