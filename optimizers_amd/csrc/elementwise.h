@@ -465,7 +465,7 @@ struct SymFactor {
   const float* packed_in;  // packed source (factor for Newton init, inverse for unpack)
   float* packed_out;       // packed destination (commit)
   const float* dense_in;   // dense source (commit)
-  float* dense_out[3];     // dense destinations
+  float* dense_out[4];     // dense destinations (Newton init: M, M_p, X, and optionally X M_p)
   unsigned int* err_bits;
   const float* norm_partial;  // Newton init: per-chunk partial sums of squares
   const float* scale;      // Newton init: optional per-factor multiplier applied after the division by bc2
@@ -570,6 +570,9 @@ __global__ __launch_bounds__(256) void sym_pass_kernel(const SymFactor* __restri
         F.dense_out[0][o] = m;
         F.dense_out[1][o] = mp;
         F.dense_out[2][o] = diag ? x0 : 0.f;
+        // X is a multiple of the identity, so the first X M_p is x0 * M_p entry by entry: exactly what the product
+        // would give (every other term of the dot product is an exact zero)
+        if (F.dense_out[3] != nullptr) F.dense_out[3][o] = __fmul_rn(x0, mp);
         if (r < d && c < d) {
           const float dv = fabsf(m - (r == c ? 1.0f : 0.0f));
           if (dv != dv) errnan = true;

@@ -266,6 +266,7 @@ struct sa_plan {
   GemmTable kl_right, kl_left;  // G X_R -> T buffer, X_L G -> P buffer
   // Newton, [0] full products / [1] symmetric products: X*M_p with M_p^2 per parity, power chain, M update per parity
   GemmTable nt_a[2][2], nt_pow[2][8], nt_m[2][2];
+  GemmTable nt_a0[2];  // first iteration: launch A without X M_p (the init kernel wrote it)
   GemmTable nt_h[8];      // Horner products of the higher-order iteration
   // mode products of order-3 blocks: [mode 1 | mode 0 | mode 2][first stage (divides by bias_correction1)][last stage (norm)]
   GemmTable g3[3][2][2];
@@ -1050,7 +1051,7 @@ void sa_plan_destroy(sa_plan* p) {
   if (!p) return;
   p->t_blocks.destroy(); p->t_chunks.destroy(); p->t_active_blocks.destroy();
   for (GemmTable* g : {&p->kl_right, &p->kl_left}) g->t.destroy();
-  for (GemmTable* g : {&p->syrk0, &p->syrk1, &p->syrk0e, &p->syrk1e, &p->g1_store, &p->g1_norm, &p->g2_norm, &p->g2g_norm, &p->nt_a[0][0],
+  for (GemmTable* g : {&p->syrk0, &p->syrk1, &p->syrk0e, &p->syrk1e, &p->g1_store, &p->g1_norm, &p->g2_norm, &p->g2g_norm, &p->nt_a[0][0], &p->nt_a0[0], &p->nt_a0[1],
                        &p->nt_a[0][1], &p->nt_m[0][0], &p->nt_m[0][1], &p->nt_a[1][0], &p->nt_a[1][1], &p->nt_m[1][0],
                        &p->nt_m[1][1]})
     g->t.destroy();
@@ -1391,6 +1392,7 @@ static int newton_batch(sa_plan* p, const std::vector<int>& ids, const std::vect
     S.dense_out[0] = newton_buf(p, NB_M0, f);
     S.dense_out[1] = newton_buf(p, NB_MP0, f);
     S.dense_out[2] = newton_buf(p, NB_X0, f);
+    S.dense_out[3] = newton_buf(p, NB_X1, f);
     S.err_bits = p->d_err + ids[i];
     S.norm_partial = p->f(p->off_norm_partial) + f.norm_off;
     S.n_norm_partial = f.norm_chunks;
@@ -1406,6 +1408,7 @@ static int newton_batch(sa_plan* p, const std::vector<int>& ids, const std::vect
   // ---- GEMM tables -------------------------------------------------------------------------
   for (int v = 0; v < 2; ++v) {
     for (int par = 0; par < 2; ++par) { p->nt_a[v][par].clear(); p->nt_m[v][par].clear(); }
+    p->nt_a0[v].clear();
     for (int k = 0; k < 8; ++k) p->nt_pow[v][k].clear();
   }
   auto prob = [&](const Factor& f, const float* A, const float* B, float* C) {
@@ -1436,6 +1439,7 @@ static int newton_batch(sa_plan* p, const std::vector<int>& ids, const std::vect
       // launch A: X <- X M_p, and the first squaring if the root needs one
       p->nt_a[v][par].add(prob(f, X, Mp, Xn), sym);
       if (!ops.empty()) p->nt_a[v][par].add(prob(f, Mp, Mp, S1), sym);
+      if (!ops.empty() && par == 0) p->nt_a0[v].add(prob(f, Mp, Mp, S1), sym);
       // the remaining chain reads only S1 / S2 / M_p of this parity
       const float* cur = ops.empty() ? Mp : S1;
       int slot = par * 4;  // nt_pow[0..3] parity 0, [4..7] parity 1
@@ -1455,6 +1459,7 @@ static int newton_batch(sa_plan* p, const std::vector<int>& ids, const std::vect
   }
   for (int v = 0; v < 2; ++v) {
     for (int par = 0; par < 2; ++par) { SACHECK(p->nt_a[v][par].commit(s)); SACHECK(p->nt_m[v][par].commit(s)); }
+    SACHECK(p->nt_a0[v].commit(s));
     for (int k = 0; k < 8; ++k) SACHECK(p->nt_pow[v][k].commit(s));
   }
 
@@ -1479,8 +1484,9 @@ static int newton_batch(sa_plan* p, const std::vector<int>& ids, const std::vect
         const Factor& f = p->factors[ids[i]];
         const double d = f.d, t = f.dpad / BM;
         const bool sym = symmetric[i] != 0;
-        flops += (sym ? d * d * (d + 1.0) : 2.0 * d * d * d) * gemms_per_iter;
-        executed += 2.0 * BM * BN * (double)f.dpad * (sym ? t * (t + 1) / 2 : t * t) * gemms_per_iter;
+        const int products = gemms_per_iter - (it == 0 ? 1 : 0);  // the first X M_p is not a product
+        flops += (sym ? d * d * (d + 1.0) : 2.0 * d * d * d) * products;
+        executed += 2.0 * BM * BN * (double)f.dpad * (sym ? t * (t + 1) / 2 : t * t) * products;
         ++live;
       }
     if (!live) break;
@@ -1495,8 +1501,8 @@ static int newton_batch(sa_plan* p, const std::vector<int>& ids, const std::vect
       // the two variants touch disjoint factors, so their launches of one stage are independent
       // symmetric variant: every operand is an exactly mirrored matrix, so A is read through its transpose (slabs
       // load and store as 16-byte rows instead of four scalar LDS stores per thread; same values, same results)
-      SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, false, true>(p->nt_a[1][parity], unit, s)));
-      SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, false>(p->nt_a[0][parity], unit, s)));
+      SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, false, true>(it == 0 ? p->nt_a0[1] : p->nt_a[1][parity], unit, s)));
+      SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, false>(it == 0 ? p->nt_a0[0] : p->nt_a[0][parity], unit, s)));
       for (int k = 0; k < 4; ++k) {
         SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, false, true>(p->nt_pow[1][parity * 4 + k], unit, s)));
         SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, false, false>(p->nt_pow[0][parity * 4 + k], unit, s)));
