@@ -3216,12 +3216,13 @@ static int qr_accumulate(sa_plan* p, const std::vector<int>& ids, hipStream_t s)
     }
     if (!any) break;
     for (int k = 0; k < 6; ++k) SACHECK(G[k].commit(s));
-    SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, true>(G[0], u, s)));
-    SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, true>(G[1], u, s)));
-    SACHECK((launch_gemm<A_MK, B_KN, EPI_SUB, true>(G[2], u, s)));
-    SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, true>(G[3], u, s)));
-    SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, true>(G[4], u, s)));
-    SACHECK((launch_gemm<A_MK, B_NK, EPI_SUB, true>(G[5], u, s)));
+    // full outer blocks of aligned factors take the unguarded loader
+    SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_STORE>(G[0], u, s)));
+    SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_STORE>(G[1], u, s)));
+    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_SUB>(G[2], u, s)));
+    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE>(G[3], u, s)));
+    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE>(G[4], u, s)));
+    SACHECK((launch_gemm_auto<A_MK, B_NK, EPI_SUB>(G[5], u, s)));
   }
   return SA_OK;
 }
