@@ -170,12 +170,14 @@ struct NormPair {
   long long ldb;
   int d;
 };
-__global__ __launch_bounds__(256) void diag_off_norm_kernel(const NormPair* __restrict__ jobs) {
-  __shared__ float red[4];
+constexpr int FACTOR_PASS_THREADS = 1024;  // one workgroup per factor: 16 waves to cover the latency of its d x d sweep
+__global__ __launch_bounds__(FACTOR_PASS_THREADS) void diag_off_norm_kernel(const NormPair* __restrict__ jobs) {
+  constexpr int NW = FACTOR_PASS_THREADS / 64;
+  __shared__ float red[2][NW];
   const NormPair& J = jobs[blockIdx.x];
   float a = 0.f, dg = 0.f;
   const long long n = (long long)J.d * J.d;
-  for (long long e = threadIdx.x; e < n; e += 256) {
+  for (long long e = threadIdx.x; e < n; e += FACTOR_PASS_THREADS) {
     const int r = (int)(e / J.d), c = (int)(e % J.d);
     const float v = J.B[r * J.ldb + c];
     a += v * v;
@@ -183,14 +185,15 @@ __global__ __launch_bounds__(256) void diag_off_norm_kernel(const NormPair* __re
   }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   a = wave_sum(a);
-  if (lane == 0) red[wave] = a;
-  __syncthreads();
-  const float ta = (red[0] + red[1]) + (red[2] + red[3]);
-  __syncthreads();
   dg = wave_sum(dg);
-  if (lane == 0) red[wave] = dg;
+  if (lane == 0) { red[0][wave] = a; red[1][wave] = dg; }
   __syncthreads();
-  if (threadIdx.x == 0) { *J.out_all = ta; *J.out_diag = (red[0] + red[1]) + (red[2] + red[3]); }
+  if (threadIdx.x == 0) {
+    float ta = 0.f, td = 0.f;
+    for (int w = 0; w < NW; ++w) { ta += red[0][w]; td += red[1][w]; }
+    *J.out_all = ta;
+    *J.out_diag = td;
+  }
 }
 
 // Rayleigh quotients ev[i] = sum_r Q[r][i] * Y[r][i], stable ascending rank of ev, and its inverse
@@ -204,16 +207,16 @@ struct SortJob {
   long long ldq, ldy;
   int d;
 };
-__global__ __launch_bounds__(256) void rayleigh_sort_kernel(const SortJob* __restrict__ jobs) {
+__global__ __launch_bounds__(FACTOR_PASS_THREADS) void rayleigh_sort_kernel(const SortJob* __restrict__ jobs) {
   const SortJob& J = jobs[blockIdx.x];
   const int d = J.d;
-  for (int i = threadIdx.x; i < d; i += 256) {
+  for (int i = threadIdx.x; i < d; i += FACTOR_PASS_THREADS) {
     float acc = 0.f;
     for (int r = 0; r < d; ++r) acc += J.Q[r * J.ldq + i] * J.Y[r * J.ldy + i];
     J.ev[i] = acc;
   }
   __syncthreads();
-  for (int i = threadIdx.x; i < d; i += 256) {
+  for (int i = threadIdx.x; i < d; i += FACTOR_PASS_THREADS) {
     const float x = J.ev[i];
     int rank = 0;
     for (int j = 0; j < d; ++j) {

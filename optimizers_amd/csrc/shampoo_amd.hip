@@ -2791,7 +2791,7 @@ int32_t sa_refresh_eigenbases_eigh(sa_plan* p, float bias_correction2, float eps
     HIPCHECK(hipGetLastError());
     SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE>(p->qr_aq, unit_scalars(), s)));
     SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_STORE>(p->qr_b, unit_scalars(), s)));
-    hipLaunchKernelGGL(diag_off_norm_kernel, dim3(n), dim3(256), 0, s, p->t_normpair.dev);
+    hipLaunchKernelGGL(diag_off_norm_kernel, dim3(n), dim3(FACTOR_PASS_THREADS), 0, s, p->t_normpair.dev);
     HIPCHECK(hipGetLastError());
     HIPCHECK(hipMemcpyAsync(p->h_pinned, p->d_final_err, F * sizeof(float), hipMemcpyDeviceToHost, s));
     HIPCHECK(hipMemcpyAsync(p->h_pinned + F, p->d_err, F * sizeof(float), hipMemcpyDeviceToHost, s));
@@ -3304,7 +3304,7 @@ int32_t sa_refresh_eigenbases_qr(sa_plan* p, float bias_correction2, float epsil
       J.out_diag = reinterpret_cast<float*>(p->d_err) + todo[k];
     }
     SACHECK(p->t_normpair.upload(s));
-    hipLaunchKernelGGL(diag_off_norm_kernel, dim3(n), dim3(256), 0, s, p->t_normpair.dev);
+    hipLaunchKernelGGL(diag_off_norm_kernel, dim3(n), dim3(FACTOR_PASS_THREADS), 0, s, p->t_normpair.dev);
     HIPCHECK(hipGetLastError());
     HIPCHECK(hipMemcpyAsync(p->h_pinned, p->d_final_err, F * sizeof(float), hipMemcpyDeviceToHost, s));
     HIPCHECK(hipMemcpyAsync(p->h_pinned + F, p->d_err, F * sizeof(float), hipMemcpyDeviceToHost, s));
@@ -3351,7 +3351,7 @@ int32_t sa_refresh_eigenbases_qr(sa_plan* p, float bias_correction2, float epsil
   }
   SACHECK(p->t_sort.upload(s));
   SACHECK(p->t_copy.upload(s));
-  hipLaunchKernelGGL(rayleigh_sort_kernel, dim3(n), dim3(256), 0, s, p->t_sort.dev);
+  hipLaunchKernelGGL(rayleigh_sort_kernel, dim3(n), dim3(FACTOR_PASS_THREADS), 0, s, p->t_sort.dev);
   hipLaunchKernelGGL(copy2d_kernel, dim3(64, n), dim3(256), 0, s, p->t_copy.dev);  // sorted basis -> NB_X0
   HIPCHECK(hipGetLastError());
 
