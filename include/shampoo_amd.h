@@ -12,7 +12,8 @@
  * Conventions: every pointer inside a descriptor is a DEVICE pointer borrowed from the
  * caller (who keeps it alive until the stream work has finished); `stream` is a
  * hipStream_t passed as void*; every call returns SA_OK or an error code and leaves a
- * message for sa_last_error().  No exceptions cross the boundary.  All arithmetic is fp32.
+ * message for sa_last_error().  No exceptions cross the boundary.  All arithmetic is fp32, except the factor
+ * averages and the coupled Newton iteration of a plan switched to fp64 factors (sa_plan_set_factor_dtype).
  * One plan describes the blocks of one parameter group on one GPU; calls on one plan must
  * not overlap.
  */
