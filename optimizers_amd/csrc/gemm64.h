@@ -177,6 +177,7 @@ struct Factor64 {
   double* M;             // dense n x n outputs of the start kernel
   double* Mp;
   double* X;
+  double* X1;            // x0 * M_p: the first X M_p (X is a multiple of the identity, the other terms are exact zeros)
   const double* result;  // dense n x n input of the commit kernel
   float* inv_packed;     // fp32 upper triangle of the result
   float* inv_dense;      // fp32 dense, mirrored from the upper triangle, n x n zero padded
@@ -247,6 +248,7 @@ __global__ __launch_bounds__(256) void f64_newton_start_kernel(const Factor64* _
     J.M[e] = m;
     J.Mp[e] = mp;
     J.X[e] = x;
+    J.X1[e] = x0 * mp;
   }
 }
 

@@ -259,7 +259,7 @@ struct sa_plan {
       build.push_back(q);
     }
   };
-  GemmTable64 n64_a[2], n64_pow[8], n64_m[2];
+  GemmTable64 n64_a[2], n64_pow[8], n64_m[2], n64_a0;
   Table<ChunkRef> t_all_chunks;  // chunks of every block, masked or not (train / eval switch of primal averaging)
   // KL-Shampoo: the Gram matrices of a two-sided block are taken of the gradient preconditioned along the other dim
   bool kl = false;
@@ -1061,7 +1061,7 @@ void sa_plan_destroy(sa_plan* p) {
   for (auto& a : p->e3) for (auto& b2 : a) for (auto& c2 : b2) for (auto& g : c2) g.t.destroy();
   p->t_all_chunks.destroy();
   p->t_f64.destroy();
-  for (auto* g : {&p->n64_a[0], &p->n64_a[1], &p->n64_m[0], &p->n64_m[1]}) g->t.destroy();
+  for (auto* g : {&p->n64_a[0], &p->n64_a[1], &p->n64_m[0], &p->n64_m[1], &p->n64_a0}) g->t.destroy();
   for (auto& g : p->n64_pow) g.t.destroy();
   if (p->d_norm64) (void)hipFree(p->d_norm64);
   p->t_ho.destroy();
@@ -1761,6 +1761,7 @@ static int newton_batch64(sa_plan* p, const std::vector<int>& ids, int root, con
     std::memset(&J, 0, sizeof(J));
     J.packed = reinterpret_cast<const double*>(f.factor);
     J.M = newton_buf64(p, NB_M0, f); J.Mp = newton_buf64(p, NB_MP0, f); J.X = newton_buf64(p, NB_X0, f);
+    J.X1 = newton_buf64(p, NB_X1, f);
     J.norm_sq = p->d_norm64 + ids[i];
     J.nonfinite = p->d_flags + ids[i];
     J.ridge = ridge[ids[i]];
@@ -1773,6 +1774,7 @@ static int newton_batch64(sa_plan* p, const std::vector<int>& ids, int root, con
   HIPCHECK(hipGetLastError());
 
   for (int par = 0; par < 2; ++par) { p->n64_a[par].clear(); p->n64_m[par].clear(); }
+  p->n64_a0.clear();
   for (auto& g : p->n64_pow) g.clear();
   auto prob = [&](const Factor& f, const double* A, const double* B, double* C) {
     GemmProblem64 q{};
@@ -1794,6 +1796,7 @@ static int newton_batch64(sa_plan* p, const std::vector<int>& ids, int root, con
       double* S2 = newton_buf64(p, NB_S2, f);
       p->n64_a[par].add(prob(f, X, Mp, Xn));
       if (!ops.empty()) p->n64_a[par].add(prob(f, Mp, Mp, S1));
+      if (!ops.empty() && par == 0) p->n64_a0.add(prob(f, Mp, Mp, S1));  // first iteration: X M_p came from the start kernel
       const double* cur = ops.empty() ? Mp : S1;
       int slot = par * 4;
       double* pong[2] = {S2, S1};
@@ -1810,6 +1813,7 @@ static int newton_batch64(sa_plan* p, const std::vector<int>& ids, int root, con
     }
   }
   for (int par = 0; par < 2; ++par) { SACHECK(commit64(p->n64_a[par], s)); SACHECK(commit64(p->n64_m[par], s)); }
+  SACHECK(commit64(p->n64_a0, s));
   for (auto& g : p->n64_pow) SACHECK(commit64(g, s));
 
   // the start error is 1 (M = z A is far from I): one control pass with err = +inf activates every factor
@@ -1830,11 +1834,11 @@ static int newton_batch64(sa_plan* p, const std::vector<int>& ids, int root, con
     int live = 0;
     double flops = 0.0;
     for (int i = 0; i < n; ++i)
-      if (h_active[ids[i]]) { ++live; const double d = p->factors[ids[i]].d; flops += 2.0 * d * d * d * (2.0 + ops.size()); }
+      if (h_active[ids[i]]) { ++live; const double d = p->factors[ids[i]].d; flops += 2.0 * d * d * d * (2.0 + ops.size() - (it == 0 ? 1.0 : 0.0)); }
     if (!live) break;
     {
       Span span("newton_gemm_f64", s, flops, 2 + (int)ops.size() - 1, it == 0);
-      SACHECK(launch_gemm64<EPI64_STORE>(p->n64_a[parity], 0.0, 0.0, s));
+      SACHECK(launch_gemm64<EPI64_STORE>(it == 0 ? p->n64_a0 : p->n64_a[parity], 0.0, 0.0, s));
       for (int k = 0; k < 4; ++k) SACHECK(launch_gemm64<EPI64_STORE>(p->n64_pow[parity * 4 + k], 0.0, 0.0, s));
       SACHECK(launch_gemm64<EPI64_NEWTON_M>(p->n64_m[parity], alpha, one_minus_alpha, s));
     }
