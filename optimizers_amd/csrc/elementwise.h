@@ -500,7 +500,7 @@ enum SymMode { SYM_UNPACK = 0, SYM_NEWTON_INIT = 1, SYM_COMMIT = 2 };
 // SYM_UNPACK:      dense_out[0] = mirror(packed_in)
 // SYM_NEWTON_INIT: a = packed_in / bc2 (+ eps on the diagonal); z = (root+1)/(2 ||A||_F);
 //                  dense_out[0] = M = z a, dense_out[1] = M_p = M*mp_scale + mp_diag I,
-//                  dense_out[2] = X = z^(1/root) I, err = max |M - I|
+//                  dense_out[2] = X = z^(1/root) I, dense_out[3] = X M_p = z^(1/root) M_p (optional), err = max |M - I|
 // SYM_COMMIT:      packed_out = upper(dense_in) (if packed_out), dense_out[0] = mirror(upper(dense_in))
 template <int MODE>
 __global__ __launch_bounds__(256) void sym_pass_kernel(const SymFactor* __restrict__ factors, int n_factors,
