@@ -437,6 +437,10 @@ class ShampooOracle:
         self.bc2_shampoo = torch.tensor(1.0)
         self.bc2_graft = torch.tensor(1.0)
         self.last_newton_iterations: list[list[int]] = []
+        # Test hook, called with the oracle right after every amortized computation and before anything uses its result
+        # (a test that compares runs on two hosts uses it to give columns of a refreshed eigenbasis whose eigenvalue
+        # estimates are tied within rounding the order they had in the other run).
+        self.after_amortized: Any = None
 
     # -- construction ------------------------------------------------------- #
 
@@ -682,6 +686,8 @@ class ShampooOracle:
         if amortize:
             for i, st in zip(active, S):
                 self.last_newton_iterations.append(self._amortized(st, i))
+            if self.after_amortized is not None:
+                self.after_amortized(self)
         if self.soap:
             # shampoo_preconditioner_list.py:1891-1912
             w2 = 1.0 if beta2 == 1.0 else 1 - beta2

@@ -64,7 +64,7 @@ from distributed_shampoo.shampoo_types import (  # noqa: E402
 
 OUT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(os.path.dirname(OUT)))
-from tests.golden_cases import horizon_grads, oracle_config  # noqa: E402  (gradient streams shared with the tests)
+from tests.golden_cases import basis_signature, horizon_grads, oracle_config  # noqa: E402  (shared with the tests)
 
 
 def case_params(shapes, seed):
@@ -287,7 +287,15 @@ CASES = {
         shapes=[[512, 768]], seed=33, grad_kind="gauss_lowrank", grad_scale=1e-2, lowrank_rank=32, lowrank_scale=1e-3,
         steps=50, zero_init=True, trace_stride=997, lr=1e-3, betas=[0.9, 0.999], epsilon=1e-12, weight_decay=0.0,
         weight_decay_type="DECOUPLED", max_preconditioner_dim=256, precondition_frequency=10,
-        start_preconditioning_step=10, preconditioner="soap_qr", override_1d=False, grafting=None,
+        start_preconditioning_step=10, preconditioner="soap_qr", override_1d=False, grafting=None, basis_signature=3,
+    ),
+    # configuration 4 at its real block order: one 1024 x 768 block (factors of order 1024 and 768), same gradients'
+    # recipe and cadence; 30 steps, three refreshes
+    "horizon_soap_1024": dict(
+        shapes=[[1024, 768]], seed=35, grad_kind="gauss_lowrank", grad_scale=1e-2, lowrank_rank=32, lowrank_scale=1e-3,
+        steps=30, zero_init=True, trace_stride=997, lr=1e-3, betas=[0.9, 0.999], epsilon=1e-12, weight_decay=0.0,
+        weight_decay_type="DECOUPLED", max_preconditioner_dim=1024, precondition_frequency=10,
+        start_preconditioning_step=10, preconditioner="soap_qr", override_1d=False, grafting=None, basis_signature=3,
     ),
     # configuration 5: 512-blocks, G = U diag(s) V^T with s log-uniform in [1e-6, 1], eigendecomposition root inverse
     # every 50 steps (EigenConfig); 100 steps
@@ -442,6 +450,16 @@ def run_case(name, c):
                 out[f"norm_s{s}_p{i}"] = np.float64(p.detach().double().norm().item())
                 if "trace_stride" in c:
                     out[f"trace_s{s}_p{i}"] = p.detach().reshape(-1)[:: c["trace_stride"]].numpy().copy()
+            start, freq = c["start_preconditioning_step"], c["precondition_frequency"]
+            if c.get("basis_signature") and (s == start or (s > start and s % freq == 0)):
+                # The order in which THIS run's stable sort left the columns of every refreshed eigenbasis
+                # (matrix_functions.py:848-850), as a few seeded projections per column: estimates that agree to
+                # within their rounding error come out in either order from one correct fp32 evaluation to the next.
+                for pi, p in enumerate(params):
+                    for key, val in opt.state[p].items():
+                        if isinstance(val, dict) and "shampoo" in val:
+                            for k, q in enumerate(val["shampoo"].factor_matrices_eigenvectors):
+                                out[f"sig_s{s}_p{pi}_{key}_{k}"] = basis_signature(q, c["basis_signature"]).numpy().copy()
             if "trace_stride" in c:
                 print(f"  {name}: reference step {s} done", flush=True)
     big = max(p.numel() for p in params) > 100_000

@@ -1,42 +1,43 @@
 """The benchmark configurations' horizons and cadences against fixtures the real reference wrote: 20 steps of coupled
 Newton on a ragged GPT-2 slice (81 x 768 tail block) and on a Llama slice, 50 steps of eigenvalue-corrected Shampoo with
-a QR refresh every 10, 100 steps with an eigendecomposition root inverse every 50 on log-uniform spectra.  The initial
-parameters are zero, so the parameters compared ARE the accumulated updates.  No oracle runs here: the native step
-(through the C ABI) is compared with the reference's stored fp32 run, step by step on a subsample and at the end, and
-the float64 run stored beside it shows how far two correct fp32 evaluations can be apart.
+a QR refresh every 10 on 256-blocks and 30 steps on one 1024 x 768 block, 100 steps with an eigendecomposition root
+inverse every 50 on log-uniform spectra.  The initial parameters are zero, so the parameters compared ARE the accumulated
+updates.  The native step (through the C ABI) is compared with the reference's stored fp32 run, step by step on a
+subsample and at the end, and the float64 run stored beside it shows how far two correct fp32 evaluations can be apart.
 
-Bound: 1e-3 relative Frobenius error on the accumulated update at every step (the stated tolerance); measured 8e-7 and
-1.3e-6 on the Newton cases and 1e-6 on the eigendecomposition case, the distance of the reference's own fp32 run from
-float64.
+Bound: 1e-3 relative Frobenius error on the accumulated update at every step (the stated tolerance), for every case.
 
-horizon_soap is bounded differently from its first refresh on.  A QR refresh ends with a stable sort of the eigenvalue
-estimates, and the second moment kept in the eigenbasis is not re-indexed (shampoo_preconditioner_list.py:1867-1912,
-matrix_functions.py:848-850).  With 6 blocks x 2 factors x 255 neighbouring pairs x 5 refreshes some pair of estimates is
-always closer than fp32 resolves (closest pair of this case in float64: 2e-8 of the largest eigenvalue), so its order is
-a coin toss of the rounding; every such flip pairs two rows (or columns) of the rotated gradient with each other's second
-moment, an error of up to about 1.4e-2 in that step's update which then decays as the moment re-averages.  The
-reference's own fp32 run is 4.4e-3 away from float64 at the end for this reason.  Which refresh flips depends on the last
-bit of the factor matrices (with the factor update's fused multiply-add in the compiler's order the first refresh agreed
-with the reference and steps 1-19 were within 5e-7; pinned to the reference's order, a pair flips at the first refresh),
-and a flipped pair stays mis-paired until the next refresh, so the error keeps growing in between.  The test therefore
-holds the native run to 1e-3 before the first refresh and to 3e-2 (two flips' worth) afterwards, and prints where the
-error moved.
-
-That the differences ARE such order flips, and nothing else, is shown by the last test: it runs the fp32 oracle beside the
-native step up to the first refresh and compares the two eigenbases of every factor.  They must agree column by column
-(|cosine| > 0.999) except for transpositions of neighbouring columns whose Rayleigh quotients, evaluated in float64, are
-closer than 2e-6 of the largest one (a few ulp of the fp32 values that were sorted)."""
+The eigenvalue-corrected cases need one thing said about the reference first.  A QR refresh ends with a stable sort of
+the eigenvalue estimates, and the second moment kept in the eigenbasis is not re-indexed
+(shampoo_preconditioner_list.py:1867-1912, matrix_functions.py:848-850).  The estimates are the diagonal of an fp32
+product and carry a rounding error of a few 1e-6 of the largest; with hundreds of neighbouring pairs per factor some are
+always closer than that, and in which order such a pair leaves the sort depends on the last bits: the reference's own
+run differs between two hosts (other BLAS kernels, another thread count) by 4e-3 after 50 steps for this reason alone,
+and by 4.4e-3 from its float64 run.  A swapped pair meets each other's second moment until the next refresh.  The
+fixtures therefore record, for every refresh of the reference's run, a signature of every column of every eigenbasis
+(tests/golden_cases.py: basis_signature).  The tests read the native bases right after each native refresh, before the
+step uses them; every column must be one of the reference run's columns, a column in another position must have moved
+between positions whose Rayleigh quotients (float64) are tied within the estimates' rounding error (tie_tolerance), and
+such columns are then put in the reference run's order, the documented route for outside writes to the state
+(sa_plan_invalidate_inverse_cache).  Anything that is not a reordering of ties fails.  With that, the run meets the
+plain 1e-3 on every step (measured 1e-6).  The same is done beside the fp32 oracle for all five refreshes with the
+columns compared directly (|cosine| > 0.999), and a run without any alignment is held to 1e-3 before the first refresh
+and to 3e-2 (a few swapped pairs' worth) afterwards, with the error's path printed."""
 
 import pytest
 import torch
 
-from tests.golden_cases import grad_stream, initial_params, load_cases, load_npz, oracle_config, rel_err
+from tests.golden_cases import (
+    assert_reordering_is_between_ties, basis_signature, grad_stream, initial_params, load_cases, load_npz, match_columns,
+    oracle_config, rel_err,
+)
 from tests.test_gpu_step_parity import native_optimizer
 
 pytestmark = pytest.mark.gpu
 
 CASES = load_cases()
 HORIZON_CASES = [n for n in CASES if n.startswith("horizon_")]
+SOAP_CASES = [n for n in HORIZON_CASES if CASES[n].get("basis_signature")]
 
 
 def _native(c, params):
@@ -50,16 +51,65 @@ def _native(c, params):
     return native_optimizer(c, params)
 
 
-@pytest.mark.parametrize("name", HORIZON_CASES)
-def test_benchmark_horizon_matches_reference_fixture(name):
-    print(f"case {name}", flush=True)
+def order_ties_like(opt, params, wanted_signature, log, compare=None, tolerance=1e-3):
+    """Wraps the amortized computation of the optimizer's (only) group: right after every native eigenbasis refresh, and
+    before the step uses the bases, every basis is matched column by column against `wanted_signature(step, block index,
+    block spec, factor)` (a (k, n) basis signature of the run to follow, or None).  Every column must be found there
+    (signatures equal to `tolerance`); a column found at another position must be a tie (assert_reordering_is_between_ties);
+    the columns are then put in the followed run's order and the plan is told that its state was written from outside.
+    `compare(step, block index, factor, reordered native basis)` may check more.  log collects
+    (step, block index, factor, columns moved, largest relative gap of their Rayleigh quotients)."""
+    from optimizers_amd import native
+
+    group = opt._groups[0]
+    inner = group._amortized_computation
+
+    def amortized_then_ordered(g, bc2, stream):
+        inner(g, bc2, stream)
+        s = int(group.step_tensor)
+        for bi in group.native_index:
+            spec = group.block_specs[bi]
+            st = opt.state[params[spec.param_index]][spec.block_key]["shampoo"]
+            for k, q in sorted(st["factor_matrices_eigenvectors"].items()):
+                want = wanted_signature(s, bi, spec, k)
+                if want is None:
+                    continue
+                where = f"step {s} block {bi} factor {k}"
+                match, dist = match_columns(basis_signature(q, want.shape[0]), want)
+                assert dist < tolerance, (where, dist)
+                moved, gap = assert_reordering_is_between_ties(match, q, st["factor_matrices"][k], where)
+                if moved:
+                    q.copy_(q[:, match.to(q.device)])
+                if compare is not None:
+                    compare(s, bi, k, q)
+                log.append((s, bi, k, moved, gap))
+        native.check(group.lib.sa_plan_invalidate_inverse_cache(group.plan), "sa_plan_invalidate_inverse_cache")
+
+    group._amortized_computation = amortized_then_ordered
+
+
+def _summary(log):
+    per_step = {}
+    for s, _, _, moved, gap in log:
+        n, g = per_step.get(s, (0, 0.0))
+        per_step[s] = (n + moved, max(g, gap))
+    return {s: (n, float(f"{g:.1e}")) for s, (n, g) in per_step.items()}
+
+
+def _run(name, align):
     c = CASES[name]
     z = load_npz(name)
     dev = torch.device("cuda:0")
     params = [torch.nn.Parameter(t.clone().to(dev)) for t in initial_params(c)]
     opt = _native(c, params)
+    log = []
+    if align:
+        def from_fixture(s, bi, spec, k):
+            key = f"sig_s{s}_p{spec.param_index}_{spec.block_key}_{k}"
+            return torch.as_tensor(z[key]) if key in z else None
+
+        order_ties_like(opt, params, from_fixture, log)
     stride = c["trace_stride"]
-    soap = name == "horizon_soap"
     freq, start = c["precondition_frequency"], c["start_preconditioning_step"]
     worst = floor = worst64 = 0.0
     errs = []
@@ -91,76 +141,76 @@ def test_benchmark_horizon_matches_reference_fixture(name):
         if s not in refresh:
             growth_between += max(errs[s - 1] - errs[s - 2], 0.0)
     print(
-        f"  {name}: native vs reference fp32: worst step {worst:.2e}, final {final:.2e}; native vs float64: worst step "
-        f"{worst64:.2e}, final {final64:.2e}; reference fp32 vs float64 (its own rounding floor): {floor:.2e}; "
-        f"Newton iteration counts differ by at most {iteration_mismatch}; error before the first refresh "
+        f"  {name}: native vs reference fp32: worst step {worst:.2e}, final {final:.2e} (bound 1e-3, no allowance); native vs "
+        f"float64: worst step {worst64:.2e}, final {final64:.2e}; reference fp32 vs float64 (its own rounding floor): "
+        f"{floor:.2e}; Newton iteration counts differ by at most {iteration_mismatch}; error before the first refresh "
         f"{max(errs[: start - 1], default=0.0):.2e}, jumps at refresh steps {({s: float(f'{j:.1e}') for s, j in jumps.items()})}, "
-        f"growth outside of refresh steps {growth_between:.2e}",
+        f"growth outside of refresh steps {growth_between:.2e}"
+        + (f"; tied columns put in the reference run's order per refresh (count, largest relative gap): {_summary(log)}" if align else ""),
         flush=True,
     )
-    if soap:
-        assert max(errs[: start - 1], default=0.0) < 1e-3
-        assert worst < 3e-2 and final < 3e-2, (worst, final)
-    else:
-        assert worst < 1e-3 and final < 1e-3, (worst, final)
+    return errs, worst, final, iteration_mismatch
+
+
+@pytest.mark.parametrize("name", HORIZON_CASES)
+def test_benchmark_horizon_matches_reference_fixture(name):
+    print(f"case {name}", flush=True)
+    _, worst, final, iteration_mismatch = _run(name, align=name in SOAP_CASES)
+    assert worst < 1e-3 and final < 1e-3, (worst, final)
     assert iteration_mismatch <= 1
 
 
-def _dense(factor, n):
-    """An oracle factor matrix as a dense float64 matrix, whether it is kept dense or as its packed upper triangle."""
-    if factor.dim() == 2:
-        return factor.double()
-    iu = torch.triu_indices(n, n)
-    full = torch.zeros(n, n, dtype=torch.float64)
-    full[iu[0], iu[1]] = factor.double()
-    return full + torch.triu(full, 1).T
+@pytest.mark.parametrize("name", SOAP_CASES)
+def test_soap_horizon_left_to_its_own_tie_order_stays_within_a_few_swapped_pairs(name):
+    """No alignment: what a user's run shows against the reference's run on another machine."""
+    print(f"case {name}", flush=True)
+    c = CASES[name]
+    errs, worst, final, _ = _run(name, align=False)
+    assert max(errs[: c["start_preconditioning_step"] - 1], default=0.0) < 1e-3
+    assert worst < 3e-2 and final < 3e-2, (worst, final)
 
 
-def test_soap_first_refresh_differs_from_the_oracle_only_by_order_flips_of_tied_estimates():
+@pytest.mark.parametrize("name", SOAP_CASES)
+def test_soap_horizon_beside_the_oracle_differs_only_by_the_order_of_tied_estimates(name):
+    """The fp32 oracle steps beside the native optimizer over the whole horizon.  After every refresh each native basis is
+    compared with the oracle's, column by column: |cosine| > 0.999 once ties are in the oracle's order, and nothing but
+    ties may be out of order.  The parameters then agree to the stated 1e-3 at every step (measured 1e-6)."""
     from oracle.shampoo_oracle import ShampooOracle
 
-    c = CASES["horizon_soap"]
+    print(f"case {name}", flush=True)
+    c = CASES[name]
     dev = torch.device("cuda:0")
     init = initial_params(c)
     params = [torch.nn.Parameter(t.clone().to(dev)) for t in init]
     opt = _native(c, params)
     ref_params = [t.clone() for t in init]
     ref = ShampooOracle(ref_params, oracle_config(c))
-    first_refresh = c["start_preconditioning_step"]
+    log = []
+    lowest = [1.0]
+
+    def from_oracle(s, bi, spec, k):
+        return basis_signature(ref.state[bi]["eigvecs"][k], 3)
+
+    def cosines(s, bi, k, q):
+        cos = (q.detach().cpu().double() * ref.state[bi]["eigvecs"][k].double()).sum(0).abs()
+        lowest[0] = min(lowest[0], float(cos.min()))
+        assert cos.min() > 0.999, (s, bi, k, float(cos.min()))
+
+    order_ties_like(opt, params, from_oracle, log, cosines)
+    worst = 0.0
     for s, grads in grad_stream(c):
+        ref.step([g.clone() for g in grads])  # the oracle first: its refreshed bases are what the native ones follow
         for p, g in zip(params, grads):
             p.grad = g.to(dev)
         opt.step()
-        ref.step([g.clone() for g in grads])
-        if s == first_refresh:
-            break
-    group = opt._groups[0]
-    flips = []
-    for bi in group.native_index:
-        spec = group.block_specs[bi]
-        native = opt.state[params[spec.param_index]][spec.block_key]["shampoo"]["factor_matrices_eigenvectors"]
-        want = ref.state[bi]
-        for j, q_ref in enumerate(want["eigvecs"]):
-            q_ref = q_ref.double()
-            n = q_ref.shape[0]
-            cos = (native[j].cpu().double().T @ q_ref).abs()
-            match = cos.argmax(dim=0).tolist()
-            rayleigh = torch.einsum("ij,ik,kj->j", q_ref, _dense(want["factors"][j], n), q_ref)
-            for col, row in enumerate(match):
-                assert cos[row, col] > 0.999, (bi, j, col, float(cos[row, col]))
-                if row == col:
-                    continue
-                assert abs(row - col) == 1 and match[row] == col, f"block {bi} factor {j}: column {col} matches {row}"
-                gap = float((rayleigh[row] - rayleigh[col]).abs() / rayleigh.abs().max())
-                assert gap < 2e-6, (bi, j, col, row, gap)
-                if col < row:
-                    flips.append((bi, j, col, row, gap))
-    err = max(rel_err(p.detach().cpu(), r) for p, r in zip(params, ref_params))
+        err = max(rel_err(p.detach().cpu(), r) for p, r in zip(params, ref_params))
+        worst = max(worst, err)
+        assert err < 1e-3, (s, err)
+    refreshes = sorted({s for s, *_ in log})
+    assert len(refreshes) == (c["steps"] - c["start_preconditioning_step"]) // c["precondition_frequency"] + 1
     print(
-        f"  step {first_refresh}: {len(flips)} neighbouring pair(s) in the other order "
-        f"{[(b, j, a, r, float(f'{g:.1e}')) for b, j, a, r, g in flips]} (block, factor, columns, relative gap of the "
-        f"Rayleigh quotients); parameters differ by {err:.1e}",
+        f"  {name}: {len(refreshes)} refreshes beside the oracle; tied columns in the other order per refresh (count, largest "
+        f"relative gap of their Rayleigh quotients): {_summary(log)}; lowest |cosine| between matched columns "
+        f"{lowest[0]:.6f}; parameters differ by at most {worst:.1e} over {c['steps']} steps",
         flush=True,
     )
-    if not flips:
-        assert err < 1e-5, err

@@ -85,8 +85,26 @@ def test_soap_fixture_case_matches_reference(name):
 @pytest.mark.parametrize("kind", ["soap_qr", "soap_eigh"])
 @pytest.mark.parametrize("shapes, b, graft", [([(256, 256)], 128, "adam"), ([(1024, 768)], 1024, None)])
 def test_soap_medium_blocks_match_oracle(shapes, b, graft, kind):
+    """Two refreshes (steps 3 and 6 of 7) beside the fp32 and the float64 oracle; (1024, 768) with b = 1024 takes the
+    outer-block QR that benchmark configuration 4 runs.
+
+    QR refresh: held to the plain 1e-3 on the accumulated update against the fp32 oracle at every step.  The refreshed
+    bases are read right after each native refresh; their columns must be the oracle's (|cosine| > 0.999), columns in
+    another position must be ties of the sorted estimates within their rounding error, and those are put in the oracle's
+    order before the step uses them (tests/test_gpu_horizons.py: order_ties_like) - the noise bulk of this spectrum holds
+    hundreds of such ties at order 1024.
+
+    Eigendecomposition refresh: no such statement exists.  Inside the noise bulk neighbouring eigenvalues are closer
+    than fp32 resolves next to the leading ones, so the eigenvectors there - not just their order - are decided by
+    rounding: two correct fp32 eigensolvers (LAPACK on two hosts, or LAPACK and the native solver) return bases that
+    differ by rotations inside the bulk, and the reference's own fp32 and float64 runs differ by about 1e-2 here.  Against
+    the reference's eigh the result is pinned only through what is invariant (orthogonality, the leading invariant
+    subspace) and through the distance to the float64 run: the native run must stay as close to it as the fp32 oracle
+    does, up to a factor of 2.5 (measured 2.1 to 2.3)."""
     import optimizers_amd as oa
     from oracle.shampoo_oracle import OracleConfig, ShampooOracle
+    from tests.golden_cases import basis_signature
+    from tests.test_gpu_horizons import _summary, order_ties_like
 
     print(f"case {shapes} b={b} graft={graft} {kind}", flush=True)
     g = torch.Generator().manual_seed(17)
@@ -102,8 +120,21 @@ def test_soap_medium_blocks_match_oracle(shapes, b, graft, kind):
     ref = ShampooOracle(ref_p, ocfg)
     ref64_p = [t.clone().double() for t in init]
     ref64 = ShampooOracle(ref64_p, ocfg)
+    qr = kind == "soap_qr"
+    log = []
+    if qr:
+        def cosines(s, bi, k, q):
+            cos = (q.detach().cpu().double() * ref.state[bi]["eigvecs"][k].double()).sum(0).abs()
+            assert cos.min() > 0.999, (s, bi, k, float(cos.min()))
+
+        # eight probes per column and a looser match than for the horizon fixtures: at the first refresh the factors have
+        # seen three gradients, and one QR step on such a matrix returns columns that differ by some 1e-3 between two fp32
+        # evaluations (the cosines are checked right after)
+        order_ties_like(opt, params, lambda s, bi, spec, k: basis_signature(ref.state[bi]["eigvecs"][k], 8), log, cosines,
+                        tolerance=1e-2)
     # low-rank + noise gradients give a skewed, well separated leading spectrum
     lows = [(torch.randn(s[0], 8, generator=g), torch.randn(8, s[1], generator=g)) if len(s) == 2 else None for s in shapes]
+    worst = 0.0
     for step in range(7):
         grads = []
         for s, lr_ in zip(shapes, lows):
@@ -111,18 +142,21 @@ def test_soap_medium_blocks_match_oracle(shapes, b, graft, kind):
             if lr_ is not None:
                 n = n + (lr_[0] * torch.rand(8, generator=g)) @ lr_[1] / 8
             grads.append(n)
+        ref.step([x.clone() for x in grads])
+        ref64.step([x.double() for x in grads])
         for p, gr in zip(params, grads):
             p.grad = gr.to(DEV)
         opt.step()
-        ref.step([x.clone() for x in grads])
-        ref64.step([x.double() for x in grads])
-        # After a refresh the stable sort of nearly equal eigenvalue estimates can order two columns
-        # differently under different rounding, and the eigenvectors of the noise bulk are decided by rounding (the
-        # reference's fp32 and fp64 runs differ by ~1e-2 here).  Any two fp32 evaluations therefore differ at that level:
-        # what is checked is that the native run stays as close to the fp64 run as an fp32 run of the reference does,
-        # up to a factor of 2.5 (measured 2.1 to 2.3 for the panel-by-panel and the outer-block QR alike).
-        for p, r, r64 in zip(params, ref_p, ref64_p):
-            assert rel_err(p.detach().cpu().double(), r64) < 1e-3 + 2.5 * rel_err(r, r64), step
+        for p, r, r64, w0 in zip(params, ref_p, ref64_p, init):
+            if qr:
+                err = rel_err(p.detach().cpu().double() - w0.double(), r.double() - w0.double())
+                worst = max(worst, err)
+                assert err < 1e-3, (step, err)
+            else:
+                assert rel_err(p.detach().cpu().double(), r64) < 1e-3 + 2.5 * rel_err(r, r64), step
+    if qr:
+        print(f"  accumulated update vs the fp32 oracle: at most {worst:.1e} (bound 1e-3, no allowance); tied columns put in "
+              f"the oracle's order per refresh (count, largest relative gap): {_summary(log)}", flush=True)
     ng = opt._groups[0]
     for k, bi in enumerate(ng.native_index):
         spec = ng.block_specs[bi]
@@ -130,8 +164,7 @@ def test_soap_medium_blocks_match_oracle(shapes, b, graft, kind):
         for j, q in enumerate(ref.state[bi]["eigvecs"]):
             got = st["factor_matrices_eigenvectors"][j].cpu()
             assert rel_err(got.T @ got, torch.eye(got.shape[0])) < 1e-4
-            # same subspaces column by column except where the sort order flipped: compare as projectors on the
-            # leading (well separated) part of the spectrum
+            # the leading (well separated) part of the spectrum spans the same subspace
             lead = slice(got.shape[0] - 8, got.shape[0])
             assert rel_err(got[:, lead] @ got[:, lead].T, q[:, lead] @ q[:, lead].T) < 1e-3
 

@@ -9,7 +9,7 @@ import pytest
 import torch
 
 from oracle import shampoo_oracle as O
-from tests.golden_cases import GOLDEN, grad_stream, initial_params, load_cases, load_npz, oracle_config, rel_err
+from tests.golden_cases import GOLDEN, align_oracle_to_fixture, grad_stream, initial_params, load_cases, load_npz, oracle_config, rel_err
 
 CASES = load_cases()
 
@@ -78,6 +78,13 @@ def test_benchmark_horizons_match_reference(name):
     z = load_npz(name)
     params = [p.clone() for p in initial_params(c)]
     opt = O.ShampooOracle(params, oracle_config(c))
+    reordered = []
+    if c.get("basis_signature"):
+        # The QR refresh ends with a stable sort of eigenvalue estimates (matrix_functions.py:848-850); estimates tied
+        # within their rounding error come out in either order depending on the host's BLAS kernels and thread count
+        # (the run of this very oracle on another machine differs from the fixture by 4e-3 after 50 steps for that
+        # reason alone).  The fixture records the order of the reference's run; ties, and only ties, follow it.
+        align_oracle_to_fixture(opt, z, reordered)
     worst = 0.0
     for s, grads in grad_stream(c):
         opt.step(grads)
@@ -87,7 +94,8 @@ def test_benchmark_horizons_match_reference(name):
             got = [i for blk in opt.last_newton_iterations for i in blk]
             assert got == [int(v) for v in z["newton_iterations"][s - 1] if v >= 0], s
     final = max(rel_err(p.reshape(-1)[::37], z[f"final_p{i}"]) for i, p in enumerate(params))
-    print(f"{name}: oracle vs reference, worst per-step {worst:.2e}, final {final:.2e}")
+    print(f"{name}: oracle vs reference, worst per-step {worst:.2e}, final {final:.2e}; tied columns put in the "
+          f"reference run's order: {sum(m for *_, m, _ in reordered)}")
     assert worst < 1e-5 and final < 1e-5
 
 
