@@ -204,7 +204,8 @@ int32_t sa_compute_root_inverses_newton_f64(sa_plan* plan, float bias_correction
  * orthogonal to rounding, cyclic Jacobi in fp64 on X^T A X finishes); the weights of
  * matrix_inverse_root_from_eigendecomposition (`stability`, `rank_rtol`, `rank_atol`, `roots` as in
  * sa_compute_root_inverses_eigh) and X = Q diag(w) Q^T in double; the result cast to the fp32 inverse-root state
- * (shampoo_preconditioner_list.py:672-678).  sweeps_out: Jacobi sweeps in fp64 (at most 16; SA_FACTOR_NOT_CONVERGED beyond). */
+ * (shampoo_preconditioner_list.py:672-678).  sweeps_out: Jacobi sweeps in fp64 (at most max_sweeps, which also bounds the fp32 solver's
+ * sweeps; SA_FACTOR_NOT_CONVERGED beyond; two to three are usual, the fp32 eigenvectors leave X^T A X diagonal to 1e-6). */
 int32_t sa_compute_root_inverses_eigh_f64(sa_plan* plan, float bias_correction2, double epsilon, const float* roots,
                                           int32_t stability, double rank_rtol, double rank_atol, int32_t max_sweeps,
                                           int32_t* sweeps_out, int32_t* status_out, void* stream);

@@ -17,6 +17,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 namespace sa {
 
@@ -81,6 +82,7 @@ struct GemmScalars {
 // generic to the compiler, and a generic (flat) load counts against the LDS counter as well as the memory counter:
 // the wait in front of the first MFMA of a slab would then also wait for the next slab's operands.
 typedef float vfloat4 __attribute__((ext_vector_type(4)));
+typedef unsigned int vuint4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ float4 gload4(const float* p) {
   const vfloat4 v = *(const __attribute__((address_space(1))) vfloat4*)p;
   return make_float4(v.x, v.y, v.z, v.w);
@@ -225,8 +227,9 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
   // two operand buffers of two slabs each; a slab is at least 32 x 36 floats, what a wavefront of the mirror epilogue
   // stages through the same memory
   constexpr int SLAB = (BK * LDS_STRIDE > 1152) ? BK * LDS_STRIDE : 1152;
-  __shared__ __attribute__((aligned(16))) float As[2][SLAB];
-  __shared__ __attribute__((aligned(16))) float Bs[2][SLAB];
+  __shared__ __attribute__((aligned(16))) float smem[4 * SLAB];
+  float (*As)[SLAB] = reinterpret_cast<float (*)[SLAB]>(smem);
+  float (*Bs)[SLAB] = reinterpret_cast<float (*)[SLAB]>(smem + 2 * SLAB);
   __shared__ float red[4];
   static_assert(WB == 2 || (EPI != EPI_STORE_SQNORM), "per-tile partial sums are laid out for 128 x 128 tiles");
 
@@ -312,7 +315,133 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
 
   float4 ra[WB], rb[WB];
   const int slabs = (K + BK - 1) / BK;
+  // In a diagonal tile of a symmetric product the wavefront below the diagonal computes nothing that is kept (its
+  // quadrant is the mirror image of the one above): it takes part in the loads and barriers and leaves the matrix
+  // cores of its SIMD to the other workgroups there.
+  const bool idle_quadrant = TRI && tm == tn && wm > wn;
 
+  if constexpr (!EDGE) {
+    // ---- unguarded main loop, written so that nothing but matrix instructions uses the vector ALU inside it: a VALU
+    // instruction of any wavefront takes the issue slot the matrix pipe of that SIMD would have used.
+    //  * global addresses = uniform base (scalar registers, advanced per slab by the scalar ALU) + a per-thread 32-bit offset
+    //    that never changes;
+    //  * LDS addresses = a per-thread base that never changes + immediate offsets (the slab loop is unrolled by two so
+    //    that the buffer a slab lives in is a compile-time constant; fragment reads are volatile so that the compiler keeps
+    //    them as single reads with 16-bit offsets instead of pairing them behind a recomputed base).
+    unsigned aoff[WB], boff[WB];
+    int ast[WB], bst[WB];  // LDS store positions (floats)
+#pragma unroll
+    for (int i = 0; i < WB; ++i) {
+      const int idx = threadIdx.x + i * GEMM_THREADS;
+      constexpr int PER_ROW = 16 * WB;
+      if (AL == A_MK) { aoff[i] = (unsigned)((idx >> 2) * (int)lda + ((idx & 3) << 2)); ast[i] = ((idx & 3) << 2) * LDS_STRIDE + (idx >> 2); }
+      else { aoff[i] = (unsigned)((idx / PER_ROW) * (int)lda + ((idx % PER_ROW) << 2)); ast[i] = (idx / PER_ROW) * LDS_STRIDE + ((idx % PER_ROW) << 2); }
+      if (BL == B_NK) { boff[i] = (unsigned)((idx >> 2) * (int)ldb + ((idx & 3) << 2)); bst[i] = ((idx & 3) << 2) * LDS_STRIDE + (idx >> 2); }
+      else { boff[i] = (unsigned)((idx / PER_ROW) * (int)ldb + ((idx % PER_ROW) << 2)); bst[i] = (idx / PER_ROW) * LDS_STRIDE + ((idx % PER_ROW) << 2); }
+    }
+    // buffer resources over the two operands: the per-thread offset goes into the instruction's vector offset, the slab's
+    // position into its scalar offset (advanced by the scalar ALU)
+    const float* abase = (AL == A_MK) ? A + (long long)m0 * lda : A + m0;
+    const float* bbase = (BL == B_NK) ? B + (long long)n0 * ldb : B + n0;
+    const long long a_floats = ((AL == A_MK) ? (long long)(M - 1) * lda + K : (long long)(K - 1) * lda + M) - (abase - A);
+    const long long b_floats = ((BL == B_NK) ? (long long)(N - 1) * ldb + K : (long long)(K - 1) * ldb + N) - (bbase - B);
+    const __amdgpu_buffer_rsrc_t ares = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(abase), 0, (int)(a_floats * 4), 0x00020000);
+    const __amdgpu_buffer_rsrc_t bres = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(bbase), 0, (int)(b_floats * 4), 0x00020000);
+    const int astep = ((AL == A_MK) ? BK : BK * (int)lda) * 4;
+    const int bstep = ((BL == B_NK) ? BK : BK * (int)ldb) * 4;
+    int apos = 0, bpos = 0;  // bytes
+    auto fetch = [&]() {
+#pragma unroll
+      for (int i = 0; i < WB; ++i) {
+        const vuint4 v = __builtin_amdgcn_raw_buffer_load_b128(ares, (int)(aoff[i] * 4), apos, 0);
+        ra[i] = make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+      }
+#pragma unroll
+      for (int i = 0; i < WB; ++i) {
+        const vuint4 v = __builtin_amdgcn_raw_buffer_load_b128(bres, (int)(boff[i] * 4), bpos, 0);
+        rb[i] = make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+      }
+      apos += astep;
+      bpos += bstep;
+    };
+    auto scale = [&]() {
+      if (a_div != 1.0f) {
+#pragma unroll
+        for (int i = 0; i < WB; ++i) { ra[i].x /= a_div; ra[i].y /= a_div; ra[i].z /= a_div; ra[i].w /= a_div; }
+      }
+      if (b_div != 1.0f) {
+#pragma unroll
+        for (int i = 0; i < WB; ++i) { rb[i].x /= b_div; rb[i].y /= b_div; rb[i].z /= b_div; rb[i].w /= b_div; }
+      }
+    };
+    auto stash = [&](auto cur_tag) {
+      constexpr int CUR = decltype(cur_tag)::value;
+#pragma unroll
+      for (int i = 0; i < WB; ++i) {
+        if (AL == A_MK) {
+          smem[CUR * SLAB + ast[i]] = ra[i].x; smem[CUR * SLAB + ast[i] + LDS_STRIDE] = ra[i].y;
+          smem[CUR * SLAB + ast[i] + 2 * LDS_STRIDE] = ra[i].z; smem[CUR * SLAB + ast[i] + 3 * LDS_STRIDE] = ra[i].w;
+        } else {
+          *reinterpret_cast<float4*>(&smem[CUR * SLAB + ast[i]]) = ra[i];
+        }
+        if (BL == B_NK) {
+          smem[(2 + CUR) * SLAB + bst[i]] = rb[i].x; smem[(2 + CUR) * SLAB + bst[i] + LDS_STRIDE] = rb[i].y;
+          smem[(2 + CUR) * SLAB + bst[i] + 2 * LDS_STRIDE] = rb[i].z; smem[(2 + CUR) * SLAB + bst[i] + 3 * LDS_STRIDE] = rb[i].w;
+        } else {
+          *reinterpret_cast<float4*>(&smem[(2 + CUR) * SLAB + bst[i]]) = rb[i];
+        }
+      }
+    };
+    // four fragment bases the compiler cannot relate to each other: every read then keeps its own 16-bit immediate offset
+    typedef const __attribute__((address_space(3))) float* lds_ptr;
+    lds_ptr fa[WB], fb[WB];
+#pragma unroll
+    for (int i = 0; i < WB; ++i) {
+      fa[i] = (lds_ptr)smem + (wm * 32 * WB + l32 + h * LDS_STRIDE + 32 * i);
+      fb[i] = (lds_ptr)smem + (wn * 32 * WB + l32 + h * LDS_STRIDE + 32 * i);
+      asm volatile("" : "+v"(fa[i]));
+      asm volatile("" : "+v"(fb[i]));
+    }
+    auto multiply = [&](auto cur_tag) {
+      constexpr int CUR = decltype(cur_tag)::value;
+      if (!idle_quadrant) {
+#pragma unroll
+        for (int ks = 0; ks < BK / 2; ++ks) {
+          float a[WB], b[WB];
+#pragma unroll
+          for (int i = 0; i < WB; ++i) a[i] = fa[i][CUR * SLAB + ks * 2 * LDS_STRIDE];
+#pragma unroll
+          for (int i = 0; i < WB; ++i) b[i] = fb[i][(2 + CUR) * SLAB + ks * 2 * LDS_STRIDE];
+#pragma unroll
+          for (int i = 0; i < WB; ++i)
+#pragma unroll
+            for (int j = 0; j < WB; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);  // the fragments of one k-step are live at a time
+        }
+      }
+    };
+    using T0 = std::integral_constant<int, 0>;
+    using T1 = std::integral_constant<int, 1>;
+    fetch();
+    scale();
+    stash(T0{});
+    __syncthreads();
+    // K is a multiple of 2 BK here.  Every slab fetches its successor without asking whether there is one: the buffer
+    // resources end with the operands, so the fetch behind the last slab reads zeros (or the next rows of a k-contiguous
+    // operand) that no one multiplies.
+    for (int s = 0; s < slabs; s += 2) {
+      fetch();
+      multiply(T0{});
+      scale();
+      stash(T1{});
+      __syncthreads();
+      fetch();
+      multiply(T1{});
+      scale();
+      stash(T0{});
+      __syncthreads();
+    }
+  } else {
   slab_load<AL == A_MK, EDGE, WB>(A, lda, m0, M, 0, K, avec, ra);
   slab_load<BL == B_NK, EDGE, WB>(B, ldb, n0, N, 0, K, bvec, rb);
   if (a_div != 1.0f) {
@@ -326,11 +455,6 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
   slab_store<AL == A_MK, WB>(As[0], ra);
   slab_store<BL == B_NK, WB>(Bs[0], rb);
   __syncthreads();
-
-  // In a diagonal tile of a symmetric product the wavefront below the diagonal computes nothing that is kept (its
-  // quadrant is the mirror image of the one above): it takes part in the loads and barriers and leaves the matrix
-  // cores of its SIMD to the other workgroups there.
-  const bool idle_quadrant = TRI && tm == tn && wm > wn;
 
   for (int s = 0; s < slabs; ++s) {
     const int cur = s & 1;
@@ -368,6 +492,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
       slab_store<BL == B_NK, WB>(Bs[cur ^ 1], rb);
     }
     __syncthreads();
+  }
   }
 
   // ---- epilogue -------------------------------------------------------------------

@@ -10,6 +10,7 @@
 #include <cstdio>
 #include <cstring>
 #include <map>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -120,6 +121,19 @@ struct Table {
   }
 };
 
+inline long long operand_bytes(long long rows, long long cols, long long ld) { return ((rows - 1) * ld + cols) * (long long)sizeof(float); }
+
+// May the unguarded main loop of grouped_gemm_kernel run this problem?  Whole 128 x 128 tiles, K in pairs of slabs,
+// 16-byte loads, and operands that a buffer resource can span (its extent is a 32-bit byte count).
+inline bool unguarded_ok(const GemmProblem& p) {
+  if (p.M % BM || p.N % BN || p.K % (2 * BK) || !p.a_vec || !p.b_vec) return false;
+  const long long lim = 0x7fffffffLL;
+  // either layout: the larger of the two possible extents bounds the operand
+  const long long a = std::max(operand_bytes(p.M, p.K, p.lda), operand_bytes(p.K, p.M, p.lda));
+  const long long b = std::max(operand_bytes(p.N, p.K, p.ldb), operand_bytes(p.K, p.N, p.ldb));
+  return a < lim && b < lim;
+}
+
 struct GemmTable {
   Table<GemmProblem> t;
   int total_tiles = 0;
@@ -139,7 +153,7 @@ struct GemmTable {
     p.tiles_n_s = (p.N + 63) / 64;
     p.tile_begin_s = total_tiles_s;
     total_tiles_s += triangular ? p.tiles_n_s * (p.tiles_n_s + 1) / 2 : p.tiles_m_s * p.tiles_n_s;
-    if (p.M % BM || p.N % BN || p.K % BK || !p.a_vec || !p.b_vec) aligned = false;
+    if (!unguarded_ok(p)) aligned = false;
     build.push_back(p);
   }
   int commit(hipStream_t s) {
@@ -3463,7 +3477,7 @@ static int sa_compute_root_inverses_eigh_f64_wave(sa_plan* p, float bias_correct
     const Eig64Job* sub = p->t_eig64.dev + k0;
     bool done = false;
     int sweep = 0;
-    for (; sweep < 16 && !done; ++sweep) {
+    for (; sweep < max_sweeps && !done; ++sweep) {
       HIPCHECK(hipMemsetAsync(p->d_iters, 0, F * sizeof(int), s));
       for (int r = 0; r < nn - 1; ++r) {
         hipLaunchKernelGGL(eig64_rotations_kernel, dim3((nn / 2 + 255) / 256, m), dim3(256), 0, s, sub, r);
@@ -4293,13 +4307,18 @@ int32_t sa_plan_import_dense_state(sa_plan* p, void* const* dense_factor, void* 
 // Single GEMM (tests, microbenchmarks)
 // --------------------------------------------------------------------------------------------
 
-static GemmTable g_test_table;
+// One problem table per stream (work on one stream is ordered, so a table is never rewritten under a launch that still
+// reads it), guarded by a mutex: the call may be made from several threads.
+static std::mutex g_test_mutex;
+static std::map<hipStream_t, GemmTable> g_test_tables;
 
 int32_t sa_gemm_f32(const float* A, const float* B, float* C, int32_t M, int32_t N, int32_t K, int64_t lda, int64_t ldb,
                     int64_t ldc, int32_t a_layout, int32_t b_layout, int32_t batch, int64_t stride_a, int64_t stride_b,
                     int64_t stride_c, void* stream) {
   if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0 || batch <= 0) return fail(SA_ERR_INVALID, "sa_gemm_f32: bad arguments");
   hipStream_t s = static_cast<hipStream_t>(stream);
+  std::lock_guard<std::mutex> lock(g_test_mutex);
+  GemmTable& g_test_table = g_test_tables[s];
   g_test_table.clear();
   for (int i = 0; i < batch; ++i) {
     GemmProblem q{};
@@ -4348,6 +4367,9 @@ __global__ void static_gemm_fill_kernel(GemmProblem* __restrict__ table, const f
   q.tiles_m = (M + BM - 1) / BM;
   q.tiles_n = (N + BN - 1) / BN;
   q.tile_begin = i * q.tiles_m * q.tiles_n;
+  q.tiles_m_s = (M + 63) / 64;
+  q.tiles_n_s = (N + 63) / 64;
+  q.tile_begin_s = i * q.tiles_m_s * q.tiles_n_s;
   q.d = 0;
   q.a_vec = a_vec; q.b_vec = b_vec;
   table[i] = q;
@@ -4366,6 +4388,13 @@ int32_t sa_gemm_f32_static(const float* A, const float* B, float* C, int32_t M, 
   int dev = -1;
   HIPCHECK(hipGetDevice(&dev));
   if (dev < 0 || dev >= STATIC_GEMM_MAX_DEVICES) return fail(SA_ERR_UNSUPPORTED, "sa_gemm_f32_static: device index out of range");
+  if (stream) {  // the table is the current device's copy of the array: the stream must belong to that device
+    int stream_dev = -1;
+    HIPCHECK(hipStreamGetDevice(static_cast<hipStream_t>(stream), &stream_dev));
+    if (stream_dev != dev)
+      return fail(SA_ERR_INVALID, "sa_gemm_f32_static: the stream belongs to device " + std::to_string(stream_dev) +
+                                      " but device " + std::to_string(dev) + " is current");
+  }
   if (!g_scratch_ptr[dev]) {
     void* ptr = nullptr;
     HIPCHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
@@ -4377,7 +4406,9 @@ int32_t sa_gemm_f32_static(const float* A, const float* B, float* C, int32_t M, 
   // every problem of the batch may use 16-byte loads only if the first one may and the batch stride keeps the alignment
   const int a_vec = (vec_ok(A, lda) && (batch == 1 || stride_a % 4 == 0)) ? 1 : 0;
   const int b_vec = (vec_ok(B, ldb) && (batch == 1 || stride_b % 4 == 0)) ? 1 : 0;
-  const bool aligned = M % BM == 0 && N % BN == 0 && K % BK == 0 && a_vec && b_vec;
+  GemmProblem shape{};
+  shape.M = M; shape.N = N; shape.K = K; shape.lda = lda; shape.ldb = ldb; shape.a_vec = a_vec; shape.b_vec = b_vec;
+  const bool aligned = unguarded_ok(shape);
   hipLaunchKernelGGL(static_gemm_fill_kernel, dim3((batch + 255) / 256), dim3(256), 0, s, table, A, B, C, M, N, K, (long long)lda,
                      (long long)ldb, (long long)ldc, batch, (long long)stride_a, (long long)stride_b, (long long)stride_c, a_vec,
                      b_vec);

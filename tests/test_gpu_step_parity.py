@@ -376,6 +376,46 @@ def test_float64_eigendecomposition_of_a_rank_deficient_factor_follows_the_refer
     assert err < 1e-5
 
 
+def test_float64_eigendecomposition_through_both_solvers_in_one_batch():
+    """EigenConfig on float64 factors of orders 600 and 130 in one group: the fp32 eigenvectors of the first come from the
+    tridiagonal solver (as rows), those of the second from block Jacobi (as columns); the two padded orders go through the
+    fp64 polish and Jacobi sweeps in one batch.  The stored inverse root must be the reference's function of the stored
+    float64 factor (matrix_functions.py:256-263, 306-366), with torch.linalg.eigh in float64 as the judge."""
+    import optimizers_amd as oa
+    from oracle.shampoo_oracle import unpack_triu
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(5)
+    p = torch.nn.Parameter(torch.zeros(600, 130, device=dev))
+    eps = 1e-12
+    pc = oa.RootInvShampooPreconditionerConfig(factor_matrix_dtype=torch.float64)
+    opt = oa.DistributedShampoo([p], lr=1e-3, betas=(0.9, 0.999), epsilon=eps, max_preconditioner_dim=1024,
+                                precondition_frequency=1, start_preconditioning_step=6, preconditioner_config=pc,
+                                grafting_config=oa.AdamPreconditionerConfig(beta2=0.999, epsilon=1e-8))
+    for _ in range(6):  # the order-600 factor has full rank from the fifth gradient on
+        p.grad = (0.1 * torch.randn(600, 130, generator=g)).to(dev)
+        opt.step()
+    ng = opt._groups[0]
+    sweeps = list(ng.last_newton_iterations)
+    st = opt.state[p]["block_0"]["shampoo"]
+    bc2 = float(torch.tensor(1.0) - 0.999 ** torch.tensor(6))
+    worst = 0.0
+    for j, d in enumerate((600, 130)):
+        a = unpack_triu(st["factor_matrices"][j].cpu(), d)
+        assert a.dtype == torch.float64
+        x = unpack_triu(st["inv_factor_matrices"][j].cpu(), d).double()
+        lam, q = torch.linalg.eigh(a / bc2 + eps * torch.eye(d, dtype=torch.float64))
+        if float(lam[0]) < eps:
+            lam = (lam - lam[0]) + eps
+        want = (q * lam.pow(-0.25)) @ q.T
+        err = rel_err(x, want)
+        worst = max(worst, err)
+        print(f"order {d}: inverse root vs float64 eigh {err:.2e}, condition number {float(lam[-1] / lam[0]):.1e}, "
+              f"fp64 Jacobi sweeps {sweeps[j]}", flush=True)
+        assert err < 1e-6, (d, err)  # the fp32 state rounds the result to 6e-8
+        assert 1 <= sweeps[j] <= 6, sweeps
+
+
 @pytest.mark.parametrize("kind", ["newton", "eigh"])
 def test_float64_factors_at_moderate_size(kind):
     """The fp64 GEMM path over several 128 x 128 tiles per factor (orders 1100 -> 9 x 9 tiles, 400, 300, 200) against the

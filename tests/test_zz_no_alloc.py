@@ -46,6 +46,29 @@ def test_static_gemm_equals_gemm_on_two_calls_in_a_row(layouts):
         assert ((got.double() - ref).norm() / ref.norm()).item() < 2e-6
 
 
+def test_static_gemm_leaves_the_free_device_memory_unchanged():
+    """The property the entry point exists for: after one warm-up call (code object, symbol address) a call takes no
+    device memory - hipMemGetInfo reads the same free byte count before and after, with the output allocated beforehand."""
+    from optimizers_amd import native
+
+    lib = native.load()
+    M, N, K, batch = 256, 256, 128, 4
+    A, B = _operands(M, N, K, 0, 0, batch, seed=3)
+    C = torch.empty((batch, M, N), device=A.device, dtype=torch.float32)
+    st = native.current_stream_ptr(A.device)
+    args = (A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, N, N, 0, 0, batch, M * K, K * N, M * N, st)
+    native.check(lib.sa_gemm_f32_static(*args), "sa_gemm_f32_static")  # warm-up
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        native.check(lib.sa_gemm_f32_static(*args), "sa_gemm_f32_static")
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, (free_before, free_after)
+    ref = torch.bmm(A.double(), B.double())
+    assert ((C.double() - ref).norm() / ref.norm()).item() < 2e-6
+
+
 def test_static_gemm_rejects_a_batch_beyond_its_table():
     from optimizers_amd import native
 
