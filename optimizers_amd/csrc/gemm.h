@@ -314,6 +314,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
   float4 ra[WB], rb[WB];
+  float4 ra2[WB], rb2[WB];
   const int slabs = (K + BK - 1) / BK;
   // In a diagonal tile of a symmetric product the wavefront below the diagonal computes nothing that is kept (its
   // quadrant is the mirror image of the one above): it takes part in the loads and barriers and leaves the matrix
@@ -350,45 +351,45 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
     const int astep = ((AL == A_MK) ? BK : BK * (int)lda) * 4;
     const int bstep = ((BL == B_NK) ? BK : BK * (int)ldb) * 4;
     int apos = 0, bpos = 0;  // bytes
-    auto fetch = [&]() {
+    auto fetch_into = [&](float4 (&xa)[WB], float4 (&xb)[WB]) {
 #pragma unroll
       for (int i = 0; i < WB; ++i) {
         const vuint4 v = __builtin_amdgcn_raw_buffer_load_b128(ares, (int)(aoff[i] * 4), apos, 0);
-        ra[i] = make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+        xa[i] = make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
       }
 #pragma unroll
       for (int i = 0; i < WB; ++i) {
         const vuint4 v = __builtin_amdgcn_raw_buffer_load_b128(bres, (int)(boff[i] * 4), bpos, 0);
-        rb[i] = make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+        xb[i] = make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
       }
       apos += astep;
       bpos += bstep;
     };
-    auto scale = [&]() {
+    auto scale = [&](float4 (&xa)[WB], float4 (&xb)[WB]) {
       if (a_div != 1.0f) {
 #pragma unroll
-        for (int i = 0; i < WB; ++i) { ra[i].x /= a_div; ra[i].y /= a_div; ra[i].z /= a_div; ra[i].w /= a_div; }
+        for (int i = 0; i < WB; ++i) { xa[i].x /= a_div; xa[i].y /= a_div; xa[i].z /= a_div; xa[i].w /= a_div; }
       }
       if (b_div != 1.0f) {
 #pragma unroll
-        for (int i = 0; i < WB; ++i) { rb[i].x /= b_div; rb[i].y /= b_div; rb[i].z /= b_div; rb[i].w /= b_div; }
+        for (int i = 0; i < WB; ++i) { xb[i].x /= b_div; xb[i].y /= b_div; xb[i].z /= b_div; xb[i].w /= b_div; }
       }
     };
-    auto stash = [&](auto cur_tag) {
+    auto stash_from = [&](auto cur_tag, float4 (&xa)[WB], float4 (&xb)[WB]) {
       constexpr int CUR = decltype(cur_tag)::value;
 #pragma unroll
       for (int i = 0; i < WB; ++i) {
         if (AL == A_MK) {
-          smem[CUR * SLAB + ast[i]] = ra[i].x; smem[CUR * SLAB + ast[i] + LDS_STRIDE] = ra[i].y;
-          smem[CUR * SLAB + ast[i] + 2 * LDS_STRIDE] = ra[i].z; smem[CUR * SLAB + ast[i] + 3 * LDS_STRIDE] = ra[i].w;
+          smem[CUR * SLAB + ast[i]] = xa[i].x; smem[CUR * SLAB + ast[i] + LDS_STRIDE] = xa[i].y;
+          smem[CUR * SLAB + ast[i] + 2 * LDS_STRIDE] = xa[i].z; smem[CUR * SLAB + ast[i] + 3 * LDS_STRIDE] = xa[i].w;
         } else {
-          *reinterpret_cast<float4*>(&smem[CUR * SLAB + ast[i]]) = ra[i];
+          *reinterpret_cast<float4*>(&smem[CUR * SLAB + ast[i]]) = xa[i];
         }
         if (BL == B_NK) {
-          smem[(2 + CUR) * SLAB + bst[i]] = rb[i].x; smem[(2 + CUR) * SLAB + bst[i] + LDS_STRIDE] = rb[i].y;
-          smem[(2 + CUR) * SLAB + bst[i] + 2 * LDS_STRIDE] = rb[i].z; smem[(2 + CUR) * SLAB + bst[i] + 3 * LDS_STRIDE] = rb[i].w;
+          smem[(2 + CUR) * SLAB + bst[i]] = xb[i].x; smem[(2 + CUR) * SLAB + bst[i] + LDS_STRIDE] = xb[i].y;
+          smem[(2 + CUR) * SLAB + bst[i] + 2 * LDS_STRIDE] = xb[i].z; smem[(2 + CUR) * SLAB + bst[i] + 3 * LDS_STRIDE] = xb[i].w;
         } else {
-          *reinterpret_cast<float4*>(&smem[(2 + CUR) * SLAB + bst[i]]) = rb[i];
+          *reinterpret_cast<float4*>(&smem[(2 + CUR) * SLAB + bst[i]]) = xb[i];
         }
       }
     };
@@ -422,23 +423,22 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
     };
     using T0 = std::integral_constant<int, 0>;
     using T1 = std::integral_constant<int, 1>;
-    fetch();
-    scale();
-    stash(T0{});
+    // slab 0 -> buffer 0; slab 1 in flight in set 2; inside the loop every slab is fetched two slabs ahead of its use
+    fetch_into(ra, rb);
+    scale(ra, rb);
+    stash_from(T0{}, ra, rb);
+    fetch_into(ra2, rb2);
     __syncthreads();
-    // K is a multiple of 2 BK here.  Every slab fetches its successor without asking whether there is one: the buffer
-    // resources end with the operands, so the fetch behind the last slab reads zeros (or the next rows of a k-contiguous
-    // operand) that no one multiplies.
     for (int s = 0; s < slabs; s += 2) {
-      fetch();
-      multiply(T0{});
-      scale();
-      stash(T1{});
+      fetch_into(ra, rb);           // slab s + 2
+      multiply(T0{});               // slab s
+      scale(ra2, rb2);
+      stash_from(T1{}, ra2, rb2);   // slab s + 1
       __syncthreads();
-      fetch();
-      multiply(T1{});
-      scale();
-      stash(T0{});
+      fetch_into(ra2, rb2);         // slab s + 3
+      multiply(T1{});               // slab s + 1
+      scale(ra, rb);
+      stash_from(T0{}, ra, rb);     // slab s + 2
       __syncthreads();
     }
   } else {
