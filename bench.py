@@ -12,7 +12,10 @@ this box's host cores: on the whole workload where that takes a minute or two, w
 scaled sample beside it as a cross-check; on a bounded sample alone where the workload amortizes
 an eigendecomposition or QR refresh), next to a torch_gpu_baseline object (the same oracle's torch
 ops on this GPU: what the reference's own code path costs here).  Every step draws its own
-gradient set.
+gradient set.  The default workload's line also carries "other_workloads": the other four benchmark
+configurations timed natively in the same process, one amortisation period each, without baselines
+(--no-other-workloads skips them).  `--gemm-standalone` times stand-alone launches of the grouped GEMM
+through the C ABI instead of a workload.
 """
 
 from __future__ import annotations
@@ -265,52 +268,18 @@ def cpu_baseline(workload: dict, name: str, budget_s: float = 25.0, whole: bool 
     return out
 
 
-def kind_of(workload: dict) -> str:
-    return workload.get("preconditioner", "newton")
-
-
-def main() -> None:
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=None, help="default: 6, or one precondition_frequency period")
-    ap.add_argument("--warmup", type=int, default=None, help="default: 3, or start_preconditioning_step")
-    ap.add_argument("--workload", default="llama3_8b_layer", choices=sorted(WORKLOADS))
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--symmetric-newton", type=int, default=2, choices=(0, 1, 2),
-                    help="coupled-Newton products: 0 = full GEMMs (the reference's arithmetic), 1 = upper triangle "
-                         "mirrored, 2 (library default) = per factor, mirrored only while the factor's previous solve "
-                         "converged within 14 iterations (condition number <~ 1e4)")
-    ap.add_argument("--eigh-solver", type=int, default=0, choices=(0, 1, 2),
-                    help="EigenConfig root inverse: 0 = by order (library default), 1 = block Jacobi, 2 = tridiagonalisation")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run one plain 1 GiB copy kernel (sa::copy_kernel) so that rocprofv3 --pmc FETCH_SIZE / "
-                         "WRITE_SIZE readings can be scaled against a kernel of known traffic")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this build targets one MI355X; --gpus must be 1 (no collectives, no sharding).")
-
+def measure(lib, name: str, workload: dict, steps: int, warmup: int, device, symmetric_newton: int, calibrate_copy: bool) -> dict:
+    """Builds the workload, runs `warmup` untimed and `steps` timed steps and returns the JSON object of the run."""
     import torch
 
     from optimizers_amd import native
 
-    assert torch.cuda.is_available(), "bench.py needs an MI355X"
-    device = torch.device("cuda:0")
-    workload = WORKLOADS[args.workload]
     start = workload.get("start_preconditioning_step", START_PRECONDITIONING_STEP)
     freq = workload.get("precondition_frequency", 1)
-    if args.steps is None:
-        args.steps = 6 if freq == 1 else freq  # one full amortisation period
-    if args.warmup is None:
-        args.warmup = max(3, start + 1) if freq == 1 else start  # the first refresh is part of the warm-up
-    if args.warmup < start:
-        sys.exit(f"bench.py: --warmup must be >= {start} so that timed steps are full Shampoo steps.")
-    lib = native.load()
-    lib.sa_set_symmetric_newton(args.symmetric_newton)
-    lib.sa_set_eigh_solver(args.eigh_solver)
     params, opt = build(workload, device)
     n_params = sum(p.numel() for p in params)
 
-    total = args.warmup + args.steps
+    total = warmup + steps
     # one pre-generated gradient set per step (seed 1000 + step), up to 32 sets (28 GB on the Llama layer); only longer
     # runs, or the workloads that name a smaller number, cycle through them
     n_sets = min(total, workload.get("distinct_gradients", 32))
@@ -322,10 +291,10 @@ def main() -> None:
             p.grad = g
         opt.step()
 
-    for i in range(args.warmup):
+    for i in range(warmup):
         one_step(i)
     torch.cuda.synchronize()
-    if args.calibrate_copy:
+    if calibrate_copy:
         src = torch.ones(1 << 28, device=device)  # 1 GiB
         dst = torch.empty_like(src)
         native.check(lib.sa_copy_f32(src.data_ptr(), dst.data_ptr(), src.numel(), native.current_stream_ptr(device)), "sa_copy_f32")
@@ -354,7 +323,7 @@ def main() -> None:
     executed = 0.0
     iters = []
     t0 = time.perf_counter()
-    for i in range(args.warmup, total):
+    for i in range(warmup, total):
         one_step(i)
         # phase timers are read after the step; the call synchronises on the recorded events only
         for ph in phases:
@@ -364,13 +333,16 @@ def main() -> None:
                 acc[ph][1] += lib.sa_phase_flops(ph.encode())
                 acc[ph][2] += lib.sa_phase_launches(ph.encode())
         executed += max(lib.sa_phase_executed_flops(b"newton_gemm"), 0.0)
+        # forget this step's spans: a phase that the next step does not enter (an amortized computation) must not be read twice
+        lib.sa_set_profiling(0)
+        lib.sa_set_profiling(1)
         iters.append(list(opt._groups[0].last_newton_iterations))
         if kind_of(workload) == "newton":
             full_product_flops += sum(it * w for it, w in zip(iters[-1], full_product_flops_per_iteration))
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     lib.sa_set_profiling(0)
-    ms_per_step = 1e3 * elapsed / args.steps
+    ms_per_step = 1e3 * elapsed / steps
 
     kind = workload.get("preconditioner", "newton")
     dominant = DOMINANT_PHASE[kind]
@@ -392,13 +364,13 @@ def main() -> None:
         "frac": achieved / peak,
         # HBM bytes per launch: not measured by this run (hardware counters need rocprofv3); the figure, when there
         # is one for this workload and product policy, is copied from the committed counter profile named beside it
-        "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get((args.workload, args.symmetric_newton)),
-        "traffic_source": (TRAFFIC_SOURCE if (args.workload, args.symmetric_newton) in MEASURED_TRAFFIC_BYTES_PER_LAUNCH
+        "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get((name, symmetric_newton)),
+        "traffic_source": (TRAFFIC_SOURCE if (name, symmetric_newton) in MEASURED_TRAFFIC_BYTES_PER_LAUNCH
                            else None),
         # `achieved` bills the algorithmic flops of the products issued (2 d^3 for a full product,
         # d^2 (d + 1) for a symmetric one); `executed_frac` adds the padding and the mirrored halves of
         # diagonal tiles, i.e. what the matrix cores really sustained.
-        "symmetric_products_policy": args.symmetric_newton,
+        "symmetric_products_policy": symmetric_newton,
         # the same iterations billed as the reference's full products (2 d^3 each); above `executed_frac` because a
         # symmetric product computes only the tiles on and above the diagonal
         # NOT a utilisation: the reference's work per second (what its full GEMMs would have to sustain to match this time)
@@ -416,17 +388,17 @@ def main() -> None:
     for ph in ("syrk", "precondition_gemm", "jacobi", "qr_refresh", "eigenbasis_rotation", "form_q"):
         ms, work, n = acc[ph]
         if ms > 0:
-            detail[ph] = {"ms_per_step": ms / args.steps, "TFLOP/s": work / (ms * 1e-3) / 1e12,
+            detail[ph] = {"ms_per_step": ms / steps, "TFLOP/s": work / (ms * 1e-3) / 1e12,
                           "frac_of_fp32_mfma_peak": work / (ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS}
     for ph in ("tridiagonal_ql", "tridiagonal_eig"):
         if acc[ph][0] > 0:
-            detail[ph] = {"ms_per_step": acc[ph][0] / args.steps}
+            detail[ph] = {"ms_per_step": acc[ph][0] / steps}
     for ph in ("grafting", "apply", "tridiagonalize"):
         ms, work, n = acc[ph]
         if ms > 0:
-            detail[ph] = {"ms_per_step": ms / args.steps, "GB/s": work / (ms * 1e-3) / 1e9,
+            detail[ph] = {"ms_per_step": ms / steps, "GB/s": work / (ms * 1e-3) / 1e9,
                           "frac_of_hbm_peak": work / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS}
-    detail[dominant] = dict(detail.get(dominant, {}), ms_per_step=ng_ms / args.steps)
+    detail[dominant] = dict(detail.get(dominant, {}), ms_per_step=ng_ms / steps)
     flat = [x for row in iters for x in row if x > 0]
     detail["newton_iterations_mean"] = sum(flat) / max(len(flat), 1)
     detail["newton_iterations_max"] = max(flat) if flat else 0
@@ -436,8 +408,8 @@ def main() -> None:
         "value": ms_per_step,
         "unit": "ms/step",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
+        "steps": steps,
+        "warmup": warmup,
         "ms_per_step": ms_per_step,
         "higher_is_better": False,
         "scaling": "weak",
@@ -445,7 +417,7 @@ def main() -> None:
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": args.workload,
+            "workload": name,
             "parameters": n_params,
             "max_preconditioner_dim": workload["max_preconditioner_dim"],
             "precondition_frequency": freq,
@@ -458,10 +430,113 @@ def main() -> None:
         "roofline": roofline,
         "phases": detail,
     }
+    out["dominant_phase"] = dominant
+    del opt, params, grads, ng
+    torch.cuda.empty_cache()
+    return out
+
+
+def gemm_standalone(lib, device, reps: int = 100) -> dict:
+    """Stand-alone launches of the grouped GEMM through the C ABI (sa_gemm_f32: full products, plain store): the Newton
+    shapes of the Llama layer (108 x 2048^3) and of GPT-2 (400 x 768^3), operand layouts A as stored / A through its
+    transpose, `reps` launches back to back timed with events on the launch stream (about 1.3 s per row: sustained
+    clocks, not a burst)."""
+    import torch
+
+    from optimizers_amd import native
+
+    rows = []
+    for batch, n in ((108, 2048), (400, 768)):
+        a = torch.randn(batch, n, n, device=device) * 0.01
+        b = torch.randn(batch, n, n, device=device) * 0.01
+        c = torch.empty(batch, n, n, device=device)
+        st = native.current_stream_ptr(device)
+        for layout, label in ((0, "A[m][k]"), (1, "A[k][m]")):
+            call = lambda: native.check(lib.sa_gemm_f32(a.data_ptr(), b.data_ptr(), c.data_ptr(), n, n, n, n, n, n, layout, 0,
+                                                        batch, n * n, n * n, n * n, st), "sa_gemm_f32")
+            call()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                call()
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / reps
+            tf = 2.0 * n**3 * batch / (ms * 1e-3) / 1e12
+            rows.append({"batch": batch, "order": n, "A": label, "ms_per_launch": ms, "TFLOP/s": tf,
+                         "frac_of_fp32_mfma_peak": tf / PEAK_FP32_MFMA_TFLOPS})
+        del a, b, c
+    return {"metric": "grouped_gemm_standalone", "unit": "TFLOP/s", "launches_per_row": reps, "rows": rows}
+
+
+def kind_of(workload: dict) -> str:
+    return workload.get("preconditioner", "newton")
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None, help="default: 6, or one precondition_frequency period")
+    ap.add_argument("--warmup", type=int, default=None, help="default: 3, or start_preconditioning_step")
+    ap.add_argument("--workload", default="llama3_8b_layer", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--symmetric-newton", type=int, default=2, choices=(0, 1, 2),
+                    help="coupled-Newton products: 0 = full GEMMs (the reference's arithmetic), 1 = upper triangle "
+                         "mirrored, 2 (library default) = per factor, mirrored only while the factor's previous solve "
+                         "converged within 14 iterations (condition number <~ 1e4)")
+    ap.add_argument("--eigh-solver", type=int, default=0, choices=(0, 1, 2),
+                    help="EigenConfig root inverse: 0 = by order (library default), 1 = block Jacobi, 2 = tridiagonalisation")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="default run only: skip the native timing of the other four benchmark configurations")
+    ap.add_argument("--gemm-standalone", action="store_true",
+                    help="time stand-alone launches of the grouped GEMM (sa_gemm_f32, 108 products of order 2048 and 400 of "
+                         "order 768, full products) instead of a workload")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 1 GiB copy kernel (sa::copy_kernel) so that rocprofv3 --pmc FETCH_SIZE / "
+                         "WRITE_SIZE readings can be scaled against a kernel of known traffic")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build targets one MI355X; --gpus must be 1 (no collectives, no sharding).")
+
+    import torch
+
+    from optimizers_amd import native
+
+    assert torch.cuda.is_available(), "bench.py needs an MI355X"
+    device = torch.device("cuda:0")
+    workload = WORKLOADS[args.workload]
+    start = workload.get("start_preconditioning_step", START_PRECONDITIONING_STEP)
+    freq = workload.get("precondition_frequency", 1)
+    if args.steps is None:
+        args.steps = 6 if freq == 1 else freq  # one full amortisation period
+    if args.warmup is None:
+        args.warmup = max(3, start + 1) if freq == 1 else start  # the first refresh is part of the warm-up
+    if args.warmup < start:
+        sys.exit(f"bench.py: --warmup must be >= {start} so that timed steps are full Shampoo steps.")
+    lib = native.load()
+    lib.sa_set_symmetric_newton(args.symmetric_newton)
+    lib.sa_set_eigh_solver(args.eigh_solver)
+    if args.gemm_standalone:
+        print(json.dumps(gemm_standalone(lib, device)))
+        return
+    out = measure(lib, args.workload, workload, args.steps, args.warmup, device, args.symmetric_newton, args.calibrate_copy)
+    if args.workload == "llama3_8b_layer" and not args.no_other_workloads:
+        # the other four benchmark configurations, natively, one amortisation period each (no baselines)
+        others = {}
+        for name in ("cfg1", "gpt2_small", "llama3_8b_layer_soap", "large_block_eigh"):
+            w = WORKLOADS[name]
+            st, fr = w.get("start_preconditioning_step", START_PRECONDITIONING_STEP), w.get("precondition_frequency", 1)
+            steps = 6 if fr == 1 else fr
+            warm = max(3, st + 1) if fr == 1 else st
+            m = measure(lib, name, w, steps, warm, device, args.symmetric_newton, False)
+            r = m["roofline"]
+            others[name] = {"ms_per_step": m["ms_per_step"], "steps": steps, "warmup": warm,
+                            "dominant_phase": m["dominant_phase"], "bound": r["bound"], "achieved": r["achieved"],
+                            "unit": r["unit"], "frac": r["frac"], "phases": m["phases"]}
+        out["other_workloads"] = others
+    out.pop("dominant_phase", None)
     if not args.no_cpu_baseline:
-        # the native optimizer's state is released first: the oracle keeps dense factors and inverse roots of its own
-        del opt, params, grads, ng
-        torch.cuda.empty_cache()
         out["torch_gpu_baseline"] = torch_gpu_baseline(workload, args.workload, device)
         torch.cuda.empty_cache()
         out["cpu_baseline"] = cpu_baseline(workload, args.workload)

@@ -1089,6 +1089,9 @@ static_assert(sizeof(sa_block_desc) == 168, "sa_block_desc layout changed: bump 
 static_assert(sizeof(sa_step_scalars) == 76, "sa_step_scalars layout changed: bump sa_abi_version and the ctypes mirror");
 
 int32_t sa_set_profiling(int32_t enabled) {
+  // switching the timers on forgets what earlier runs recorded: a phase that the coming calls never enter reads -1
+  if (enabled != 0 && !g_profiling)
+    for (auto& kv : g_phases) { kv.second.used = 0; kv.second.work = 0.0; kv.second.executed = 0.0; kv.second.launches = 0; }
   g_profiling = enabled != 0;
   return SA_OK;
 }
