@@ -149,6 +149,15 @@ int32_t sa_plan_num_factors(const sa_plan* plan);
  * in the eigenbasis (after the caller wrote inv_factor, eigenvectors or filtered_grad itself, e.g. load_state_dict). */
 int32_t sa_plan_invalidate_inverse_cache(sa_plan* plan);
 
+/* How sa_compute_root_inverses_newton schedules a batch (no counterpart in the reference, whose loop runs factor by
+ * factor): a batch whose stages are launches of fewer than `tiles` 128 x 128 tiles is cut into two halves that iterate
+ * side by side, the second on a stream the plan owns (joined with the caller's stream before the call's result pass).
+ * Every stage of an iteration waits for the one before it, so a short launch alone leaves the chip idle while it ramps
+ * up and drains; the other half's launch fills that.  The factors are independent: results and iteration counts are the
+ * bits of the unsplit run.  Default 0 = never split: on the GPT-2 parameter set the two halves measured slower than the
+ * whole batch (73.8 against 69.6 ms per step), so the switch is kept for experiments only. */
+int32_t sa_plan_set_newton_split_tiles(sa_plan* plan, int32_t tiles);
+
 /* Gradients of this step, one device pointer per block (same rows/cols/ld as the block); NULL
  * masks a block out of every following call (shampoo_distributor.py:269-277). */
 int32_t sa_plan_bind_gradients(sa_plan* plan, float* const* grads, void* stream);

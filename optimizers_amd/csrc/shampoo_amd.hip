@@ -10,6 +10,7 @@
 #include <cstdio>
 #include <cstring>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -369,6 +370,18 @@ struct sa_plan {
   // Newton, [0] full products / [1] symmetric products: X*M_p with M_p^2 per parity, power chain, M update per parity
   GemmTable nt_a[2][2], nt_pow[2][8], nt_m[2][2];
   GemmTable nt_a0[2];  // first iteration: launch A without X M_p (the init kernel wrote it)
+  // Second lane of the coupled Newton iteration: a batch whose launches are too short to keep the chip busy between one
+  // dependent stage and the next is cut into two halves that iterate side by side on two streams, each with its own
+  // tables, control pass and mailbox.
+  struct NewtonLane2 {
+    GemmTable a[2][2], pow[2][8], m[2][2], a0[2];
+    Table<int> ids;
+    Table<SymFactor> sym;
+  } nlane2;
+  hipStream_t newton_stream = nullptr;
+  hipEvent_t newton_ev[2] = {nullptr, nullptr};
+  unsigned int ctl_seq2 = 0;
+  int newton_split_tiles = 0;  // batches of fewer tiles per stage iterate as two halves (0 = never, the default)
   GemmTable nt_h[8];      // Horner products of the higher-order iteration
   // mode products of order-3 blocks: [mode 1 | mode 0 | mode 2][first stage (divides by bias_correction1)][last stage (norm)]
   GemmTable g3[3][2][2];
@@ -1297,7 +1310,7 @@ int32_t sa_plan_create(const sa_block_desc* blocks, int32_t n_blocks, sa_plan** 
   p->d_flags_in = p->d_report + 2 * F;
   p->d_flags = p->d_report + 3 * F;
   p->d_first_bad = p->d_report + 4 * F;
-  *p->h_mailbox = 0ull;
+  std::memset(p->h_mailbox, 0, 64);
   *plan_out = p;
   return SA_OK;
 }
@@ -1311,6 +1324,13 @@ void sa_plan_destroy(sa_plan* p) {
                        &p->nt_m[1][1]})
     g->destroy();
   for (auto& row : p->nt_pow) for (auto& g : row) g.destroy();
+  for (auto& row : p->nlane2.a) for (auto& g : row) g.destroy();
+  for (auto& row : p->nlane2.pow) for (auto& g : row) g.destroy();
+  for (auto& row : p->nlane2.m) for (auto& g : row) g.destroy();
+  for (auto& g : p->nlane2.a0) g.destroy();
+  p->nlane2.ids.destroy(); p->nlane2.sym.destroy();
+  if (p->newton_stream) (void)hipStreamDestroy(p->newton_stream);
+  for (hipEvent_t e : p->newton_ev) if (e) (void)hipEventDestroy(e);
   for (auto& g : p->nt_h) g.t.destroy();
   for (auto& a : p->g3) for (auto& b2 : a) for (auto& g : b2) g.t.destroy();
   for (auto& a : p->e3) for (auto& b2 : a) for (auto& c2 : b2) for (auto& g : c2) g.t.destroy();
@@ -1358,6 +1378,13 @@ int32_t sa_plan_bind_workspace(sa_plan* p, void* workspace, int64_t bytes) {
 int32_t sa_plan_num_factors(const sa_plan* p) { return p ? (int32_t)p->factors.size() : 0; }
 
 int64_t sa_plan_shared_rotation_steps(const sa_plan* p) { return p ? p->shared_rotation_steps : 0; }
+
+int32_t sa_plan_set_newton_split_tiles(sa_plan* p, int32_t tiles) {
+  if (!p) return fail(SA_ERR_INVALID, "NULL plan");
+  if (tiles < 0) return fail(SA_ERR_INVALID, "sa_plan_set_newton_split_tiles: the tile count must not be negative");
+  p->newton_split_tiles = tiles;
+  return SA_OK;
+}
 
 int32_t sa_plan_invalidate_inverse_cache(sa_plan* p) {
   if (!p) return fail(SA_ERR_INVALID, "NULL plan");
@@ -1626,8 +1653,8 @@ static int power_ops(int root, std::vector<char>* ops) {
 // Waits, without synchronising the stream, until the control pass with sequence number `seq` (or a later one) has
 // reported into the plan's mailbox; *n_active = the count it reported.  The stream is queried now and then so that a
 // failed launch or a lost report ends the wait with an error instead of a hang.
-static int wait_for_control(sa_plan* p, unsigned int seq, hipStream_t s, int* n_active) {
-  volatile unsigned long long* box = p->h_mailbox;
+static int wait_for_control(sa_plan* p, unsigned int seq, hipStream_t s, int* n_active, int lane = 0) {
+  volatile unsigned long long* box = p->h_mailbox + 4 * lane;
   const auto t0 = std::chrono::steady_clock::now();
   for (unsigned long long spin = 0;; ++spin) {
     const unsigned long long v = *box;
@@ -1646,173 +1673,266 @@ static int wait_for_control(sa_plan* p, unsigned int seq, hipStream_t s, int* n_
   }
 }
 
-// `symmetric[i]` selects the product variant of ids[i].  The loop is enqueued ahead of the device: the control pass
-// after every iteration decides on the device which factors go on (the products skip the others), and the host only
-// follows its reports, `lag` iterations behind, to stop enqueueing once no factor is active.  Nothing is read back
-// here; iteration counts, final errors and parities stay in the plan's device arrays.
-static int newton_batch(sa_plan* p, const std::vector<int>& ids, const std::vector<char>& symmetric, int root, float eps,
-                        float bc2, int max_iter, float tol, hipStream_t s, int* launches_acc) {
-  const int n = (int)ids.size();
-  if (n == 0) return SA_OK;
-  // torch.linalg.matrix_power(M_p, root) as a chain of products
+// One batch of coupled Newton iterations (all factors of one root, or one half of them) as a resumable run:
+// start() enqueues the start matrices and uploads the tables, every step() enqueues one iteration.  `symmetric[i]`
+// selects the product variant of ids[i].  The loop is enqueued ahead of the device: the control pass after every
+// iteration decides on the device which factors go on (the products skip the others), and the host only follows its
+// reports, `lag` iterations behind, to stop enqueueing once no factor is active.  Nothing is read back here; iteration
+// counts, final errors and parities stay in the plan's device arrays.  Lane 0 uses the plan's own tables, mailbox word
+// and the caller's stream; lane 1 the second set, for a half that iterates beside lane 0 on the plan's second stream.
+struct NewtonRun {
+  sa_plan* p = nullptr;
+  std::vector<int> ids;
+  std::vector<char> symmetric;
+  int root = 0, max_iter = 0, lane = 0;
+  float eps = 0.f, bc2 = 1.f, tol = 0.f;
+  hipStream_t s = nullptr;
+  // state
+  int n = 0, parity = 0, lag = 1, expected = 0, it = 0;
+  unsigned int seq0 = 0;
+  bool done = false;
+  bool spans = true;  // record one timing span per iteration (off when two lanes overlap: their spans would add up twice)
+  float alpha = 0.f, one_minus_alpha = 0.f;
   std::vector<char> ops;
-  SACHECK(power_ops(root, &ops));
-  const float alpha = (float)(-1.0 / root);          // M.mul(alpha)
-  const float one_minus_alpha = (float)(1.0 - (-1.0 / root));  // .add_(I, alpha = 1 - alpha)
 
-  // ---- init: M0, Mp0, X0, err --------------------------------------------------------------
-  SACHECK(p->t_ids.begin(n));
-  std::memcpy(p->t_ids.host, ids.data(), n * sizeof(int));
-  SACHECK(p->t_ids.upload(s));
-  // the batch starts active with cleared counters; every other factor keeps its state
-  hipLaunchKernelGGL(newton_activate_kernel, dim3(1), dim3(256), 0, s,
-                     NewtonCtl{p->d_err, p->d_active, p->d_iters, p->d_final_parity, p->d_final_err}, p->t_ids.dev, n);
-  HIPCHECK(hipGetLastError());
-  SACHECK(p->t_sym.begin(n));
-  int sym_tiles = 0;
-  for (int i = 0; i < n; ++i) {
-    const Factor& f = p->factors[ids[i]];
-    SymFactor& S = p->t_sym.host[i];
-    std::memset(&S, 0, sizeof(S));
-    S.packed_in = f.factor;
-    S.scale = p->scale_of(ids[i]);
-    S.dense_out[0] = newton_buf(p, NB_M0, f);
-    S.dense_out[1] = newton_buf(p, NB_MP0, f);
-    S.dense_out[2] = newton_buf(p, NB_X0, f);
-    S.dense_out[3] = newton_buf(p, NB_X1, f);
-    S.err_bits = p->d_err + ids[i];
-    S.norm_partial = p->f(p->off_norm_partial) + f.norm_off;
-    S.n_norm_partial = f.norm_chunks;
-    S.d = f.d; S.dpad = f.dpad; S.tiles = f.dpad / ST; S.root = root; S.enabled = 1;
-    S.tile_begin = sym_tiles;
-    sym_tiles += S.tiles * (S.tiles + 1) / 2;
-  }
-  SACHECK(p->t_sym.upload(s));
-  hipLaunchKernelGGL((sym_pass_kernel<SYM_NEWTON_INIT>), dim3(sym_tiles), dim3(256), 0, s, p->t_sym.dev, n, bc2, eps,
-                     alpha, one_minus_alpha);
-  HIPCHECK(hipGetLastError());
+  GemmTable (&nt_a())[2][2] { return lane ? p->nlane2.a : p->nt_a; }
+  GemmTable (&nt_pow())[2][8] { return lane ? p->nlane2.pow : p->nt_pow; }
+  GemmTable (&nt_m())[2][2] { return lane ? p->nlane2.m : p->nt_m; }
+  GemmTable (&nt_a0())[2] { return lane ? p->nlane2.a0 : p->nt_a0; }
+  Table<int>& t_ids() { return lane ? p->nlane2.ids : p->t_ids; }
+  Table<SymFactor>& t_sym() { return lane ? p->nlane2.sym : p->t_sym; }
+  unsigned int& seq() { return lane ? p->ctl_seq2 : p->ctl_seq; }
+  int* d_nactive() { return p->d_nactive + 8 * lane; }
+  unsigned long long* d_mailbox() { return p->d_mailbox + 4 * lane; }
+  NewtonCtl ctl() { return NewtonCtl{p->d_err, p->d_active, p->d_iters, p->d_final_parity, p->d_final_err}; }
 
-  // ---- GEMM tables -------------------------------------------------------------------------
-  for (int v = 0; v < 2; ++v) {
-    for (int par = 0; par < 2; ++par) { p->nt_a[v][par].clear(); p->nt_m[v][par].clear(); }
-    p->nt_a0[v].clear();
-    for (int k = 0; k < 8; ++k) p->nt_pow[v][k].clear();
-  }
-  auto prob = [&](const Factor& f, const float* A, const float* B, float* C) {
-    GemmProblem q{};
-    q.A = A; q.B = B; q.C = C;
-    q.lda = q.ldb = q.ldc = f.dpad;
-    q.M = q.N = q.K = f.dpad;
-    q.d = f.d;
-    q.a_vec = q.b_vec = 1;
-    q.active = p->d_active + (&f - p->factors.data());
-    return q;
-  };
-  for (int i = 0; i < n; ++i) {
-    const Factor& f = p->factors[ids[i]];
-    const bool sym = symmetric[i] != 0;
-    const int v = sym ? 1 : 0;
-    // buffer that finally holds M_p^root (depends only on the chain length)
-    const float* power = nullptr;
-    for (int par = 0; par < 2; ++par) {
-      const float* X = newton_buf(p, par ? NB_X1 : NB_X0, f);
-      float* Xn = newton_buf(p, par ? NB_X0 : NB_X1, f);
-      const float* Mp = newton_buf(p, par ? NB_MP1 : NB_MP0, f);
-      float* Mpn = newton_buf(p, par ? NB_MP0 : NB_MP1, f);
-      const float* M = newton_buf(p, par ? NB_M1 : NB_M0, f);
-      float* Mn = newton_buf(p, par ? NB_M0 : NB_M1, f);
-      float* S1 = newton_buf(p, NB_S1, f);
-      float* S2 = newton_buf(p, NB_S2, f);
-      // launch A: X <- X M_p, and the first squaring if the root needs one
-      p->nt_a[v][par].add(prob(f, X, Mp, Xn), sym);
-      if (!ops.empty()) p->nt_a[v][par].add(prob(f, Mp, Mp, S1), sym);
-      if (!ops.empty() && par == 0) p->nt_a0[v].add(prob(f, Mp, Mp, S1), sym);
-      // the remaining chain reads only S1 / S2 / M_p of this parity
-      const float* cur = ops.empty() ? Mp : S1;
-      int slot = par * 4;  // nt_pow[0..3] parity 0, [4..7] parity 1
-      float* pong[2] = {S2, S1};
-      int which = 0;
-      for (size_t q = 1; q < ops.size(); ++q) {
-        p->nt_pow[v][slot++].add(prob(f, cur, ops[q] == 'S' ? cur : Mp, pong[which]), sym);
-        cur = pong[which];
-        which ^= 1;
+  int start() {
+    n = (int)ids.size();
+    if (n == 0) { done = true; return SA_OK; }
+    // torch.linalg.matrix_power(M_p, root) as a chain of products
+    SACHECK(power_ops(root, &ops));
+    alpha = (float)(-1.0 / root);                   // M.mul(alpha)
+    one_minus_alpha = (float)(1.0 - (-1.0 / root));  // .add_(I, alpha = 1 - alpha)
+
+    // ---- init: M0, Mp0, X0, err --------------------------------------------------------------
+    SACHECK(t_ids().begin(n));
+    std::memcpy(t_ids().host, ids.data(), n * sizeof(int));
+    SACHECK(t_ids().upload(s));
+    // the batch starts active with cleared counters; every other factor keeps its state
+    hipLaunchKernelGGL(newton_activate_kernel, dim3(1), dim3(256), 0, s, ctl(), t_ids().dev, n);
+    HIPCHECK(hipGetLastError());
+    SACHECK(t_sym().begin(n));
+    int sym_tiles = 0;
+    for (int i = 0; i < n; ++i) {
+      const Factor& f = p->factors[ids[i]];
+      SymFactor& S = t_sym().host[i];
+      std::memset(&S, 0, sizeof(S));
+      S.packed_in = f.factor;
+      S.scale = p->scale_of(ids[i]);
+      S.dense_out[0] = newton_buf(p, NB_M0, f);
+      S.dense_out[1] = newton_buf(p, NB_MP0, f);
+      S.dense_out[2] = newton_buf(p, NB_X0, f);
+      S.dense_out[3] = newton_buf(p, NB_X1, f);
+      S.err_bits = p->d_err + ids[i];
+      S.norm_partial = p->f(p->off_norm_partial) + f.norm_off;
+      S.n_norm_partial = f.norm_chunks;
+      S.d = f.d; S.dpad = f.dpad; S.tiles = f.dpad / ST; S.root = root; S.enabled = 1;
+      S.tile_begin = sym_tiles;
+      sym_tiles += S.tiles * (S.tiles + 1) / 2;
+    }
+    SACHECK(t_sym().upload(s));
+    hipLaunchKernelGGL((sym_pass_kernel<SYM_NEWTON_INIT>), dim3(sym_tiles), dim3(256), 0, s, t_sym().dev, n, bc2, eps,
+                       alpha, one_minus_alpha);
+    HIPCHECK(hipGetLastError());
+
+    // ---- GEMM tables -------------------------------------------------------------------------
+    for (int v = 0; v < 2; ++v) {
+      for (int par = 0; par < 2; ++par) { nt_a()[v][par].clear(); nt_m()[v][par].clear(); }
+      nt_a0()[v].clear();
+      for (int k = 0; k < 8; ++k) nt_pow()[v][k].clear();
+    }
+    auto prob = [&](const Factor& f, const float* A, const float* B, float* C) {
+      GemmProblem q{};
+      q.A = A; q.B = B; q.C = C;
+      q.lda = q.ldb = q.ldc = f.dpad;
+      q.M = q.N = q.K = f.dpad;
+      q.d = f.d;
+      q.a_vec = q.b_vec = 1;
+      q.active = p->d_active + (&f - p->factors.data());
+      return q;
+    };
+    for (int i = 0; i < n; ++i) {
+      const Factor& f = p->factors[ids[i]];
+      const bool sym = symmetric[i] != 0;
+      const int v = sym ? 1 : 0;
+      // buffer that finally holds M_p^root (depends only on the chain length)
+      const float* power = nullptr;
+      for (int par = 0; par < 2; ++par) {
+        const float* X = newton_buf(p, par ? NB_X1 : NB_X0, f);
+        float* Xn = newton_buf(p, par ? NB_X0 : NB_X1, f);
+        const float* Mp = newton_buf(p, par ? NB_MP1 : NB_MP0, f);
+        float* Mpn = newton_buf(p, par ? NB_MP0 : NB_MP1, f);
+        const float* M = newton_buf(p, par ? NB_M1 : NB_M0, f);
+        float* Mn = newton_buf(p, par ? NB_M0 : NB_M1, f);
+        float* S1 = newton_buf(p, NB_S1, f);
+        float* S2 = newton_buf(p, NB_S2, f);
+        // launch A: X <- X M_p, and the first squaring if the root needs one
+        nt_a()[v][par].add(prob(f, X, Mp, Xn), sym);
+        if (!ops.empty()) nt_a()[v][par].add(prob(f, Mp, Mp, S1), sym);
+        if (!ops.empty() && par == 0) nt_a0()[v].add(prob(f, Mp, Mp, S1), sym);
+        // the remaining chain reads only S1 / S2 / M_p of this parity
+        const float* cur = ops.empty() ? Mp : S1;
+        int slot = par * 4;  // nt_pow[0..3] parity 0, [4..7] parity 1
+        float* pong[2] = {S2, S1};
+        int which = 0;
+        for (size_t q = 1; q < ops.size(); ++q) {
+          nt_pow()[v][slot++].add(prob(f, cur, ops[q] == 'S' ? cur : Mp, pong[which]), sym);
+          cur = pong[which];
+          which ^= 1;
+        }
+        power = cur;
+        GemmProblem m = prob(f, power, M, Mn);
+        m.C2 = Mpn;
+        m.err_bits = p->d_err + ids[i];
+        nt_m()[v][par].add(m, sym);
       }
-      power = cur;
-      GemmProblem m = prob(f, power, M, Mn);
-      m.C2 = Mpn;
-      m.err_bits = p->d_err + ids[i];
-      p->nt_m[v][par].add(m, sym);
     }
-  }
-  for (int v = 0; v < 2; ++v) {
-    for (int par = 0; par < 2; ++par) { SACHECK(p->nt_a[v][par].commit(s)); SACHECK(p->nt_m[v][par].commit(s)); }
-    SACHECK(p->nt_a0[v].commit(s));
-    for (int k = 0; k < 8; ++k) SACHECK(p->nt_pow[v][k].commit(s));
+    for (int v = 0; v < 2; ++v) {
+      for (int par = 0; par < 2; ++par) { SACHECK(nt_a()[v][par].commit(s)); SACHECK(nt_m()[v][par].commit(s)); }
+      SACHECK(nt_a0()[v].commit(s));
+      for (int k = 0; k < 8; ++k) SACHECK(nt_pow()[v][k].commit(s));
+    }
+
+    parity = 0;
+    seq0 = seq();
+    hipLaunchKernelGGL(newton_control_kernel, dim3(1), dim3(256), 0, s, ctl(), t_ids().dev, n, tol, max_iter, parity, d_nactive(),
+                       d_mailbox(), ++seq());
+    HIPCHECK(hipGetLastError());
+    // small batches finish an iteration faster than the host enqueues the next one: stay further ahead there (an
+    // iteration enqueued after the last factor stopped costs a few launches of workgroups that exit at once)
+    long long tiles_per_stage = 0;
+    for (int v = 0; v < 2; ++v) tiles_per_stage += nt_m()[v][0].total_tiles;
+    lag = tiles_per_stage >= 2048 ? 1 : 3;
+    // Factors drift slowly between two amortized computations, so the batch most likely needs as many iterations as its
+    // slowest factor took last time.  Up to that count the host runs ahead as above; from there on it waits for the
+    // control pass that decides the very iteration it is about to enqueue, so that a correct guess enqueues no iteration
+    // that finds nothing to do (and a short guess costs one host round trip per extra iteration).
+    expected = 0;
+    if ((int)p->newton_history.size() == (int)p->factors.size()) {
+      for (int i : ids) {
+        if (p->newton_history[i] <= 0) { expected = 0; break; }
+        expected = std::max(expected, p->newton_history[i]);
+      }
+    }
+    it = 0;
+    done = false;
+    return SA_OK;
   }
 
-  NewtonCtl ctl{p->d_err, p->d_active, p->d_iters, p->d_final_parity, p->d_final_err};
-  int parity = 0;
-  const unsigned int seq0 = p->ctl_seq;
-  hipLaunchKernelGGL(newton_control_kernel, dim3(1), dim3(256), 0, s, ctl, p->t_ids.dev, n, tol, max_iter, parity, p->d_nactive,
-                     p->d_mailbox, ++p->ctl_seq);
-  HIPCHECK(hipGetLastError());
-  GemmScalars unit = unit_scalars();
-  GemmScalars msc = unit_scalars();
-  msc.mp_scale = alpha;
-  msc.mp_diag = one_minus_alpha;
-  // small batches finish an iteration faster than the host enqueues the next one: stay further ahead there (an
-  // iteration enqueued after the last factor stopped costs a few launches of workgroups that exit at once)
-  long long tiles_per_stage = 0;
-  for (int v = 0; v < 2; ++v) tiles_per_stage += p->nt_m[v][0].total_tiles;
-  const int lag = tiles_per_stage >= 2048 ? 1 : 3;
-  // Factors drift slowly between two amortized computations, so the batch most likely needs as many iterations as its
-  // slowest factor took last time.  Up to that count the host runs ahead as above; from there on it waits for the
-  // control pass that decides the very iteration it is about to enqueue, so that a correct guess enqueues no iteration
-  // that finds nothing to do (and a short guess costs one host round trip per extra iteration).
-  int expected = 0;
-  if ((int)p->newton_history.size() == (int)p->factors.size()) {
-    for (int i : ids) {
-      if (p->newton_history[i] <= 0) { expected = 0; break; }
-      expected = std::max(expected, p->newton_history[i]);
-    }
-  }
-  for (int it = 0; it < max_iter; ++it) {
-    // control pass k (k = 0 is the one above) decides iteration k; before iteration `it` is enqueued, pass it - lag
+  // Enqueues one more iteration, or finds that the batch has finished.
+  int step(int* launches_acc) {
+    if (done) return SA_OK;
+    if (it >= max_iter) { done = true; return SA_OK; }
+    // control pass k (k = 0 is the one of start()) decides iteration k; before iteration `it` is enqueued, pass it - lag
     // must have reported, and any newer report that shows no active factor ends the loop
     int n_active = 1;
     if (expected > 0 && it >= expected) {
-      SACHECK(wait_for_control(p, seq0 + 1 + (unsigned int)it, s, &n_active));
+      SACHECK(wait_for_control(p, seq0 + 1 + (unsigned int)it, s, &n_active, lane));
     } else if (it >= lag) {
-      SACHECK(wait_for_control(p, seq0 + 1 + (unsigned int)(it - lag), s, &n_active));
+      SACHECK(wait_for_control(p, seq0 + 1 + (unsigned int)(it - lag), s, &n_active, lane));
     } else {
-      const unsigned long long v = *(volatile unsigned long long*)p->h_mailbox;
+      const unsigned long long v = *(volatile unsigned long long*)(p->h_mailbox + 4 * lane);
       if ((unsigned int)(v >> 32) > seq0) n_active = (int)(unsigned int)(v & 0xffffffffull);
     }
-    if (n_active == 0) break;
+    if (n_active == 0) { done = true; return SA_OK; }
+    GemmScalars unit = unit_scalars();
+    GemmScalars msc = unit_scalars();
+    msc.mp_scale = alpha;
+    msc.mp_diag = one_minus_alpha;
     {
       int nl = 0;
       for (int v = 0; v < 2; ++v) {
-        nl += ((it == 0 ? p->nt_a0[v] : p->nt_a[v][parity]).total_tiles ? 1 : 0) + (p->nt_m[v][parity].total_tiles ? 1 : 0);
-        for (int k = 0; k < 4; ++k) nl += p->nt_pow[v][parity * 4 + k].total_tiles ? 1 : 0;
+        nl += ((it == 0 ? nt_a0()[v] : nt_a()[v][parity]).total_tiles ? 1 : 0) + (nt_m()[v][parity].total_tiles ? 1 : 0);
+        for (int k = 0; k < 4; ++k) nl += nt_pow()[v][parity * 4 + k].total_tiles ? 1 : 0;
       }
-      Span span("newton_gemm", s, 0.0, nl, false);
+      std::unique_ptr<Span> span;
+      if (spans) span.reset(new Span("newton_gemm", s, 0.0, nl, false));
+      else if (g_profiling) g_phases["newton_gemm"].launches += nl;
       // the two variants touch disjoint factors, so their launches of one stage are independent
       // symmetric variant: every operand is an exactly mirrored matrix, so A is read through its transpose (slabs
       // load and store as 16-byte rows instead of four scalar LDS stores per thread; same values, same results)
-      SACHECK((launch_gemm_live<A_KM, B_KN, EPI_STORE, false, true>(it == 0 ? p->nt_a0[1] : p->nt_a[1][parity], unit, s)));
-      SACHECK((launch_gemm_live<A_MK, B_KN, EPI_STORE, false, false>(it == 0 ? p->nt_a0[0] : p->nt_a[0][parity], unit, s)));
+      SACHECK((launch_gemm_live<A_KM, B_KN, EPI_STORE, false, true>(it == 0 ? nt_a0()[1] : nt_a()[1][parity], unit, s)));
+      SACHECK((launch_gemm_live<A_MK, B_KN, EPI_STORE, false, false>(it == 0 ? nt_a0()[0] : nt_a()[0][parity], unit, s)));
       for (int k = 0; k < 4; ++k) {
-        SACHECK((launch_gemm_live<A_KM, B_KN, EPI_STORE, false, true>(p->nt_pow[1][parity * 4 + k], unit, s)));
-        SACHECK((launch_gemm_live<A_MK, B_KN, EPI_STORE, false, false>(p->nt_pow[0][parity * 4 + k], unit, s)));
+        SACHECK((launch_gemm_live<A_KM, B_KN, EPI_STORE, false, true>(nt_pow()[1][parity * 4 + k], unit, s)));
+        SACHECK((launch_gemm_live<A_MK, B_KN, EPI_STORE, false, false>(nt_pow()[0][parity * 4 + k], unit, s)));
       }
-      SACHECK((launch_gemm_live<A_KM, B_KN, EPI_NEWTON_M, false, true>(p->nt_m[1][parity], msc, s)));
-      SACHECK((launch_gemm_live<A_MK, B_KN, EPI_NEWTON_M, false, false>(p->nt_m[0][parity], msc, s)));
+      SACHECK((launch_gemm_live<A_KM, B_KN, EPI_NEWTON_M, false, true>(nt_m()[1][parity], msc, s)));
+      SACHECK((launch_gemm_live<A_MK, B_KN, EPI_NEWTON_M, false, false>(nt_m()[0][parity], msc, s)));
       *launches_acc += nl;
     }
     parity ^= 1;
-    hipLaunchKernelGGL(newton_control_kernel, dim3(1), dim3(256), 0, s, ctl, p->t_ids.dev, n, tol, max_iter, parity, p->d_nactive,
-                       p->d_mailbox, ++p->ctl_seq);
+    hipLaunchKernelGGL(newton_control_kernel, dim3(1), dim3(256), 0, s, ctl(), t_ids().dev, n, tol, max_iter, parity, d_nactive(),
+                       d_mailbox(), ++seq());
     HIPCHECK(hipGetLastError());
+    ++it;
+    return SA_OK;
+  }
+};
+
+// The coupled Newton iterations of `ids` (one root).  Optionally (sa_plan_set_newton_split_tiles, off by default) a
+// batch whose stages are short launches is cut into two halves that iterate side by side, the second on the plan's own
+// stream: every stage of an iteration depends on the stage before it, so one half alone leaves the chip idle while a
+// launch ramps up and while its last workgroups finish, and the other half's launch can fill that.  The factors are
+// independent of each other, so the halves give the bits the whole batch gives.  Measured on the GPT-2 parameter set
+// the halves are slower (73.8 against 69.6 ms per step: two control passes, two tile-layout passes per stage and launches
+// of half the size cost more than the overlap returns), hence the default.
+static int newton_batch(sa_plan* p, const std::vector<int>& ids, const std::vector<char>& symmetric, int root, float eps,
+                        float bc2, int max_iter, float tol, hipStream_t s, int* launches_acc) {
+  if (ids.empty()) return SA_OK;
+  long long tiles = 0;
+  for (size_t i = 0; i < ids.size(); ++i) {
+    const long long t = p->factors[ids[i]].dpad / BM;
+    tiles += symmetric[i] ? t * (t + 1) / 2 : t * t;
+  }
+  const bool split = p->newton_split_tiles > 0 && tiles < p->newton_split_tiles && tiles >= 512 && ids.size() >= 8;
+  NewtonRun run[2];
+  for (int h = 0; h < 2; ++h) {
+    run[h].p = p; run[h].root = root; run[h].max_iter = max_iter; run[h].lane = h;
+    run[h].eps = eps; run[h].bc2 = bc2; run[h].tol = tol; run[h].s = s; run[h].spans = !split;
+  }
+  if (!split) {
+    run[0].ids = ids; run[0].symmetric = symmetric;
+    SACHECK(run[0].start());
+    while (!run[0].done) SACHECK(run[0].step(launches_acc));
+    return SA_OK;
+  }
+  // halves of equal work: the factors in descending order of their tile count, dealt out in turn
+  std::vector<int> order(ids.size());
+  for (size_t i = 0; i < order.size(); ++i) order[i] = (int)i;
+  std::stable_sort(order.begin(), order.end(), [&](int x, int y) { return p->factors[ids[x]].dpad > p->factors[ids[y]].dpad; });
+  for (size_t k = 0; k < order.size(); ++k) {
+    run[k & 1].ids.push_back(ids[order[k]]);
+    run[k & 1].symmetric.push_back(symmetric[order[k]]);
+  }
+  if (!p->newton_stream) HIPCHECK(hipStreamCreateWithFlags(&p->newton_stream, hipStreamNonBlocking));
+  for (hipEvent_t& e : p->newton_ev)
+    if (!e) HIPCHECK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+  run[1].s = p->newton_stream;
+  // the second stream starts behind everything the caller's stream holds so far, and the caller's stream goes on
+  // behind the second stream's last iteration
+  HIPCHECK(hipEventRecord(p->newton_ev[0], s));
+  HIPCHECK(hipStreamWaitEvent(p->newton_stream, p->newton_ev[0], 0));
+  {
+    Span span("newton_gemm", s, 0.0, 0, false);  // one span over both lanes: from here to the join on the caller's stream
+    SACHECK(run[0].start());
+    SACHECK(run[1].start());
+    while (!run[0].done || !run[1].done) {
+      SACHECK(run[0].step(launches_acc));
+      SACHECK(run[1].step(launches_acc));
+    }
+    HIPCHECK(hipEventRecord(p->newton_ev[1], p->newton_stream));
+    HIPCHECK(hipStreamWaitEvent(s, p->newton_ev[1], 0));
   }
   return SA_OK;
 }

@@ -324,6 +324,11 @@ class _NativeGroup(_AmortizedComputation):
     # SHAMPOO_AMD_SCRATCH_BYTES overrides it.
     scratch_budget_bytes: int | None = 32 << 30
 
+    # Coupled Newton: a batch whose stages are launches of fewer 128 x 128 tiles than this iterates as two halves side by
+    # side on two streams (sa_plan_set_newton_split_tiles; same bits either way).  None = the library's default (0 = never;
+    # the halves measured slower than the whole batch on the GPT-2 parameter set).  The environment variable SHAMPOO_AMD_NEWTON_SPLIT_TILES overrides it.
+    newton_split_tiles: int | None = None
+
     def __init__(self, optimizer: "DistributedShampoo", group: dict[str, Any], group_index: int) -> None:
         self.lib = native.load()
         self.group_index = group_index
@@ -593,6 +598,9 @@ class _NativeGroup(_AmortizedComputation):
                     self.lib.sa_plan_set_trace_scaling(self.plan, 1, pc.trace_scaling_exponent, group[EPSILON]),
                     "sa_plan_set_trace_scaling",
                 )
+            split = os.environ.get("SHAMPOO_AMD_NEWTON_SPLIT_TILES", self.newton_split_tiles)
+            if split is not None:
+                native.check(self.lib.sa_plan_set_newton_split_tiles(self.plan, int(split)), "sa_plan_set_newton_split_tiles")
             if self.kl:
                 try:
                     native.check(self.lib.sa_plan_set_kl_shampoo(self.plan, 1), "sa_plan_set_kl_shampoo")

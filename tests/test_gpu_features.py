@@ -592,3 +592,48 @@ def test_every_amortized_computation_gives_the_same_bits_in_waves(kind):
         assert torch.equal(a, b)
     for a, b in zip(s_c, s_u):
         assert torch.equal(a, b)
+
+
+def test_newton_batch_in_two_halves_side_by_side_gives_the_bits_of_the_whole_batch():
+    """sa_plan_set_newton_split_tiles: a batch of coupled Newton iterations whose stages are short launches iterates as
+    two halves on two streams.  Factors are independent of each other, so parameters, every state tensor and the
+    per-factor iteration counts must equal those of the unsplit run bit for bit; factors of five orders (1024, 768, 512,
+    384, 256), some of which converge earlier than others, and a second amortized computation that predicts its iteration
+    count from the first."""
+    import optimizers_amd as oa
+
+    g = torch.Generator().manual_seed(23)
+    from optimizers_amd import native
+
+    # 36 factors, 574 tiles per stage with symmetric products (a batch splits from 512 tiles and 8 factors on)
+    shapes = [(768, 512), (512, 384), (384, 256), (256, 768), (512, 512), (768, 768)] + [(1024, 1024)] * 6
+    init = [torch.randn(s, generator=g) * 0.1 for s in shapes]
+    # a few low-rank directions on top of the noise give the factors different condition numbers
+    lows = [(torch.randn(s[0], 4, generator=g), torch.randn(4, s[1], generator=g)) for s in shapes]
+    grads = [[0.1 * torch.randn(s, generator=g) + 0.05 * k * (a @ b) for k, (s, (a, b)) in enumerate(zip(shapes, lows))]
+             for _ in range(6)]
+    runs = []
+    for split_tiles in (1 << 20, 0):
+        ps = [torch.nn.Parameter(t.clone().to(DEV)) for t in init]
+        o = oa.DistributedShampoo(
+            ps, lr=0.01, betas=(0.9, 0.99), epsilon=1e-8, max_preconditioner_dim=1024, precondition_frequency=1,
+            start_preconditioning_step=4,
+            preconditioner_config=oa.RootInvShampooPreconditionerConfig(amortized_computation_config=oa.CoupledNewtonConfig()),
+            grafting_config=oa.AdamPreconditionerConfig(beta2=0.99, epsilon=1e-8))
+        ng = o._groups[0]
+        native.check(ng.lib.sa_plan_set_newton_split_tiles(ng.plan, split_tiles), "sa_plan_set_newton_split_tiles")
+        counts = []
+        for gs in grads:
+            for p, gr in zip(ps, gs):
+                p.grad = gr.to(DEV)
+            o.step()
+            counts.append(list(ng.last_newton_iterations))
+        torch.cuda.synchronize()
+        runs.append(([p.detach().clone() for p in ps], [t.clone() for _, _, _, t in ng._slots], counts))
+    (p_s, s_s, c_s), (p_u, s_u, c_u) = runs
+    print(f"iteration counts per amortized computation: {[c for c in c_u if c]}", flush=True)
+    assert c_s == c_u and any(len(set(c)) > 1 for c in c_u if c)
+    for a, b in zip(p_s, p_u):
+        assert torch.isfinite(a).all() and torch.equal(a, b)
+    for a, b in zip(s_s, s_u):
+        assert torch.equal(a, b)
