@@ -158,6 +158,15 @@ int32_t sa_plan_invalidate_inverse_cache(sa_plan* plan);
  * whole batch (73.8 against 69.6 ms per step), so the switch is kept for experiments only. */
 int32_t sa_plan_set_newton_split_tiles(sa_plan* plan, int32_t tiles);
 
+/* Lanes of the Householder tridiagonalisation behind sa_compute_root_inverses_eigh / sa_refresh_eigenbases_eigh for
+ * orders from 512 on (no counterpart in the reference, which calls torch.linalg.eigh factor by factor): a batch of
+ * factors is reduced in `lanes` parts (1..4, default 3; at least two factors per part), the parts after the first on
+ * streams the plan owns, joined with the caller's stream when the reduction ends.  Per column the reduction is one
+ * latency-bound workgroup per factor and one bandwidth-bound product, each waiting for the other; parts side by side fill
+ * each other's gaps (32 factors of order 4096: 415 / 376 / 361 / 527 ms with 1 / 2 / 3 / 4 lanes).  Same bits for every
+ * number of lanes. */
+int32_t sa_plan_set_tridiagonal_lanes(sa_plan* plan, int32_t lanes);
+
 /* Gradients of this step, one device pointer per block (same rows/cols/ld as the block); NULL
  * masks a block out of every following call (shampoo_distributor.py:269-277). */
 int32_t sa_plan_bind_gradients(sa_plan* plan, float* const* grads, void* stream);

@@ -411,7 +411,10 @@ struct sa_plan {
   GemmTable qr_aq, qr_b;
   Table<TrdJob> t_trd, t_trd_ql;  // every factor of the batch; those that take the QL iteration
   Table<TransposeJob> t_transpose;
-  hipStream_t trd_stream = nullptr;  // applies QL rotations concurrently with the next chase
+  hipStream_t trd_stream = nullptr;  // second lane of the tridiagonalisation; applies QL rotations concurrently with the next chase
+  int trd_lanes = 3;                 // the tridiagonalisation reduces a batch in this many parts side by side, one stream each
+  hipStream_t trd_lane_stream[2] = {nullptr, nullptr};
+  hipEvent_t trd_lane_ev[3] = {nullptr, nullptr, nullptr};
   hipEvent_t trd_ev[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
   Table<GemmProblem> t_trd_gemm;
   Table<RowScale> t_rowscale;
@@ -1343,6 +1346,8 @@ void sa_plan_destroy(sa_plan* p) {
   p->t_sym.destroy(); p->t_normjobs.destroy(); p->t_ids.destroy();
   p->t_jacobi.destroy(); p->t_sched.destroy(); p->t_eiginit.destroy(); p->t_eigfinal.destroy(); p->eig_gemm.t.destroy();
   if (p->trd_stream) { (void)hipStreamSynchronize(p->trd_stream); (void)hipStreamDestroy(p->trd_stream); }
+  for (hipStream_t q : p->trd_lane_stream) if (q) { (void)hipStreamSynchronize(q); (void)hipStreamDestroy(q); }
+  for (hipEvent_t e : p->trd_lane_ev) if (e) (void)hipEventDestroy(e);
   for (hipEvent_t e : p->trd_ev) if (e) (void)hipEventDestroy(e);
   p->t_dense_state[0].destroy(); p->t_dense_state[1].destroy();
   p->t_ids_out.destroy(); p->t_normjobs_out.destroy(); p->t_sym_out.destroy();
@@ -1378,6 +1383,13 @@ int32_t sa_plan_bind_workspace(sa_plan* p, void* workspace, int64_t bytes) {
 int32_t sa_plan_num_factors(const sa_plan* p) { return p ? (int32_t)p->factors.size() : 0; }
 
 int64_t sa_plan_shared_rotation_steps(const sa_plan* p) { return p ? p->shared_rotation_steps : 0; }
+
+int32_t sa_plan_set_tridiagonal_lanes(sa_plan* p, int32_t lanes) {
+  if (!p) return fail(SA_ERR_INVALID, "NULL plan");
+  if (lanes < 1 || lanes > 4) return fail(SA_ERR_INVALID, "sa_plan_set_tridiagonal_lanes: 1 to 4 lanes");
+  p->trd_lanes = lanes;
+  return SA_OK;
+}
 
 int32_t sa_plan_set_newton_split_tiles(sa_plan* p, int32_t tiles) {
   if (!p) return fail(SA_ERR_INVALID, "NULL plan");
@@ -2844,7 +2856,9 @@ inline long long trd_int_offset(const Factor& f) { return trd_tmat_offset(f) + (
 static int trd_side_stream(sa_plan* p) {
   if (p->trd_stream) return SA_OK;
   HIPCHECK(hipStreamCreateWithFlags(&p->trd_stream, hipStreamNonBlocking));  // default priority
+  for (hipStream_t& q : p->trd_lane_stream) HIPCHECK(hipStreamCreateWithFlags(&q, hipStreamNonBlocking));
   for (hipEvent_t& e : p->trd_ev) HIPCHECK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+  for (hipEvent_t& e : p->trd_lane_ev) HIPCHECK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
   return SA_OK;
 }
 
@@ -2909,7 +2923,16 @@ static int eigh_tridiagonal(sa_plan* p, const std::vector<int>& ids, hipStream_t
 
   // GEMM problem tables: [trailing update per panel | V T for every panel | G = (V T)^T Y per panel | Y -= V G per panel]
   std::vector<GemmProblem> probs;
-  std::vector<int> trail_off(panels), trail_tiles(panels, 0);
+  // The reduction runs the factors as one or two lanes (halves of the batch on two streams, see step 1): the trailing
+  // update has one table per panel and lane.
+  constexpr int ML = 4;  // most lanes
+  const int lanes = std::max(1, std::min({p->trd_lanes, ML, n / 2}));
+  int lane_n[ML] = {0, 0, 0, 0}, lane_first[ML] = {0, 0, 0, 0};
+  for (int h = 0; h < lanes; ++h) {
+    lane_n[h] = n / lanes + (h < n % lanes ? 1 : 0);
+    lane_first[h] = h == 0 ? 0 : lane_first[h - 1] + lane_n[h - 1];
+  }
+  std::vector<int> trail_off(ML * panels, 0), trail_tiles(ML * panels, 0);
   // small: walked in 64 x 64 tiles.  The rank-64 / rank-128 updates of a large matrix are a read-modify-write of that
   // matrix with a short product in between: small tiles put four times as many independent chains of loads on a CU
   // (rank-64 update of 32 triangles of order 4096: 0.62 ms against 0.83 ms with 128 x 128 tiles).
@@ -2934,19 +2957,21 @@ static int eigh_tridiagonal(sa_plan* p, const std::vector<int>& ids, hipStream_t
   };
   for (int b = 0; b < panels; ++b) {
     const int q0 = std::min(b * TRD_NB + TRD_NB, d - 1);  // first row / column after the panel
-    trail_off[b] = (int)probs.size();
-    if (d - q0 > 0)
-      for (int k = 0; k < n; ++k) {
-        const TrdJob& J = p->t_trd.host[k];
-        // every reader of the trailing matrix uses its lower triangle only: so does the update
-        // (the panels are stored by columns: both operands are read as K x M / K x N with unit stride along the rows).
-        // The updated region starts at the tile boundary at or in front of q0 and runs to the padded order, so that
-        // every tile is whole and aligned and the unguarded loader and epilogue serve: the rows and columns in front of
-        // q0 belong to the reduced part, which nothing reads again (the products multiply them by the zeros in front
-        // of the Householder vector), and the panel is zero beyond the order.
-        const int q0a = q0 & ~(BM - 1);
-        push(J.P1 + q0a, ld, J.P2 + q0a, ld, J.A + q0a * ld + q0a, ld, dpad - q0a, dpad - q0a, TRD_PW, &trail_tiles[b], true, true);
-      }
+    for (int h = 0; h < lanes; ++h) {
+      trail_off[ML * b + h] = (int)probs.size();
+      if (d - q0 > 0)
+        for (int k = lane_first[h]; k < lane_first[h] + lane_n[h]; ++k) {
+          const TrdJob& J = p->t_trd.host[k];
+          // every reader of the trailing matrix uses its lower triangle only: so does the update
+          // (the panels are stored by columns: both operands are read as K x M / K x N with unit stride along the rows).
+          // The updated region starts at the tile boundary at or in front of q0 and runs to the padded order, so that
+          // every tile is whole and aligned and the unguarded loader and epilogue serve: the rows and columns in front of
+          // q0 belong to the reduced part, which nothing reads again (the products multiply them by the zeros in front
+          // of the Householder vector), and the panel is zero beyond the order.
+          const int q0a = q0 & ~(BM - 1);
+          push(J.P1 + q0a, ld, J.P2 + q0a, ld, J.A + q0a * ld + q0a, ld, dpad - q0a, dpad - q0a, TRD_PW, &trail_tiles[ML * b + h], true, true);
+        }
+    }
   }
   // accumulation of Q1 = H_0 H_1 ... with block reflectors of 128 vectors, last block first (only the trailing corner
   // of Q differs from the identity then): [S = V^T V for every block | V T for every block | G = V^T Q per block |
@@ -3007,41 +3032,70 @@ static int eigh_tridiagonal(sa_plan* p, const std::vector<int>& ids, hipStream_t
                                    2 * TRD_MAX_DIM * (int)sizeof(float)));
       symv_attr = true;
     }
-    // Per column two launches on the one stream: the column step, then the product of that column together with the
-    // row terms of the next column step (extra workgroups of the same launch).
-    auto launch_col = [&](int j, int p0, int flags) {
-      if (d <= TRD_COL_THREADS) hipLaunchKernelGGL(trd_col_kernel<1>, dim3(n), dim3(TRD_COL_THREADS), 0, s, jobs, j, p0, flags);
-      else if (d <= 2 * TRD_COL_THREADS) hipLaunchKernelGGL(trd_col_kernel<2>, dim3(n), dim3(TRD_COL_THREADS), 0, s, jobs, j, p0, flags);
-      else if (d <= 4 * TRD_COL_THREADS) hipLaunchKernelGGL(trd_col_kernel<4>, dim3(n), dim3(TRD_COL_THREADS), 0, s, jobs, j, p0, flags);
-      else hipLaunchKernelGGL(trd_col_kernel<TRD_ROWS_PER_THREAD>, dim3(n), dim3(TRD_COL_THREADS), 0, s, jobs, j, p0, flags);
+    // Per column two launches on one stream: the column step, then the product of that column together with the
+    // row terms of the next column step (extra workgroups of the same launch).  The column step is one workgroup per
+    // factor and all latency, and every launch waits for the one before it, so a batch on one stream leaves most of the
+    // chip idle for a quarter of the time: the batch is reduced in `lanes` parts on as many streams (streams the plan
+    // owns take the parts after the first), whose column steps and launch gaps fall into each other's products: 32
+    // factors of order 4096 take 415 / 376 / 361 / 527 ms with 1 / 2 / 3 / 4 lanes (four streams are as many as the
+    // process has hardware queues).  The factors are independent of each other: the bits are those of one lane.
+    hipStream_t sl[ML] = {s, s, s, s};
+    if (lanes >= 2) {
+      SACHECK(trd_side_stream(p));
+      HIPCHECK(hipEventRecord(p->trd_ev[4], s));
+      for (int h = 1; h < lanes; ++h) {
+        sl[h] = h == 1 ? p->trd_stream : p->trd_lane_stream[h - 2];
+        HIPCHECK(hipStreamWaitEvent(sl[h], p->trd_ev[4], 0));
+      }
+    }
+    auto launch_col = [&](int h, int j, int p0, int flags) {
+      const TrdJob* jl = jobs + lane_first[h];
+      const dim3 g(lane_n[h]);
+      if (d <= TRD_COL_THREADS) hipLaunchKernelGGL(trd_col_kernel<1>, g, dim3(TRD_COL_THREADS), 0, sl[h], jl, j, p0, flags);
+      else if (d <= 2 * TRD_COL_THREADS) hipLaunchKernelGGL(trd_col_kernel<2>, g, dim3(TRD_COL_THREADS), 0, sl[h], jl, j, p0, flags);
+      else if (d <= 4 * TRD_COL_THREADS) hipLaunchKernelGGL(trd_col_kernel<4>, g, dim3(TRD_COL_THREADS), 0, sl[h], jl, j, p0, flags);
+      else hipLaunchKernelGGL(trd_col_kernel<TRD_ROWS_PER_THREAD>, g, dim3(TRD_COL_THREADS), 0, sl[h], jl, j, p0, flags);
     };
     // product of column j (j < 0: none) and the row terms of column step (aj, p0, flags)
-    auto launch_product = [&](int j, int aj, int p0, int flags) {
+    auto launch_product = [&](int h, int j, int aj, int p0, int flags) {
       int nbk = 0;
       if (j >= 0) {
         const int sbase = (j + 1) & ~(TRD_SB - 1);
         nbk = (d - sbase + TRD_SB - 1) / TRD_SB;
       }
       const size_t lds = std::max<size_t>(2 * (size_t)nbk * TRD_SB, 4 * TRD_NB) * sizeof(float);
-      hipLaunchKernelGGL(trd_symv_kernel, dim3(TRD_AUX_WGS + (nbk + 1) / 2, n), dim3(256), lds, s, jobs, j, TRD_AUX_WGS, aj, p0, flags);
+      hipLaunchKernelGGL(trd_symv_kernel, dim3(TRD_AUX_WGS + (nbk + 1) / 2, lane_n[h]), dim3(256), lds, sl[h], jobs + lane_first[h], j,
+                         TRD_AUX_WGS, aj, p0, flags);
     };
     for (int b = 0; b < panels; ++b) {
       const int p0 = b * TRD_NB, kcols = std::min(TRD_NB, d - 1 - p0);
-      hipLaunchKernelGGL(trd_clear_panel_kernel, dim3(std::max(1, dpad / 32), n), dim3(256), 0, s, jobs);
-      launch_product(-1, p0, p0, 2);  // first column of the panel: after the clear and the trailing update
+      for (int h = 0; h < lanes; ++h) {
+        hipLaunchKernelGGL(trd_clear_panel_kernel, dim3(std::max(1, dpad / 32), lane_n[h]), dim3(256), 0, sl[h], jobs + lane_first[h]);
+        launch_product(h, -1, p0, p0, 2);  // first column of the panel: after the clear and the trailing update
+      }
       for (int i = 0; i < kcols; ++i) {
         const int j = p0 + i;
-        launch_col(j, p0, (i > 0 ? 1 : 0) | 2);
-        launch_product(j, j + 1, p0, i + 1 < kcols ? 3 : 1);
+        for (int h = 0; h < lanes; ++h) {
+          launch_col(h, j, p0, (i > 0 ? 1 : 0) | 2);
+          launch_product(h, j, j + 1, p0, i + 1 < kcols ? 3 : 1);
+        }
       }
-      launch_col(p0 + kcols, p0, 1);
-      HIPCHECK(hipGetLastError());
-      SACHECK((launch_gemm_raw<A_KM, B_KN, EPI_SUB, false, true, 1>(gp + trail_off[b], n, trail_tiles[b], unit, s)));
+      for (int h = 0; h < lanes; ++h) {
+        launch_col(h, p0 + kcols, p0, 1);
+        HIPCHECK(hipGetLastError());
+        SACHECK((launch_gemm_raw<A_KM, B_KN, EPI_SUB, false, true, 1>(gp + trail_off[ML * b + h], lane_n[h], trail_tiles[ML * b + h], unit, sl[h])));
+      }
     }
     // last diagonal entry (a fresh, empty panel: no pending corrections)
-    launch_product(-1, d - 1, d - 1, 2);
-    launch_col(d - 1, d - 1, 2);
+    for (int h = 0; h < lanes; ++h) {
+      launch_product(h, -1, d - 1, d - 1, 2);
+      launch_col(h, d - 1, d - 1, 2);
+    }
     HIPCHECK(hipGetLastError());
+    for (int h = 1; h < lanes; ++h) {
+      HIPCHECK(hipEventRecord(p->trd_lane_ev[h - 1], sl[h]));
+      HIPCHECK(hipStreamWaitEvent(s, p->trd_lane_ev[h - 1], 0));
+    }
   }
 
   // ---- 2. Q1 = H_0 H_1 ... in the Y array (identity on entry): Q <- (I - V_b T_b V_b^T) Q for b = last .. 0, which

@@ -598,6 +598,9 @@ class _NativeGroup(_AmortizedComputation):
                     self.lib.sa_plan_set_trace_scaling(self.plan, 1, pc.trace_scaling_exponent, group[EPSILON]),
                     "sa_plan_set_trace_scaling",
                 )
+            lanes = os.environ.get("SHAMPOO_AMD_TRIDIAGONAL_LANES")
+            if lanes is not None:
+                native.check(self.lib.sa_plan_set_tridiagonal_lanes(self.plan, int(lanes)), "sa_plan_set_tridiagonal_lanes")
             split = os.environ.get("SHAMPOO_AMD_NEWTON_SPLIT_TILES", self.newton_split_tiles)
             if split is not None:
                 native.check(self.lib.sa_plan_set_newton_split_tiles(self.plan, int(split)), "sa_plan_set_newton_split_tiles")

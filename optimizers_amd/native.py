@@ -28,7 +28,7 @@ SA_GRAFT_ADAGRAD = 2
 
 EXPORTS = (
     "sa_last_error", "sa_abi_version", "sa_plan_create", "sa_plan_destroy", "sa_plan_workspace_bytes",
-    "sa_plan_bind_workspace", "sa_plan_num_factors", "sa_plan_invalidate_inverse_cache", "sa_plan_set_newton_split_tiles",
+    "sa_plan_bind_workspace", "sa_plan_num_factors", "sa_plan_invalidate_inverse_cache", "sa_plan_set_newton_split_tiles", "sa_plan_set_tridiagonal_lanes",
     "sa_plan_bind_gradients", "sa_add_l2_regularization", "sa_update_factor_matrices",
     "sa_compute_root_inverses_newton", "sa_compute_root_inverses_eigh", "sa_refresh_eigenbases_qr", "sa_refresh_eigenbases_eigh", "sa_update_corrected_eigenvalues",
     "sa_precondition_eigenvalue_corrected", "sa_update_and_precondition_eigenvalue_corrected", "sa_plan_shared_rotation_steps", "sa_update_grafting_and_filtered_grad", "sa_precondition",
@@ -138,6 +138,7 @@ def load() -> ctypes.CDLL:
     lib.sa_plan_num_factors.argtypes = [c_void_p]
     lib.sa_plan_invalidate_inverse_cache.argtypes = [c_void_p]
     lib.sa_plan_set_newton_split_tiles.argtypes = [c_void_p, c_int32]
+    lib.sa_plan_set_tridiagonal_lanes.argtypes = [c_void_p, c_int32]
     lib.sa_plan_bind_gradients.argtypes = [c_void_p, POINTER(c_void_p), c_void_p]
     lib.sa_add_l2_regularization.argtypes = [c_void_p, c_float, c_void_p]
     lib.sa_update_factor_matrices.argtypes = [c_void_p, c_float, c_float, c_void_p]

@@ -269,3 +269,37 @@ def test_pseudo_inverse_root_of_rank_deficient_factors(m, n, eigh_solver):
         got = st["inv_factor_matrices"][j].cpu()
         want = pack_triu(eigh_pseudo_inverse_root(A64, 4, rank_rtol=A64.shape[0] * 1.1920929e-7).float())
         assert rel_err(got, want) < 1e-3, (j, rel_err(got, want))
+
+
+def test_tridiagonalisation_in_lanes_gives_the_bits_of_one_lane():
+    """sa_plan_set_tridiagonal_lanes: a batch of factors reduced in two, three (the default) or four parts on as many
+    streams must leave the bits the whole batch leaves on one stream -- eight factors of order 640 (orders from 512 on
+    take the tridiagonal solver; three lanes take 3 + 3 + 2 of them), eigenbases after the refreshes and parameters
+    after the steps that use them."""
+    import optimizers_amd as oa
+    from optimizers_amd import native
+
+    g = torch.Generator().manual_seed(77)
+    shapes = [(640, 640)] * 4
+    init = [0.1 * torch.randn(s, generator=g) for s in shapes]
+    grads = [[torch.randn(s, generator=g) for s in shapes] for _ in range(2)]
+    runs = []
+    for lanes in (1, 2, 3, 4):
+        ps = [torch.nn.Parameter(t.clone().to(DEV)) for t in init]
+        cfg = oa.EigenvalueCorrectedShampooPreconditionerConfig(amortized_computation_config=oa.EighEigendecompositionConfig())
+        opt = oa.DistributedShampoo(ps, lr=0.01, betas=(0.9, 0.99), epsilon=1e-6, max_preconditioner_dim=1024,
+                                    precondition_frequency=1, start_preconditioning_step=2, preconditioner_config=cfg)
+        ng = opt._groups[0]
+        native.check(ng.lib.sa_plan_set_tridiagonal_lanes(ng.plan, lanes), "sa_plan_set_tridiagonal_lanes")
+        for gs in grads:
+            for p, gr in zip(ps, gs):
+                p.grad = gr.to(DEV)
+            opt.step()
+        torch.cuda.synchronize()
+        runs.append(([p.detach().clone() for p in ps], [t.clone() for _, _, _, t in ng._slots]))
+    p1, s1 = runs[0]
+    for pk, sk in runs[1:]:
+        for a, b in zip(pk, p1):
+            assert torch.isfinite(a).all() and torch.equal(a, b)
+        for a, b in zip(sk, s1):
+            assert torch.equal(a, b)
