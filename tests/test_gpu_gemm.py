@@ -55,3 +55,36 @@ def test_gemm_batched_2048_matches_fp64_sample():
     want = torch.bmm(A.double(), B.double())
     err = ((got.double() - want).norm() / want.norm()).item()
     assert err < 2e-6, err
+
+
+@pytest.mark.parametrize("al", [0, 1])
+@pytest.mark.parametrize("bl", [0, 1])
+@pytest.mark.parametrize("shape", [(256, 128, 32), (128, 256, 64), (256, 256, 96), (128, 128, 48), (256, 128, 80)])
+def test_gemm_on_views_that_end_with_their_allocation(al, bl, shape):
+    """Whole-tile shapes take the unguarded main loop when K is a multiple of 32 (two slabs per trip; its loads go
+    through buffer resources that end with the operand and fetch two slabs ahead without asking whether there are any)
+    and the guarded one otherwise (K = 48, 80).  The operands are column slices of wider parents whose last row ends
+    the allocation, so an extent computed too short would read zeros for the last rows and one computed from the
+    parent's pitch would reach past the allocation."""
+    from optimizers_amd import native
+
+    lib = native.load()
+    M, N, K = shape
+    print(f"case al={al} bl={bl} shape={shape}", flush=True)
+    g = torch.Generator().manual_seed(M + 3 * N + 7 * K + al + 2 * bl)
+    ra, ca = (M, K) if al == 0 else (K, M)
+    rb, cb = (K, N) if bl == 0 else (N, K)
+    pa = torch.randn(ra, ca + 64, generator=g).cuda()
+    pb = torch.randn(rb, cb + 192, generator=g).cuda()
+    A, B = pa[:, 64:], pb[:, 192:]
+    want = (A if al == 0 else A.T).double() @ (B if bl == 0 else B.T).double()
+    C = torch.full((M, N), float("nan"), device="cuda", dtype=torch.float32)
+    st = native.current_stream_ptr(C.device)
+    native.check(
+        lib.sa_gemm_f32(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, ca + 64, cb + 192, N, al, bl, 1, 0, 0, 0, st),
+        "sa_gemm_f32",
+    )
+    torch.cuda.synchronize()
+    assert torch.isfinite(C).all()
+    err = ((C.double() - want).norm() / want.norm()).item()
+    assert err < 2e-6, err
