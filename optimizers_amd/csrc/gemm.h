@@ -321,14 +321,24 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
   // cores of its SIMD to the other workgroups there.
   const bool idle_quadrant = TRI && tm == tn && wm > wn;
 
-  if constexpr (!EDGE) {
+  // A launch that may hold ragged problems (EDGE) still runs the unguarded loop on every tile that lies inside its
+  // problem, when the problem's K is a whole number of slab pairs and its operands allow 16-byte loads and fit a buffer
+  // resource: only the tiles on a ragged edge pay for the guards.
+  bool whole_tile = true;
+  if constexpr (EDGE) {
+    const long long a_ext = (AL == A_MK) ? (long long)(M - 1) * lda + K : (long long)(K - 1) * lda + M;
+    const long long b_ext = (BL == B_NK) ? (long long)(N - 1) * ldb + K : (long long)(K - 1) * ldb + N;
+    whole_tile = avec && bvec && (K % (2 * BK) == 0) && m0 + BM <= M && n0 + BN <= N && a_ext < (1ll << 29) && b_ext < (1ll << 29);
+  }
+  if (whole_tile) {
     // ---- unguarded main loop, written so that nothing but matrix instructions uses the vector ALU inside it: a VALU
     // instruction of any wavefront takes the issue slot the matrix pipe of that SIMD would have used.
-    //  * global addresses = uniform base (scalar registers, advanced per slab by the scalar ALU) + a per-thread 32-bit offset
-    //    that never changes;
+    //  * global addresses = a buffer resource per operand + a per-thread 32-bit offset that never changes + the slab's
+    //    position as the instruction's scalar offset (advanced by the scalar ALU);
     //  * LDS addresses = a per-thread base that never changes + immediate offsets (the slab loop is unrolled by two so
-    //    that the buffer a slab lives in is a compile-time constant; fragment reads are volatile so that the compiler keeps
-    //    them as single reads with 16-bit offsets instead of pairing them behind a recomputed base).
+    //    that the buffer a slab lives in is a compile-time constant; the four fragment bases are made opaque to the
+    //    compiler so that it keeps every fragment read as a single read with a 16-bit offset instead of pairing two
+    //    behind a recomputed base).
     unsigned aoff[WB], boff[WB];
     int ast[WB], bst[WB];  // LDS store positions (floats)
 #pragma unroll
