@@ -448,8 +448,10 @@ int32_t sa_set_eigh_solver(int32_t solver);
 int32_t sa_plan_set_eigh_solver(sa_plan* plan, int32_t solver);
 
 /* New parameter pointers for the blocks of a plan, one per block in plan order (same shapes and strides): for callers
- * whose parameter storage moved after the plan was built (`p.data = ...`, weight swaps, some checkpoint loaders).  The
- * reference holds views of the parameters, which follow such a change by themselves. */
+ * whose parameter storage moved after the plan was built (`p.data = ...`, weight swaps, some checkpoint loaders).
+ * A deliberate deviation, not parity: the reference blocks detached views of the storage the parameters had when the
+ * optimizer was built (shampoo_distributor.py:202-216) and goes on updating that old storage after such a change, so the
+ * parameter stops moving; following the new storage is what the caller of `p.data = ...` means. */
 int32_t sa_plan_rebind_params(sa_plan* plan, float* const* params);
 
 /* KL-Shampoo (RootInvKLShampooPreconditionerConfig / EigendecomposedKLShampooPreconditionerConfig,

@@ -770,9 +770,11 @@ class _NativeGroup(_AmortizedComputation):
         return active
 
     def _follow_parameter_storage(self) -> None:
-        """The plan holds raw pointers into the parameters.  The reference holds views, which follow a parameter whose
-        storage is replaced after the optimizer was built (`p.data = ...`, weight swaps, some checkpoint loaders); here
-        the pointers of every step are compared with the ones the plan has and the plan is re-pointed when they moved."""
+        """The plan holds raw pointers into the parameters.  When a parameter's storage is replaced after the optimizer
+        was built (`p.data = ...`, weight swaps, some checkpoint loaders) the pointers of the step differ from the ones
+        the plan has, and the plan is re-pointed.  This is a deliberate deviation from the reference, which blocks
+        detached views of the storage that existed at construction (shampoo_distributor.py:202-216) and keeps updating
+        that old storage, so that the parameter no longer moves."""
         ptrs = [p.data_ptr() for p in self.params]
         if ptrs == self._param_ptrs:
             return

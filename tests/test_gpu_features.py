@@ -325,8 +325,10 @@ def test_order_three_blocks_with_every_kind_of_split(kind):
 
 
 def test_parameter_storage_replaced_between_steps_is_followed():
-    """`p.data = ...` after the optimizer was built: the reference's block views follow the parameter; the native plan
-    holds raw pointers and must be re-pointed, or it would keep updating (and reading) the old allocation."""
+    """`p.data = ...` after the optimizer was built: the native plan holds raw pointers and is re-pointed, so the new
+    storage is what gets updated.  Not parity but a deliberate deviation: the reference's blocks are detached views of the
+    storage that existed at construction (shampoo_distributor.py:202-216), and it would keep updating (and reading) the
+    old allocation."""
     import optimizers_amd as oa
 
     def run(swap: bool):
