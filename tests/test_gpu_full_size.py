@@ -138,6 +138,59 @@ def test_large_blocks_4096_eigh():
         assert rel_err(delta.cpu(), want.cpu()) < 5e-4
 
 
+def test_large_blocks_4096_eigh_at_the_stated_cadence():
+    """Benchmark configuration 5 at full size AND with its own schedule: 49 grafting-only steps, the eigendecomposition
+    of all 32 factors at step 50, one more step that uses it.  Two gradient sets alternate (as in the benchmark), so the
+    factors have a closed form: c_1 G_1 G_1^T + c_2 G_2 G_2^T with the two sums of EMA weights."""
+    w = bench.WORKLOADS["large_block_eigh"]
+    assert w["precondition_frequency"] == 50 and w["start_preconditioning_step"] == 50
+    beta1, beta2 = w["betas"]
+    steps = 51
+    params, opt = bench.build(w, DEV)
+    sets = [bench.make_grads(w, params, s, DEV) for s in (1, 2)]
+    before = None
+    for s in range(1, steps + 1):
+        if s == steps:
+            before = [p.detach().clone() for p in params]
+        for p, g in zip(params, sets[s % 2]):
+            p.grad = g.clone()
+        opt.step()
+    torch.cuda.synchronize()
+    ng = opt._groups[0]
+    assert len(ng.native_index) == 16 and ng.n_factors == 32
+    # the factors the root inverse saw are those of step 50; the update of step 51 uses the moments of step 51
+    weight = {50: [0.0, 0.0], 51: [0.0, 0.0]}
+    for upto in (50, 51):
+        for t in range(1, upto + 1):
+            weight[upto][t % 2] += (beta2 ** (upto - t)) * (1 - beta2)
+    bc1 = 1.0 - beta1**steps
+    bc2 = 1.0 - beta2**steps
+    for k in (3, 12):
+        spec = ng.block_specs[ng.native_index[k]]
+        print(f"block {k} shape {spec.shape}", flush=True)
+        st = opt.state[params[spec.param_index]][spec.block_key]
+        G = [_block_view(sets[i][spec.param_index], spec).double() for i in range(2)]
+        X = []
+        for j in range(2):
+            gram = [(g @ g.T) if j == 0 else (g.T @ g) for g in G]
+            d = gram[0].shape[0]
+            F51 = weight[51][0] * gram[0] + weight[51][1] * gram[1]
+            assert rel_err(_unpack64(st["shampoo"]["factor_matrices"][j], d).cpu(), F51.cpu()) < 1e-5
+            F50 = weight[50][0] * gram[0] + weight[50][1] * gram[1]
+            Xj = _unpack64(st["shampoo"]["inv_factor_matrices"][j], d)
+            lam, q = torch.linalg.eigh(F50 / (1.0 - beta2**50))
+            keep = lam > 1e-4 * lam.max()  # the part of the spectrum fp32 resolves
+            qk = q[:, keep]
+            assert rel_err((qk.T @ Xj @ qk).cpu(), torch.diag(lam[keep].pow(-0.25)).cpu()) < 2e-3
+            X.append(Xj)
+        ghat = st["filtered_grad"].double() / bc1
+        graft = ghat / ((st["adagrad"].double() / bc2).sqrt() + w["graft_eps"])
+        P = X[0] @ ghat @ X[1]
+        want = -w["lr"] * (graft.norm() / (P.norm() + 1e-16)) * P
+        delta = (_block_view(params[spec.param_index], spec) - _block_view(before[spec.param_index], spec)).double()
+        assert rel_err(delta.cpu(), want.cpu()) < 5e-4
+
+
 def test_llama_layer_blocks_1024_eigenvalue_corrected():
     """Benchmark configuration 4 at full size (216 blocks, 424 eigenbases of order 1024), QR refresh at steps 2 and 3."""
     w = dict(bench.WORKLOADS["llama3_8b_layer_soap"], precondition_frequency=1, start_preconditioning_step=2)
@@ -156,6 +209,55 @@ def test_llama_layer_blocks_1024_eigenvalue_corrected():
         for q in Q:
             d = q.shape[0]
             assert (q.T @ q - torch.eye(d, dtype=torch.float64, device=DEV)).abs().max().item() < 1e-5
+        ghat = st["filtered_grad"].double() / bc1
+        rot = Q[0].T @ ghat @ Q[1]
+        rot = rot / ((st["shampoo"]["corrected_eigenvalues"].double() / bc2).sqrt() + w["epsilon"])
+        want = -w["lr"] * (Q[0] @ rot @ Q[1].T)
+        delta = (_block_view(params[spec.param_index], spec) - _block_view(before[spec.param_index], spec)).double()
+        assert rel_err(delta.cpu(), want.cpu()) < 1e-4
+
+
+def test_llama_layer_blocks_1024_eigenvalue_corrected_at_the_stated_cadence():
+    """Benchmark configuration 4 at full size AND with its own schedule: first eigenbases at step 10, QR refreshes at
+    steps 20 and 30, one more step on the bases of step 30.  Sampled blocks: the Kronecker factors are the EMA of the 31
+    Gram matrices, the bases are orthogonal, and the update is the one rebuilt from the stored state."""
+    w = bench.WORKLOADS["llama3_8b_layer_soap"]
+    assert w["precondition_frequency"] == 10 and w["start_preconditioning_step"] == 10
+    beta1, beta2 = w["betas"]
+    steps = 31
+    params, opt = bench.build(w, DEV)
+    ng = opt._groups[0]
+    assert len(ng.native_index) == 216 and ng.n_factors == 424
+    sampled = _sample_blocks(ng, 4)
+    seen = {k: [] for k in sampled}
+    before = None
+    for s in range(1, steps + 1):
+        grads = bench.make_grads(w, params, s, DEV)
+        for k in sampled:
+            spec = ng.block_specs[ng.native_index[k]]
+            seen[k].append(_block_view(grads[spec.param_index], spec).clone())
+        if s == steps:
+            before = [p.detach().clone() for p in params]
+        for p, g in zip(params, grads):
+            p.grad = g
+        opt.step()
+    torch.cuda.synchronize()
+    bc2 = 1.0 - beta2**steps
+    bc1 = 1.0 - beta1**steps
+    for k in sampled:
+        spec = ng.block_specs[ng.native_index[k]]
+        print(f"block {k} shape {spec.shape}", flush=True)
+        st = opt.state[params[spec.param_index]][spec.block_key]
+        Q = [st["shampoo"]["factor_matrices_eigenvectors"][j].double() for j in range(2)]
+        for j, q in enumerate(Q):
+            d = q.shape[0]
+            # each column passes through up to 1024 fp32 reflections: the bound is d * 2^-24 = 6e-5, measured 1.0e-5
+            departure = (q.T @ q - torch.eye(d, dtype=torch.float64, device=DEV)).abs().max().item()
+            print(f"  basis {j}: max |Q^T Q - I| = {departure:.2e}", flush=True)
+            assert departure < 3e-5
+            grams = [(g.double() @ g.double().T) if j == 0 else (g.double().T @ g.double()) for g in seen[k]]
+            F31 = sum((beta2 ** (steps - 1 - t)) * (1 - beta2) * gm for t, gm in enumerate(grams))
+            assert rel_err(_unpack64(st["shampoo"]["factor_matrices"][j], d).cpu(), F31.cpu()) < 1e-5
         ghat = st["filtered_grad"].double() / bc1
         rot = Q[0].T @ ghat @ Q[1]
         rot = rot / ((st["shampoo"]["corrected_eigenvalues"].double() / bc2).sqrt() + w["epsilon"])
