@@ -143,6 +143,143 @@ __global__ __launch_bounds__(QR_THREADS) void qr_panel_kernel(const QrPanel* __r
   }
 }
 
+// Sums of 32 values over the 64 lanes of a wavefront in 32 exchanges: at every stage a lane keeps one half of its values
+// and sends the other half to the lane whose index differs in one bit.  On return lane l holds the total of value (l >> 1).
+__device__ __forceinline__ float wave_sum32(const float (&q)[32], int lane) {
+  float a[16], b[8], c[4], d[2];
+  const bool h5 = lane & 32, h4 = lane & 16, h3 = lane & 8, h2 = lane & 4, h1 = lane & 2;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) a[i] = (h5 ? q[i + 16] : q[i]) + __shfl_xor(h5 ? q[i] : q[i + 16], 32);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) b[i] = (h4 ? a[i + 8] : a[i]) + __shfl_xor(h4 ? a[i] : a[i + 8], 16);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) c[i] = (h3 ? b[i + 4] : b[i]) + __shfl_xor(h3 ? b[i] : b[i + 4], 8);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) d[i] = (h2 ? c[i + 2] : c[i]) + __shfl_xor(h2 ? c[i] : c[i + 2], 4);
+  float e = (h1 ? d[1] : d[0]) + __shfl_xor(h1 ? d[0] : d[1], 2);
+  return e + __shfl_xor(e, 1);
+}
+
+// The same factorisation with the panel in registers: thread t holds row t of the panel, 32 columns, so the panel has at
+// most 1024 rows, and j0 is a multiple of 32.  Column k needs the products of column k below the diagonal with EVERY
+// column of the panel: with the columns to its right they give the update of the panel, with itself the norm, with the
+// columns to its left (Householder vectors by then) the entries of V^T V that the triangular factor is built from.  None
+// of them needs the scaling of the vector, so one reduction of 32 values and two barriers do a column.  The registers of a
+// row form a ring that turns by one column per step: the current column is always ring[0], so the loop stays rolled (its
+// unrolled form, 100 KB of straight-line code run once, is bound by instruction fetches) and after 32 steps every column
+// is back in its place.  Writes V and T like qr_panel_kernel.
+__global__ __launch_bounds__(QR_THREADS) void qr_panel_rows_kernel(const QrPanel* __restrict__ jobs) {
+  constexpr int NW = QR_THREADS / 64, PW = QR_MAX_PANEL;
+  __shared__ float wred[NW][PW];
+  __shared__ float rowk[PW];
+  __shared__ __align__(16) float wfin[PW];
+  __shared__ float tau_s[PW];
+  __shared__ float S[PW][PW + 1];
+  __shared__ float Tm[PW][PW + 1];
+  __shared__ float bcast[2];
+  const QrPanel& J = jobs[blockIdx.x];
+  if (J.active != nullptr && *J.active == 0) return;
+  const int rows = J.d - J.j0, pc = J.pcols;
+  const int r = threadIdx.x, lane = r & 63, wave = r >> 6;
+  const int waves_with_rows = min(NW, (rows + 63) / 64);
+  float ring[PW];
+  if (r < rows) {
+    const float4* src = reinterpret_cast<const float4*>(J.B + (long long)(J.j0 + r) * J.ldb + J.j0);
+#pragma unroll
+    for (int c4 = 0; c4 < PW / 4; ++c4) {
+      const float4 x = src[c4];
+      ring[4 * c4 + 0] = (4 * c4 + 0 < pc) ? x.x : 0.f;
+      ring[4 * c4 + 1] = (4 * c4 + 1 < pc) ? x.y : 0.f;
+      ring[4 * c4 + 2] = (4 * c4 + 2 < pc) ? x.z : 0.f;
+      ring[4 * c4 + 3] = (4 * c4 + 3 < pc) ? x.w : 0.f;
+    }
+  } else {
+#pragma unroll
+    for (int c = 0; c < PW; ++c) ring[c] = 0.f;
+  }
+  if (lane < PW) wred[wave][lane] = 0.f;
+  for (int e = r; e < PW * (PW + 1); e += QR_THREADS) { (&S[0][0])[e] = 0.f; (&Tm[0][0])[e] = 0.f; }
+  __syncthreads();
+#pragma unroll 1
+  for (int k = 0; k < PW; ++k) {
+    // ring[i] is column (k + i) mod 32: the current one, those to its right, then the finished ones
+    if (k < pc) {  // the same for every thread
+      if (wave < waves_with_rows) {
+        const float x = (r > k) ? ring[0] : 0.f;  // rows beyond the panel hold zeros
+        float q[PW];
+#pragma unroll
+        for (int i = 0; i < PW; ++i) q[i] = x * ring[i];
+        const float total = wave_sum32(q, lane);
+        if ((lane & 1) == 0) wred[wave][lane >> 1] = total;
+      }
+      if (r == k) {
+#pragma unroll
+        for (int i = 0; i < PW; ++i) rowk[i] = ring[i];
+      }
+      __syncthreads();
+      if (wave == 0) {
+        const int i = lane & (PW - 1), j = (k + i) & (PW - 1);  // ring position and the column it holds
+        float s = 0.f;
+        for (int w = 0; w < waves_with_rows; ++w) s += wred[w][i];
+        const float sigma2 = __shfl(s, 0);
+        const float alpha = rowk[0], x = rowk[i];
+        float tau = 0.f, scale = 0.f, beta = alpha;
+        if (sigma2 != 0.f) {  // LAPACK slarfg
+          beta = -copysignf(sqrtf(alpha * alpha + sigma2), alpha);
+          tau = (beta - alpha) / beta;
+          scale = 1.0f / (alpha - beta);
+        }
+        if (lane < PW) {
+          wfin[i] = (j > k) ? tau * (x + scale * s) : 0.f;  // tau v^T P[:, j] with v = (1, scale x); finished columns stay
+          if (j < k) S[j][k] = x + scale * s;               // v_j^T v_k
+          if (j == k) { tau_s[k] = tau; bcast[0] = scale; bcast[1] = beta; }
+        }
+      }
+      __syncthreads();
+      if (r >= k) {
+        const float v = (r > k) ? ring[0] * bcast[0] : 1.0f;
+        ring[0] = (r > k) ? v : bcast[1];
+#pragma unroll
+        for (int i = 1; i < PW; ++i) ring[i] -= wfin[i] * v;
+      }
+    }
+    const float first = ring[0];
+#pragma unroll
+    for (int i = 0; i < PW - 1; ++i) ring[i] = ring[i + 1];
+    ring[PW - 1] = first;
+  }
+  // --- T (LAPACK slarft, forward columnwise): T[i][i] = tau_i, T[0:i, i] = -tau_i T[0:i,0:i] S[0:i, i]
+  for (int i = 0; i < pc; ++i) {
+    if (r < i) {
+      float acc = 0.f;
+      for (int m = r; m < i; ++m) acc += Tm[r][m] * S[m][i];
+      Tm[r][i] = -tau_s[i] * acc;
+    }
+    if (r == i) Tm[i][i] = tau_s[i];
+    __syncthreads();
+  }
+  for (int e = r; e < J.t_rows * pc; e += QR_THREADS) {
+    const int tr = e / pc, c = e - tr * pc, i = tr - J.top;
+    J.T[(long long)tr * J.ldt + c] = (i >= 0 && i < pc) ? Tm[i][c] : 0.f;
+  }
+  for (int e = r; e < J.top * pc; e += QR_THREADS) J.V[(long long)(e / pc) * J.ldv + e % pc] = 0.f;
+  if (r < rows) {
+    float* dst = J.V + (long long)(J.top + r) * J.ldv;
+    float v[PW];
+#pragma unroll
+    for (int c = 0; c < PW; ++c) v[c] = (r > c) ? ring[c] : (r == c ? 1.0f : 0.0f);
+    if (pc == PW && (J.ldv & 3) == 0 && (reinterpret_cast<uintptr_t>(J.V) & 15) == 0) {
+#pragma unroll
+      for (int c4 = 0; c4 < PW / 4; ++c4)
+        reinterpret_cast<float4*>(dst)[c4] = make_float4(v[4 * c4], v[4 * c4 + 1], v[4 * c4 + 2], v[4 * c4 + 3]);
+    } else {
+#pragma unroll
+      for (int c = 0; c < PW; ++c)
+        if (c < pc) dst[c] = v[c];
+    }
+  }
+}
+
 // Generic strided 2-D copy: dst[r][c] = src[r][c]
 struct Copy2D {
   const float* src;

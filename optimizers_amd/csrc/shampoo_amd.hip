@@ -4135,8 +4135,10 @@ static int qr_accumulate(sa_plan* p, const std::vector<int>& ids, hipStream_t s)
     dmax = std::max(dmax, p->factors[i].d);
     dpad_min = std::min(dpad_min, p->factors[i].dpad);
   }
+  // panels of up to 1024 rows are factored in registers (32 columns wide), taller ones in LDS (narrower)
+  const bool in_registers = dmax <= QR_THREADS;
   const int lds_floats = 34816;  // 136 KB for the panel, the rest of the 160 KB holds the small arrays
-  const int ip = std::min(QR_MAX_PANEL, lds_floats / dmax - 1);  // panel width
+  const int ip = in_registers ? QR_MAX_PANEL : std::min(QR_MAX_PANEL, lds_floats / dmax - 1);  // panel width
   if (ip < 1) return fail(SA_ERR_UNSUPPORTED, "QR refresh: factor dimension too large for an LDS resident panel");
   static bool attr_set = false;
   if (!attr_set) {
@@ -4206,7 +4208,8 @@ static int qr_accumulate(sa_plan* p, const std::vector<int>& ids, hipStream_t s)
       SACHECK(R.panel.upload(s));
       for (int k = 0; k < 3; ++k) { SACHECK(R.upd[k].commit(s)); SACHECK(R.merge[k].commit(s)); }
       const size_t lds_bytes = (size_t)max_rows * (ip + 1) * sizeof(float);
-      hipLaunchKernelGGL(qr_panel_kernel, dim3(jobs), dim3(QR_THREADS), lds_bytes, s, R.panel.dev);
+      if (in_registers) hipLaunchKernelGGL(qr_panel_rows_kernel, dim3(jobs), dim3(QR_THREADS), 0, s, R.panel.dev);
+      else hipLaunchKernelGGL(qr_panel_kernel, dim3(jobs), dim3(QR_THREADS), lds_bytes, s, R.panel.dev);
       HIPCHECK(hipGetLastError());
       SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, true>(R.upd[0], u, s)));
       SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, true>(R.upd[1], u, s)));
