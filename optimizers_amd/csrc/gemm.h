@@ -321,16 +321,18 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
   // cores of its SIMD to the other workgroups there.
   const bool idle_quadrant = TRI && tm == tn && wm > wn;
 
-  // A launch that may hold ragged problems (EDGE) still runs the unguarded loop on every tile that lies inside its
-  // problem, when the problem's K is a whole number of slab pairs and its operands allow 16-byte loads and fit a buffer
-  // resource: only the tiles on a ragged edge pay for the guards.
-  bool whole_tile = true;
+  // A launch that may hold ragged problems (EDGE) still runs the unguarded loop on every problem whose K is a whole
+  // number of slab pairs and whose operands allow 16-byte loads and fit a buffer resource, ragged M and N included:
+  // the threads that would fetch rows or columns past M or N are pointed past the resource and get zeros.
+  bool fast_loop = true;
   if constexpr (EDGE) {
     const long long a_ext = (AL == A_MK) ? (long long)(M - 1) * lda + K : (long long)(K - 1) * lda + M;
     const long long b_ext = (BL == B_NK) ? (long long)(N - 1) * ldb + K : (long long)(K - 1) * ldb + N;
-    whole_tile = avec && bvec && (K % (2 * BK) == 0) && m0 + BM <= M && n0 + BN <= N && a_ext < (1ll << 29) && b_ext < (1ll << 29);
+    // (16-byte loads along M or N must not straddle the end of the operand: M, N multiples of 4 there)
+    fast_loop = avec && bvec && (K % (2 * BK) == 0) && a_ext < (1ll << 29) && b_ext < (1ll << 29) &&
+                (AL == A_MK || M % 4 == 0) && (BL == B_NK || N % 4 == 0);
   }
-  if (whole_tile) {
+  if (fast_loop) {
     // ---- unguarded main loop, written so that nothing but matrix instructions uses the vector ALU inside it: a VALU
     // instruction of any wavefront takes the issue slot the matrix pipe of that SIMD would have used.
     //  * global addresses = a buffer resource per operand + a per-thread 32-bit offset that never changes + the slab's
@@ -349,6 +351,12 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
       else { aoff[i] = (unsigned)((idx / PER_ROW) * (int)lda + ((idx % PER_ROW) << 2)); ast[i] = (idx / PER_ROW) * LDS_STRIDE + ((idx % PER_ROW) << 2); }
       if (BL == B_NK) { boff[i] = (unsigned)((idx >> 2) * (int)ldb + ((idx & 3) << 2)); bst[i] = ((idx & 3) << 2) * LDS_STRIDE + (idx >> 2); }
       else { boff[i] = (unsigned)((idx / PER_ROW) * (int)ldb + ((idx % PER_ROW) << 2)); bst[i] = (idx / PER_ROW) * LDS_STRIDE + ((idx % PER_ROW) << 2); }
+      if constexpr (EDGE) {
+        // a thread whose vector lies past M or N fetches from past the resource instead: zero, and no memory traffic
+        constexpr unsigned NOWHERE = 0x3fffffffu;  // in floats; four times it is still a 32-bit offset
+        if (m0 + ((AL == A_MK) ? (idx >> 2) : ((idx % PER_ROW) << 2)) >= M) aoff[i] = NOWHERE;
+        if (n0 + ((BL == B_NK) ? (idx >> 2) : ((idx % PER_ROW) << 2)) >= N) boff[i] = NOWHERE;
+      }
     }
     // buffer resources over the two operands: the per-thread offset goes into the instruction's vector offset, the slab's
     // position into its scalar offset (advanced by the scalar ALU)
@@ -360,6 +368,9 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
     const __amdgpu_buffer_rsrc_t bres = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(bbase), 0, (int)(b_floats * 4), 0x00020000);
     const int astep = ((AL == A_MK) ? BK : BK * (int)lda) * 4;
     const int bstep = ((BL == B_NK) ? BK : BK * (int)ldb) * 4;
+    // the loop fetches two slabs ahead without asking whether there are any: past the last slab it fetches the last one
+    // again (the scalar offset of a buffer load is not checked against the resource, so it must stay inside the operand)
+    const int a_last = (slabs - 1) * astep, b_last = (slabs - 1) * bstep;
     int apos = 0, bpos = 0;  // bytes
     auto fetch_into = [&](float4 (&xa)[WB], float4 (&xb)[WB]) {
 #pragma unroll
@@ -372,8 +383,8 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
         const vuint4 v = __builtin_amdgcn_raw_buffer_load_b128(bres, (int)(boff[i] * 4), bpos, 0);
         xb[i] = make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
       }
-      apos += astep;
-      bpos += bstep;
+      apos = min(apos + astep, a_last);
+      bpos = min(bpos + bstep, b_last);
     };
     auto scale = [&](float4 (&xa)[WB], float4 (&xb)[WB]) {
       if (a_div != 1.0f) {

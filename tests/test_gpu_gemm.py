@@ -59,13 +59,18 @@ def test_gemm_batched_2048_matches_fp64_sample():
 
 @pytest.mark.parametrize("al", [0, 1])
 @pytest.mark.parametrize("bl", [0, 1])
-@pytest.mark.parametrize("shape", [(256, 128, 32), (128, 256, 64), (256, 256, 96), (128, 128, 48), (256, 128, 80)])
+@pytest.mark.parametrize(
+    "shape",
+    [(256, 128, 32), (128, 256, 64), (256, 256, 96), (128, 128, 48), (256, 128, 80), (32, 96, 1024), (81, 200, 64), (4, 8, 32), (300, 132, 160)],
+)
 def test_gemm_on_views_that_end_with_their_allocation(al, bl, shape):
-    """Whole-tile shapes take the unguarded main loop when K is a multiple of 32 (two slabs per trip; its loads go
-    through buffer resources that end with the operand and fetch two slabs ahead without asking whether there are any)
-    and the guarded one otherwise (K = 48, 80).  The operands are column slices of wider parents whose last row ends
-    the allocation, so an extent computed too short would read zeros for the last rows and one computed from the
-    parent's pitch would reach past the allocation."""
+    """Shapes with K a multiple of 32 take the unguarded main loop (two slabs per trip; its loads go through buffer
+    resources that end with the operand and fetch two slabs ahead without asking whether there are any), ragged M and N
+    included: what such a tile fetches past M or N lands in rows and columns the guarded epilogue drops (the parents are
+    filled with NaN outside the operands here, so a dropped guard would show).  Other K (48, 80) take the guarded loop.
+    The operands are column slices of wider parents whose last row ends the allocation, so an extent computed too
+    short would read zeros for the last rows and one computed from the parent's pitch would reach past the
+    allocation."""
     from optimizers_amd import native
 
     lib = native.load()
@@ -74,8 +79,11 @@ def test_gemm_on_views_that_end_with_their_allocation(al, bl, shape):
     g = torch.Generator().manual_seed(M + 3 * N + 7 * K + al + 2 * bl)
     ra, ca = (M, K) if al == 0 else (K, M)
     rb, cb = (K, N) if bl == 0 else (N, K)
-    pa = torch.randn(ra, ca + 64, generator=g).cuda()
-    pb = torch.randn(rb, cb + 192, generator=g).cuda()
+    pa = torch.full((ra, ca + 64), float("nan"))
+    pb = torch.full((rb, cb + 192), float("nan"))
+    pa[:, 64:] = torch.randn(ra, ca, generator=g)
+    pb[:, 192:] = torch.randn(rb, cb, generator=g)
+    pa, pb = pa.cuda(), pb.cuda()
     A, B = pa[:, 64:], pb[:, 192:]
     want = (A if al == 0 else A.T).double() @ (B if bl == 0 else B.T).double()
     C = torch.full((M, N), float("nan"), device="cuda", dtype=torch.float32)
