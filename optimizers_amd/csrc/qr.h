@@ -143,13 +143,14 @@ __global__ __launch_bounds__(QR_THREADS) void qr_panel_kernel(const QrPanel* __r
   }
 }
 
-// Sums of 32 values over the 64 lanes of a wavefront in 32 exchanges: at every stage a lane keeps one half of its values
-// and sends the other half to the lane whose index differs in one bit.  On return lane l holds the total of value (l >> 1).
-__device__ __forceinline__ float wave_sum32(const float (&q)[32], int lane) {
+// Sums of the 32 values x q[i] over the 64 lanes of a wavefront in 32 exchanges: at every stage a lane keeps one half of
+// its values and sends the other half to the lane whose index differs in one bit.  On return lane l holds the total of
+// value (l >> 1).
+__device__ __forceinline__ float wave_sum32(const float (&q)[32], float x, int lane) {
   float a[16], b[8], c[4], d[2];
   const bool h5 = lane & 32, h4 = lane & 16, h3 = lane & 8, h2 = lane & 4, h1 = lane & 2;
 #pragma unroll
-  for (int i = 0; i < 16; ++i) a[i] = (h5 ? q[i + 16] : q[i]) + __shfl_xor(h5 ? q[i] : q[i + 16], 32);
+  for (int i = 0; i < 16; ++i) a[i] = x * (h5 ? q[i + 16] : q[i]) + __shfl_xor(x * (h5 ? q[i] : q[i + 16]), 32);
 #pragma unroll
   for (int i = 0; i < 8; ++i) b[i] = (h4 ? a[i + 8] : a[i]) + __shfl_xor(h4 ? a[i] : a[i + 8], 16);
 #pragma unroll
@@ -168,7 +169,7 @@ __device__ __forceinline__ float wave_sum32(const float (&q)[32], int lane) {
 // row form a ring that turns by one column per step: the current column is always ring[0], so the loop stays rolled (its
 // unrolled form, 100 KB of straight-line code run once, is bound by instruction fetches) and after 32 steps every column
 // is back in its place.  Writes V and T like qr_panel_kernel.
-__global__ __launch_bounds__(QR_THREADS) void qr_panel_rows_kernel(const QrPanel* __restrict__ jobs) {
+__global__ __launch_bounds__(QR_THREADS, 8) void qr_panel_rows_kernel(const QrPanel* __restrict__ jobs) {
   constexpr int NW = QR_THREADS / 64, PW = QR_MAX_PANEL;
   __shared__ float wred[NW][PW];
   __shared__ float rowk[PW];
@@ -206,10 +207,7 @@ __global__ __launch_bounds__(QR_THREADS) void qr_panel_rows_kernel(const QrPanel
     if (k < pc) {  // the same for every thread
       if (wave < waves_with_rows) {
         const float x = (r > k) ? ring[0] : 0.f;  // rows beyond the panel hold zeros
-        float q[PW];
-#pragma unroll
-        for (int i = 0; i < PW; ++i) q[i] = x * ring[i];
-        const float total = wave_sum32(q, lane);
+        const float total = wave_sum32(ring, x, lane);
         if ((lane & 1) == 0) wred[wave][lane >> 1] = total;
       }
       if (r == k) {
@@ -220,7 +218,8 @@ __global__ __launch_bounds__(QR_THREADS) void qr_panel_rows_kernel(const QrPanel
       if (wave == 0) {
         const int i = lane & (PW - 1), j = (k + i) & (PW - 1);  // ring position and the column it holds
         float s = 0.f;
-        for (int w = 0; w < waves_with_rows; ++w) s += wred[w][i];
+#pragma unroll
+        for (int w = 0; w < NW; ++w) s += wred[w][i];  // wavefronts without rows left their zeros there
         const float sigma2 = __shfl(s, 0);
         const float alpha = rowk[0], x = rowk[i];
         float tau = 0.f, scale = 0.f, beta = alpha;
