@@ -406,8 +406,13 @@ struct sa_plan {
   GemmTable ec_stat1, ec_stat2, ec_stat_l, ec_stat_r;          // corrected-eigenvalue update
   GemmTable ec_p1, ec_p1d, ec_p2, ec_p2d, ec_p3, ec_p3n, ec_p4, ec_p4n;  // eigenvalue-corrected preconditioning
   struct QrInner { Table<QrPanel> panel; GemmTable upd[3], merge[3]; };
-  QrInner qr_in[4];        // rings, so that the host can fill the tables of the next panels while the GPU works
-  GemmTable qr_outer[2][6];
+  // Tables of the QR refresh.  Panels factored in registers (orders up to 1024) keep a set per panel and per outer block:
+  // a refresh rewrites every set with the bytes it already holds and uploads nothing (an upload is a copy command of its
+  // own on the stream, seven per panel).  Taller factors have narrow panels, hundreds of them: they share rings of four
+  // and two sets, so that the host can fill the tables of the next panels while the GPU works.
+  struct QrOuter { GemmTable g[6]; };
+  std::vector<std::unique_ptr<QrInner>> qr_in;
+  std::vector<std::unique_ptr<QrOuter>> qr_outer;
   GemmTable qr_aq, qr_b;
   Table<TrdJob> t_trd, t_trd_ql;  // every factor of the batch; those that take the QL iteration
   Table<TransposeJob> t_transpose;
@@ -1355,8 +1360,8 @@ void sa_plan_destroy(sa_plan* p) {
   for (GemmTable* g : {&p->ec_stat1, &p->ec_stat2, &p->ec_stat_l, &p->ec_stat_r, &p->ec_p1, &p->ec_p1d, &p->ec_p2, &p->ec_p2d,
                        &p->ec_p3, &p->ec_p3n, &p->ec_p4, &p->ec_p4n, &p->qr_aq, &p->qr_b})
     g->t.destroy();
-  for (auto& r : p->qr_in) { r.panel.destroy(); for (auto& g : r.upd) g.t.destroy(); for (auto& g : r.merge) g.t.destroy(); }
-  for (auto& a : p->qr_outer) for (auto& g : a) g.t.destroy();
+  for (auto& r : p->qr_in) { r->panel.destroy(); for (auto& g : r->upd) g.t.destroy(); for (auto& g : r->merge) g.t.destroy(); }
+  for (auto& a : p->qr_outer) for (auto& g : a->g) g.t.destroy();
   p->t_copy.destroy(); p->t_normpair.destroy(); p->t_sort.destroy();
   for (void* q : {(void*)p->d_err, (void*)p->d_active, (void*)p->d_report, (void*)p->d_final_parity, (void*)p->d_nactive,
                   (void*)p->d_scale, (void*)p->d_ho, (void*)p->d_kept_err, (void*)p->d_hoflag})
@@ -4164,7 +4169,9 @@ static int qr_accumulate(sa_plan* p, const std::vector<int>& ids, hipStream_t s)
   int inner_no = 0, outer_no = 0;
   for (int J0 = 0; J0 < dmax; J0 += OB, ++outer_no) {
     for (int off = 0; off < OB && J0 + off < dmax; off += ip, ++inner_no) {
-      sa_plan::QrInner& R = p->qr_in[inner_no % 4];
+      const size_t in_slot = in_registers ? (size_t)inner_no : (size_t)(inner_no % 4);
+      while (p->qr_in.size() <= in_slot) p->qr_in.emplace_back(new sa_plan::QrInner());
+      sa_plan::QrInner& R = *p->qr_in[in_slot];
       const int j0 = J0 + off;
       SACHECK(R.panel.begin(n));
       for (int k = 0; k < 3; ++k) { R.upd[k].clear(); R.merge[k].clear(); }
@@ -4219,7 +4226,9 @@ static int qr_accumulate(sa_plan* p, const std::vector<int>& ids, hipStream_t s)
       SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, true>(R.merge[2], neg, s)));
     }
     // the outer block's reflectors I - V T V^T on the trailing matrix (from the left, transposed) and on Qacc (from the right)
-    GemmTable* G = p->qr_outer[outer_no % 2];
+    const size_t out_slot = in_registers ? (size_t)outer_no : (size_t)(outer_no % 2);
+    while (p->qr_outer.size() <= out_slot) p->qr_outer.emplace_back(new sa_plan::QrOuter());
+    GemmTable* G = p->qr_outer[out_slot]->g;
     for (int k = 0; k < 6; ++k) G[k].clear();
     bool any = false;
     for (int i : ids) {
