@@ -402,7 +402,7 @@ struct EigInit {
   const float* packed;
   const float* scale;  // optional per-factor multiplier applied after the division by bc2 (trace scaling)
   float* A;
-  float* V;
+  float* V;  // optional
   int d, dpad;
   int tile_begin;  // first 64 x 64 tile id of this factor (full grid, not triangular)
   int tiles;       // dpad / 64
@@ -421,17 +421,25 @@ __global__ __launch_bounds__(256) void eig_init_kernel(const EigInit* __restrict
   const int bi = t / J.tiles, bj = t % J.tiles;
   const int d = J.d, dpad = J.dpad;
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  // the packed rows are read along themselves: a tile below the diagonal reads its mirror image and turns it in LDS
+  __shared__ float tile[64][65];
+  const int r0 = 64 * min(bi, bj), c0 = 64 * max(bi, bj);
   for (int rr = ty; rr < 64; rr += 4) {
-    const int r = bi * 64 + rr, c = bj * 64 + tx;
+    const int r = r0 + rr, c = c0 + tx;
     float v = 0.0f;
-    if (r < d && c < d) {
-      const int rs = min(r, c), cs = max(r, c);
-      v = J.packed[(long long)rs * d - ((long long)rs * (rs - 1)) / 2 + (cs - rs)] / bc2;
+    if (r < d && c < d && c >= r) {
+      v = J.packed[(long long)r * d - ((long long)r * (r - 1)) / 2 + (c - r)] / bc2;
       if (J.scale != nullptr) v = v * J.scale[0];
       if (r == c && eps != 0.0f) v = v + eps;
     }
-    J.A[(long long)r * dpad + c] = v;
-    J.V[(long long)r * dpad + c] = (r == c) ? 1.0f : 0.0f;
+    tile[rr][tx] = v;
+  }
+  __syncthreads();
+  for (int rr = ty; rr < 64; rr += 4) {
+    const int r = bi * 64 + rr, c = bj * 64 + tx;
+    const bool as_read = bi < bj || (bi == bj && tx >= rr);
+    J.A[(long long)r * dpad + c] = as_read ? tile[rr][tx] : tile[tx][rr];
+    if (J.V != nullptr) J.V[(long long)r * dpad + c] = (r == c) ? 1.0f : 0.0f;
   }
 }
 

@@ -4293,7 +4293,7 @@ static int sa_refresh_eigenbases_qr_wave(sa_plan* p, float bias_correction2, flo
     const Factor& f = p->factors[todo[i]];
     EigInit& J = p->t_eiginit.host[i];
     std::memset(&J, 0, sizeof(J));
-    J.packed = packed32(p, f); J.scale = p->scale_of(todo[i]); J.A = newton_buf(p, NB_M0, f); J.V = newton_buf(p, NB_MP0, f);
+    J.packed = packed32(p, f); J.scale = p->scale_of(todo[i]); J.A = newton_buf(p, NB_M0, f); J.V = nullptr;  // the basis comes from the state
     J.d = f.d; J.dpad = f.dpad; J.tiles = f.dpad / 64; J.enabled = 1; J.tile_begin = tiles;
     tiles += J.tiles * J.tiles;
     Copy2D& C = p->t_copy.host[i];
