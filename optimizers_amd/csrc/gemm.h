@@ -369,7 +369,8 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
     const int astep = ((AL == A_MK) ? BK : BK * (int)lda) * 4;
     const int bstep = ((BL == B_NK) ? BK : BK * (int)ldb) * 4;
     // the loop fetches two slabs ahead without asking whether there are any: past the last slab it fetches the last one
-    // again (the scalar offset of a buffer load is not checked against the resource, so it must stay inside the operand)
+    // again, so every address it forms lies inside the operand whatever part the scalar offset plays in the range check
+    // of a buffer load (on gfx950 it is checked together with the vector offset, on other parts it is not)
     const int a_last = (slabs - 1) * astep, b_last = (slabs - 1) * bstep;
     int apos = 0, bpos = 0;  // bytes
     auto fetch_into = [&](float4 (&xa)[WB], float4 (&xb)[WB]) {
