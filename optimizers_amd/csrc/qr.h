@@ -143,16 +143,27 @@ __global__ __launch_bounds__(QR_THREADS) void qr_panel_kernel(const QrPanel* __r
   }
 }
 
-// Sums of the 32 values x q[i] over the 64 lanes of a wavefront in 32 exchanges: at every stage a lane keeps one half of
-// its values and sends the other half to the lane whose index differs in one bit.  On return lane l holds the total of
-// value (l >> 1).
+// Sums of the 32 values x q[i] over the 64 lanes of a wavefront: at every stage a lane keeps one half of its values and
+// trades the other half with the lane whose index differs in one bit.  The first two stages (bits 5 and 4) are the lane
+// swaps of gfx950, v_permlane32_swap and v_permlane16_swap, which exchange the upper half of one register with the lower
+// half of another (of every 32 lanes, of every 16): one instruction per pair of values and no trip through LDS.  On
+// return lane l holds the total of value (l >> 1).
+typedef unsigned qr_uint2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ float wave_sum32(const float (&q)[32], float x, int lane) {
   float a[16], b[8], c[4], d[2];
-  const bool h5 = lane & 32, h4 = lane & 16, h3 = lane & 8, h2 = lane & 4, h1 = lane & 2;
+  const bool h3 = lane & 8, h2 = lane & 4, h1 = lane & 2;
 #pragma unroll
-  for (int i = 0; i < 16; ++i) a[i] = x * (h5 ? q[i + 16] : q[i]) + __shfl_xor(x * (h5 ? q[i] : q[i + 16]), 32);
+  for (int i = 0; i < 16; ++i) {
+    // lanes 0-31 end up with both halves' value i, lanes 32-63 with both halves' value i + 16
+    const qr_uint2 t = __builtin_amdgcn_permlane32_swap(__float_as_uint(x * q[i]), __float_as_uint(x * q[i + 16]), false, false);
+    a[i] = __uint_as_float(t.x) + __uint_as_float(t.y);
+  }
 #pragma unroll
-  for (int i = 0; i < 8; ++i) b[i] = (h4 ? a[i + 8] : a[i]) + __shfl_xor(h4 ? a[i] : a[i + 8], 16);
+  for (int i = 0; i < 8; ++i) {
+    // even rows of 16 lanes end up with value i of both rows, odd rows with value i + 8
+    const qr_uint2 t = __builtin_amdgcn_permlane16_swap(__float_as_uint(a[i]), __float_as_uint(a[i + 8]), false, false);
+    b[i] = __uint_as_float(t.x) + __uint_as_float(t.y);
+  }
 #pragma unroll
   for (int i = 0; i < 4; ++i) c[i] = (h3 ? b[i + 4] : b[i]) + __shfl_xor(h3 ? b[i] : b[i + 4], 8);
 #pragma unroll
