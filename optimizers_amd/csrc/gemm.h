@@ -90,37 +90,76 @@ __device__ __forceinline__ float4 gload4(const float* p) {
 __device__ __forceinline__ float gload1(const float* p) { return *(const __attribute__((address_space(1))) float*)p; }
 
 // live_begin[i] = number of tiles of the active problems in front of problem i (i = 0 .. n), for a launch that
-// passes it to grouped_gemm_kernel.  One workgroup; `triangular` = the launch computes upper-triangle tiles only.
+// passes it to grouped_gemm_kernel, followed by NUM_XCD + 1 tile offsets that cut the live tiles into one run per XCD
+// of equal WORK (a tile's work is its K): problems of different orders in one launch would otherwise leave the XCDs
+// that drew the long tiles running after the others have drained.  No run is longer than `cap` tiles (the launch has
+// cap workgroups per XCD).  One workgroup; `triangular` = the launch computes upper-triangle tiles only.  `live_begin`
+// holds live_ints(n) ints: the offsets, the cuts, and behind them the running work as 64-bit integers.
+__host__ __device__ inline size_t live_work_offset(int n) { return ((size_t)n + 1 + NUM_XCD + 1 + 1) & ~(size_t)1; }
+__host__ __device__ inline size_t live_ints(int n) { return live_work_offset(n) + 2 * ((size_t)n + 1); }
 __global__ __launch_bounds__(256) void gemm_live_tiles_kernel(const GemmProblem* __restrict__ problems, int n, int triangular,
-                                                              int* __restrict__ live_begin) {
+                                                              int* __restrict__ live_begin, int cap) {
   __shared__ int part[256];
+  __shared__ long long wpart[256];
   __shared__ int carry;
-  if (threadIdx.x == 0) carry = 0;
+  __shared__ long long wcarry;
+  long long* __restrict__ work_begin = reinterpret_cast<long long*>(live_begin + live_work_offset(n));
+  int* __restrict__ cut = live_begin + n + 1;
+  if (threadIdx.x == 0) { carry = 0; wcarry = 0; }
   __syncthreads();
   for (int base = 0; base < n; base += 256) {
     const int i = base + threadIdx.x;
     int w = 0;
+    long long ww = 0;
     if (i < n) {
       const GemmProblem& P = problems[i];
       const bool on = P.active == nullptr || *P.active != 0;
       w = !on ? 0 : (triangular ? P.tiles_n * (P.tiles_n + 1) / 2 : P.tiles_m * P.tiles_n);
+      ww = (long long)w * max(P.K, 1);
     }
     part[threadIdx.x] = w;
+    wpart[threadIdx.x] = ww;
     __syncthreads();
-    // inclusive scan of the 256 widths
+    // inclusive scans of the 256 widths and of their work
     for (int o = 1; o < 256; o <<= 1) {
       const int add = threadIdx.x >= o ? part[threadIdx.x - o] : 0;
+      const long long wadd = threadIdx.x >= o ? wpart[threadIdx.x - o] : 0;
       __syncthreads();
       part[threadIdx.x] += add;
+      wpart[threadIdx.x] += wadd;
       __syncthreads();
     }
     const int c = carry;
-    if (i < n) live_begin[i] = c + part[threadIdx.x] - w;
+    const long long wc = wcarry;
+    if (i < n) {
+      live_begin[i] = c + part[threadIdx.x] - w;
+      work_begin[i] = wc + wpart[threadIdx.x] - ww;
+    }
     __syncthreads();
-    if (threadIdx.x == 255) carry = c + part[255];
+    if (threadIdx.x == 255) { carry = c + part[255]; wcarry = wc + wpart[255]; }
     __syncthreads();
   }
-  if (threadIdx.x == 0) live_begin[n] = carry;
+  const int total = carry;
+  const long long total_work = wcarry;
+  if (threadIdx.x == 0) { live_begin[n] = total; work_begin[n] = total_work; cut[0] = 0; cut[NUM_XCD] = total; }
+  __syncthreads();  // the offsets written above are read below by other threads of this workgroup
+  if (threadIdx.x >= 1 && threadIdx.x < NUM_XCD) {
+    const long long target = total_work / NUM_XCD * threadIdx.x + total_work % NUM_XCD * threadIdx.x / NUM_XCD;
+    int lo = 0, hi = n - 1;  // the last problem whose work begins at or before the target
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (work_begin[mid] <= target) lo = mid; else hi = mid - 1;
+    }
+    const int tiles_here = live_begin[lo + 1] - live_begin[lo];
+    const long long into = (target - work_begin[lo]) / max(problems[lo].K, 1);
+    cut[threadIdx.x] = live_begin[lo] + (int)min((long long)tiles_here, into);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int x = 0; x < NUM_XCD; ++x) cut[x + 1] = max(cut[x], min(cut[x + 1], cut[x] + cap));  // no run above the cap ...
+    cut[NUM_XCD] = total;
+    for (int x = NUM_XCD - 1; x >= 1; --x) cut[x] = max(cut[x], cut[x + 1] - cap);              // ... the last one included
+  }
 }
 
 __device__ __forceinline__ float4 load4_guarded(const float* p, bool vec, int valid) {
@@ -233,15 +272,21 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
   __shared__ float red[4];
   static_assert(WB == 2 || (EPI != EPI_STORE_SQNORM), "per-tile partial sums are laid out for 128 x 128 tiles");
 
-  // With live_begin (n_problems + 1 ascending tile offsets written by gemm_live_tiles_kernel) the launch walks only
-  // the tiles of the problems that are still active: a skipped problem has no tiles there, so the 8 XCDs share the
-  // live tiles evenly however the active problems are spread over the table.
-  if (live_begin != nullptr) total_tiles = live_begin[n_problems];
-
-  // XCD-aware remap of the hardware workgroup id to a logical tile id.
-  const int per_xcd = (total_tiles + NUM_XCD - 1) / NUM_XCD;
-  const int logical = (blockIdx.x % NUM_XCD) * per_xcd + blockIdx.x / NUM_XCD;
-  if (logical >= total_tiles) return;
+  // XCD-aware remap of the hardware workgroup id to a logical tile id: every XCD walks one run of consecutive tiles.
+  // With live_begin (n_problems + 1 ascending tile offsets and the NUM_XCD + 1 cuts between the runs, written by
+  // gemm_live_tiles_kernel) the launch walks only the tiles of the problems that are still active, in runs of equal
+  // work; without it the runs hold equal numbers of tiles.
+  int logical;
+  if (live_begin != nullptr) {
+    const int* __restrict__ cut = live_begin + n_problems + 1;
+    const int x = blockIdx.x % NUM_XCD;
+    logical = cut[x] + blockIdx.x / NUM_XCD;
+    if (logical >= cut[x + 1]) return;
+  } else {
+    const int per_xcd = (total_tiles + NUM_XCD - 1) / NUM_XCD;
+    logical = (blockIdx.x % NUM_XCD) * per_xcd + blockIdx.x / NUM_XCD;
+    if (logical >= total_tiles) return;
+  }
 
   // Which problem owns this tile (tile offsets ascend; of several equal offsets the last one owns the tile).
   int lo = 0, hi = n_problems - 1;

@@ -166,7 +166,7 @@ struct GemmTable {
     if (live_cap >= t.n + 1) return SA_OK;
     if (live) HIPCHECK(hipFree(live));
     live = nullptr; live_cap = 0;
-    HIPCHECK(hipMalloc(&live, (t.n + 1) * sizeof(int)));
+    HIPCHECK(hipMalloc(&live, live_ints((int)t.n) * sizeof(int)));
     live_cap = t.n + 1;
     return SA_OK;
   }
@@ -206,9 +206,10 @@ int launch_gemm_live(GemmTable& g, GemmScalars sc, hipStream_t s) {
   }
   if (g.total_tiles < 2048) return launch_gemm<AL, BL, EPI, EDGE, TRI>(g, sc, s);
   SACHECK(g.need_live());
-  hipLaunchKernelGGL(gemm_live_tiles_kernel, dim3(1), dim3(256), 0, s, g.t.dev, (int)g.t.n, TRI ? 1 : 0, g.live);
-  const int per = (g.total_tiles + NUM_XCD - 1) / NUM_XCD;
-  hipLaunchKernelGGL((grouped_gemm_kernel<AL, BL, EPI, EDGE, TRI>), dim3(per * NUM_XCD), dim3(GEMM_THREADS), 0, s,
+  // runs of equal work may differ in their numbers of tiles: a quarter more workgroups per XCD than an even split needs
+  const int per = (g.total_tiles + NUM_XCD - 1) / NUM_XCD, cap = per + per / 4 + 1;
+  hipLaunchKernelGGL(gemm_live_tiles_kernel, dim3(1), dim3(256), 0, s, g.t.dev, (int)g.t.n, TRI ? 1 : 0, g.live, cap);
+  hipLaunchKernelGGL((grouped_gemm_kernel<AL, BL, EPI, EDGE, TRI>), dim3(cap * NUM_XCD), dim3(GEMM_THREADS), 0, s,
                      g.t.dev, (int)g.t.n, g.total_tiles, sc, (const int*)g.live);
   HIPCHECK(hipGetLastError());
   return SA_OK;
