@@ -407,7 +407,11 @@ int32_t sa_copy_f32(const float* src, float* dst, int64_t n, void* stream);
 /* Averaged duration (milliseconds, HIP events on `stream`) of the kernels of the named phase during
  * the most recent call that ran it: "newton_gemm", "syrk", "precondition_gemm", "grafting", "apply".
  * Timing is off unless sa_set_profiling(1) was called; switching it on (from off) forgets every recorded phase.
- * Returns a negative value if unavailable. */
+ * Returns a negative value if unavailable.
+ * Independently of the timing, SHAMPOO_AMD_ROCTX=1 in the environment brackets the same phases on the host with
+ * roctxRangePush / roctxRangePop (looked up at run time, nothing links against the marker library): the ranges a tracer
+ * shows under the Python ranges of the optimizer, as the reference's record_function ranges do
+ * (preconditioner/preconditioner_list.py:23-46). */
 int32_t sa_set_profiling(int32_t enabled);
 double sa_phase_ms(const char* phase);
 double sa_phase_flops(const char* phase); /* algorithmic flops (or bytes for HBM-bound phases) of that call */

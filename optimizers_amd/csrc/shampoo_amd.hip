@@ -3,11 +3,13 @@
 // parameter group ("plan"), the batched coupled-Newton driver, and per-phase HIP-event timing.
 
 #include <hip/hip_runtime.h>
+#include <dlfcn.h>
 
 #include <algorithm>
 #include <chrono>
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <memory>
@@ -264,11 +266,35 @@ constexpr int SYM_MAX_PREVIOUS_ITERATIONS = 14;
 constexpr int SYM_REDO_ITERATIONS = 17;  // a symmetric solve that needed more is repeated with full products
 std::map<std::string, Phase> g_phases;
 
+// Named ranges for a tracer (rocprofv3 --marker-trace): with SHAMPOO_AMD_ROCTX=1 in the environment every phase of a call
+// is bracketed on the host by roctxRangePush / roctxRangePop, the counterpart of the record_function ranges of the
+// reference (preconditioner/preconditioner_list.py:23-46).  The marker library is looked up when the first phase starts,
+// so nothing links against it and a process that does not ask for ranges never loads it.
+struct Roctx {
+  int (*push)(const char*) = nullptr;
+  int (*pop)() = nullptr;
+  Roctx() {
+    const char* want = std::getenv("SHAMPOO_AMD_ROCTX");
+    if (!want || want[0] == '\0' || want[0] == '0') return;
+    for (const char* lib : {"librocprofiler-sdk-roctx.so", "libroctx64.so"}) {
+      void* h = dlopen(lib, RTLD_NOW | RTLD_GLOBAL);
+      if (!h) continue;
+      push = reinterpret_cast<int (*)(const char*)>(dlsym(h, "roctxRangePushA"));
+      pop = reinterpret_cast<int (*)()>(dlsym(h, "roctxRangePop"));
+      if (push && pop) return;
+      push = nullptr; pop = nullptr;
+    }
+  }
+};
+const Roctx& roctx() { static const Roctx r; return r; }
+
 struct Span {
   Phase* ph = nullptr;
   hipStream_t s = nullptr;
   hipEvent_t stop = nullptr;
+  bool range = false;
   Span(const char* name, hipStream_t st, double work, int launches, bool reset) {
+    if (roctx().push) { (void)roctx().push(name); range = true; }
     if (!g_profiling) return;
     ph = &g_phases[name];
     if (reset) { ph->used = 0; ph->work = 0.0; ph->executed = 0.0; ph->launches = 0; }
@@ -286,6 +312,7 @@ struct Span {
   }
   ~Span() {
     if (ph) (void)hipEventRecord(stop, s);
+    if (range) (void)roctx().pop();
   }
 };
 
