@@ -4351,13 +4351,16 @@ static int sa_refresh_eigenbases_qr_wave(sa_plan* p, float bias_correction2, flo
         b.A = newton_buf(p, NB_X1, f); b.lda = f.dpad; b.a_vec = 1;   // Qacc^T (A_KM)
         b.B = newton_buf(p, NB_M1, f); b.ldb = f.dpad; b.b_vec = 1;
         b.C = newton_buf(p, NB_X0, f); b.ldc = f.dpad; b.M = b.N = b.K = f.d;
-        p->qr_b.add(b, false);  // B = Qacc^T Y
+        p->qr_b.add(b, true);   // B = Qacc^T Y = Qacc^T A Qacc is symmetric: upper-triangle tiles, mirrored
       }
     }
     SACHECK(p->qr_aq.commit(s));
     SACHECK(p->qr_b.commit(s));
     SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE>(p->qr_aq, unit_scalars(), s)));
-    if (also_B) SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_STORE>(p->qr_b, unit_scalars(), s)));
+    if (also_B) {
+      if (p->qr_b.aligned) SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, false, true>(p->qr_b, unit_scalars(), s)));
+      else SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, true, true>(p->qr_b, unit_scalars(), s)));
+    }
     return SA_OK;
   };
 
