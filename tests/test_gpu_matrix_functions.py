@@ -225,6 +225,7 @@ def test_qr_refresh_of_large_matrices_against_fp64(d):
     import optimizers_amd as oa
     from optimizers_amd.matrix_functions import matrix_eigendecomposition
     from oracle.shampoo_oracle import qr_refresh
+    from tests.golden_cases import assert_reordering_is_between_ties
 
     g = torch.Generator().manual_seed(d)
     a = torch.randn(d, 2 * d, generator=g, dtype=torch.float64)
@@ -236,6 +237,14 @@ def test_qr_refresh_of_large_matrices_against_fp64(d):
         eigendecomposition_config=oa.QREigendecompositionConfig(max_iterations=1))
     Qd = Q.cpu().double()
     assert (Qd.T @ Qd - torch.eye(d, dtype=torch.float64)).abs().max() < 2e-5
-    signs = torch.sign((Qd * want_q).sum(0))
-    assert rel_err(Qd * signs, want_q) < 1e-4
-    assert rel_err(L.cpu().double(), want_l) < 1e-5
+    # The refresh ends with a stable sort of the eigenvalue estimates (matrix_functions.py:848-850): two estimates that
+    # agree to fp32 rounding may come out in either order, so the columns are matched by direction first, and any that
+    # sit elsewhere than in the fp64 run must be such ties (Rayleigh quotients in float64).
+    match = (want_q.T @ Qd).abs().argmax(dim=1)
+    assert sorted(match.tolist()) == list(range(d)), "the columns are not a permutation of the oracle's"
+    moved, gap = assert_reordering_is_between_ties(match, Qd, A, f"order {d}")
+    print(f"order {d}: {moved} columns in another position than in the fp64 run, estimates {gap:.1e} apart", flush=True)
+    Qm = Qd[:, match]
+    signs = torch.sign((Qm * want_q).sum(0))
+    assert rel_err(Qm * signs, want_q) < 1e-4
+    assert rel_err(L.cpu().double()[match], want_l) < 1e-5
