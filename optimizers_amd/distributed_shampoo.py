@@ -942,7 +942,16 @@ class _NativeGroup(_AmortizedComputation):
                     "sa_precondition_eigenvalue_corrected",
                 )
             else:
-                native.check(lib.sa_precondition(self.plan, ref, stream), "sa_precondition")
+                # With grafting the search direction only enters through P / ||P|| (distributed_shampoo.py:1110-1122), which
+                # does not change when P is scaled: the product is then formed from the filtered gradient as it is
+                # stored, without its bias correction, and the GEMM's loader has no division to do per element and
+                # slab.  (The reference divides first; the results differ by fp32 rounding.)
+                if self.graft_type != native.SA_GRAFT_NONE and s.bias_correction1 != 1.0:
+                    unscaled = native.StepScalars.from_buffer_copy(s)
+                    unscaled.bias_correction1 = 1.0
+                    native.check(lib.sa_precondition(self.plan, ctypes.byref(unscaled), stream), "sa_precondition")
+                else:
+                    native.check(lib.sa_precondition(self.plan, ref, stream), "sa_precondition")
             native.check(lib.sa_apply_update(self.plan, ref, stream), "sa_apply_update")
         # drop the references so param.grad can be freed (distributed_shampoo.py:1666-1667)
         self._grads_alive = None
