@@ -4246,10 +4246,25 @@ static int qr_accumulate(sa_plan* p, const std::vector<int>& ids, hipStream_t s)
       if (in_registers) hipLaunchKernelGGL(qr_panel_rows_kernel, dim3(jobs), dim3(QR_THREADS), 0, s, R.panel.dev);
       else hipLaunchKernelGGL(qr_panel_kernel, dim3(jobs), dim3(QR_THREADS), lds_bytes, s, R.panel.dev);
       HIPCHECK(hipGetLastError());
-      SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, true>(R.upd[0], u, s)));
+      // the products over the panel's rows have 32 rows or columns of output: in 64 x 64 tiles they waste a quarter of the
+      // matrix instructions that 128 x 128 tiles spend on rows and columns nobody keeps
+      auto launch_small_tiles = [&](const GemmTable& g) -> int {
+        if (g.total_tiles_s == 0) return SA_OK;
+        const int per = (g.total_tiles_s + NUM_XCD - 1) / NUM_XCD;
+        hipLaunchKernelGGL((grouped_gemm_kernel<A_KM, B_KN, EPI_STORE, true, false, false, 1>), dim3(per * NUM_XCD), dim3(GEMM_THREADS), 0, s,
+                           g.t.dev, (int)g.t.n, g.total_tiles_s, u, (const int*)nullptr);
+        HIPCHECK(hipGetLastError());
+        return SA_OK;
+      };
+      SACHECK(launch_small_tiles(R.upd[0]));
       SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, true>(R.upd[1], u, s)));
-      SACHECK((launch_gemm<A_MK, B_KN, EPI_SUB, true>(R.upd[2], u, s)));
-      SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, true>(R.merge[0], u, s)));
+      if (R.upd[2].total_tiles_s) {
+        const int per = (R.upd[2].total_tiles_s + NUM_XCD - 1) / NUM_XCD;
+        hipLaunchKernelGGL((grouped_gemm_kernel<A_MK, B_KN, EPI_SUB, true, false, false, 1>), dim3(per * NUM_XCD), dim3(GEMM_THREADS), 0, s,
+                           R.upd[2].t.dev, (int)R.upd[2].t.n, R.upd[2].total_tiles_s, u, (const int*)nullptr);
+        HIPCHECK(hipGetLastError());
+      }
+      SACHECK(launch_small_tiles(R.merge[0]));
       SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, true>(R.merge[1], u, s)));
       SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, true>(R.merge[2], neg, s)));
     }
