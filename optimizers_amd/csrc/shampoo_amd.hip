@@ -232,6 +232,23 @@ int launch_gemm_auto(const GemmTable& g, GemmScalars sc, hipStream_t s) {
   return g.aligned ? launch_gemm<AL, BL, EPI, false>(g, sc, s) : launch_gemm<AL, BL, EPI, true>(g, sc, s);
 }
 
+// launch_gemm_auto in 64 x 64 tiles whatever the size of the launch: for products whose tiles hold little arithmetic
+// (K of 32 or 128, or outputs of 32 to 96 rows or columns), where four times the workgroups hide more latency and a
+// ragged edge wastes a smaller tile
+template <int AL, int BL, int EPI>
+int launch_gemm_small_tiles(const GemmTable& g, GemmScalars sc, hipStream_t s) {
+  if (g.total_tiles_s == 0) return SA_OK;
+  const int per = (g.total_tiles_s + NUM_XCD - 1) / NUM_XCD;
+  if (g.aligned)
+    hipLaunchKernelGGL((grouped_gemm_kernel<AL, BL, EPI, false, false, false, 1>), dim3(per * NUM_XCD), dim3(GEMM_THREADS), 0, s,
+                       g.t.dev, (int)g.t.n, g.total_tiles_s, sc, (const int*)nullptr);
+  else
+    hipLaunchKernelGGL((grouped_gemm_kernel<AL, BL, EPI, true, false, false, 1>), dim3(per * NUM_XCD), dim3(GEMM_THREADS), 0, s,
+                       g.t.dev, (int)g.t.n, g.total_tiles_s, sc, (const int*)nullptr);
+  HIPCHECK(hipGetLastError());
+  return SA_OK;
+}
+
 // launch_gemm_auto, with 64 x 64 tiles when the launch is small and every problem is whole tiles
 template <int AL, int BL, int EPI>
 int launch_gemm_auto_small(const GemmTable& g, GemmScalars sc, hipStream_t s) {
@@ -4248,23 +4265,10 @@ static int qr_accumulate(sa_plan* p, const std::vector<int>& ids, hipStream_t s)
       HIPCHECK(hipGetLastError());
       // the products over the panel's rows have 32 rows or columns of output: in 64 x 64 tiles they waste a quarter of the
       // matrix instructions that 128 x 128 tiles spend on rows and columns nobody keeps
-      auto launch_small_tiles = [&](const GemmTable& g) -> int {
-        if (g.total_tiles_s == 0) return SA_OK;
-        const int per = (g.total_tiles_s + NUM_XCD - 1) / NUM_XCD;
-        hipLaunchKernelGGL((grouped_gemm_kernel<A_KM, B_KN, EPI_STORE, true, false, false, 1>), dim3(per * NUM_XCD), dim3(GEMM_THREADS), 0, s,
-                           g.t.dev, (int)g.t.n, g.total_tiles_s, u, (const int*)nullptr);
-        HIPCHECK(hipGetLastError());
-        return SA_OK;
-      };
-      SACHECK(launch_small_tiles(R.upd[0]));
+      SACHECK((launch_gemm_small_tiles<A_KM, B_KN, EPI_STORE>(R.upd[0], u, s)));
       SACHECK((launch_gemm<A_KM, B_KN, EPI_STORE, true>(R.upd[1], u, s)));
-      if (R.upd[2].total_tiles_s) {
-        const int per = (R.upd[2].total_tiles_s + NUM_XCD - 1) / NUM_XCD;
-        hipLaunchKernelGGL((grouped_gemm_kernel<A_MK, B_KN, EPI_SUB, true, false, false, 1>), dim3(per * NUM_XCD), dim3(GEMM_THREADS), 0, s,
-                           R.upd[2].t.dev, (int)R.upd[2].t.n, R.upd[2].total_tiles_s, u, (const int*)nullptr);
-        HIPCHECK(hipGetLastError());
-      }
-      SACHECK(launch_small_tiles(R.merge[0]));
+      SACHECK((launch_gemm_small_tiles<A_MK, B_KN, EPI_SUB>(R.upd[2], u, s)));
+      SACHECK((launch_gemm_small_tiles<A_KM, B_KN, EPI_STORE>(R.merge[0], u, s)));
       SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, true>(R.merge[1], u, s)));
       SACHECK((launch_gemm<A_MK, B_KN, EPI_STORE, true>(R.merge[2], neg, s)));
     }
@@ -4302,11 +4306,11 @@ static int qr_accumulate(sa_plan* p, const std::vector<int>& ids, hipStream_t s)
     for (int k = 0; k < 6; ++k) SACHECK(G[k].commit(s));
     // full outer blocks of aligned factors take the unguarded loader
     SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_STORE>(G[0], u, s)));
-    SACHECK((launch_gemm_auto<A_KM, B_KN, EPI_STORE>(G[1], u, s)));
-    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_SUB>(G[2], u, s)));
+    SACHECK((launch_gemm_small_tiles<A_KM, B_KN, EPI_STORE>(G[1], u, s)));
+    SACHECK((launch_gemm_small_tiles<A_MK, B_KN, EPI_SUB>(G[2], u, s)));
     SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE>(G[3], u, s)));
-    SACHECK((launch_gemm_auto<A_MK, B_KN, EPI_STORE>(G[4], u, s)));
-    SACHECK((launch_gemm_auto<A_MK, B_NK, EPI_SUB>(G[5], u, s)));
+    SACHECK((launch_gemm_small_tiles<A_MK, B_KN, EPI_STORE>(G[4], u, s)));
+    SACHECK((launch_gemm_small_tiles<A_MK, B_NK, EPI_SUB>(G[5], u, s)));
   }
   return SA_OK;
 }
