@@ -568,6 +568,78 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
   bool local_nan = false;
   float* __restrict__ C = P.C;
   const long long ldc = P.ldc;
+  // Tiles above the diagonal of a symmetric product (all but 16 of 136 at order 2048) have nothing to decide per element:
+  // their epilogue is written like the main loop, with the addresses on the scalar side.  Every vector-ALU instruction
+  // here is taken from the matrix pipe of the other workgroups on the SIMD, and the general epilogue below spends 750
+  // (store) to 1900 (Newton M) of them per wavefront on 64-bit addresses and per-element predicates.
+  constexpr bool FAST_SYM = TRI && !EDGE && WB == 2 && (EPI == EPI_STORE || EPI == EPI_NEWTON_M);
+  bool stored = false;
+  if constexpr (FAST_SYM) {
+    if (tm != tn) {
+      stored = true;
+      const int ld = (int)ldc;
+      const int tile_bytes = ((BM - 1) * ld + BN) * 4;
+      const __amdgpu_buffer_rsrc_t cd = __builtin_amdgcn_make_buffer_rsrc(C + (long long)m0 * ldc + n0, 0, tile_bytes, 0x00020000);
+      float* const C2 = P.C2;
+      const __amdgpu_buffer_rsrc_t c2d = __builtin_amdgcn_make_buffer_rsrc(C2 + (long long)m0 * ldc + n0, 0, tile_bytes, 0x00020000);
+      const float mp_scale = sc.mp_scale;
+      // as computed: element e of block (i, j) is row 32 i + 8 (e / 4) + 4 h + e % 4, column 32 j + l32 of the wavefront's quadrant
+      const int vdir = ((wm * 64 + 4 * h) * ld + wn * 64 + l32) * 4;
+      unsigned worst = 0;  // largest |M| as a bit pattern: NaN above infinity above every finite value
+#pragma unroll
+      for (int i = 0; i < WB; ++i)
+#pragma unroll
+        for (int j = 0; j < WB; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int soff = ((i * 32 + 8 * (e >> 2) + (e & 3)) * ld + j * 32) * 4;
+            const float v = acc[i][j][e];
+            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), cd, vdir, soff, 0);
+            if (EPI == EPI_NEWTON_M) {
+              __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(__fmul_rn(v, mp_scale)), c2d, vdir, soff, 0);
+              worst = max(worst, __float_as_uint(v) & 0x7fffffffu);
+            }
+          }
+      // mirrored: each 32 x 32 block is turned in LDS (a private region per wavefront) and leaves as 16-byte stores
+      constexpr int TS = 36;
+      float* stage = (wave < 2) ? &As[wave & 1][0] : &Bs[wave & 1][0];
+      const int vmir = ((wn * 64 + (lane >> 3)) * ld + wm * 64 + (lane & 7) * 4) * 4;
+      float* const put = stage + l32 * TS + 4 * h;
+      const float* const get = stage + (lane >> 3) * TS + (lane & 7) * 4;
+#pragma unroll
+      for (int i = 0; i < WB; ++i)
+#pragma unroll
+        for (int j = 0; j < WB; ++j) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            *reinterpret_cast<float4*>(put + 8 * q) = make_float4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+          __builtin_amdgcn_wave_barrier();
+          asm volatile("" ::: "memory");
+#pragma unroll
+          for (int it = 0; it < 4; ++it) {
+            const float4 v = *reinterpret_cast<const float4*>(get + 8 * it * TS);
+            // The position of the four rows goes into the resource's base, not into the store's scalar offset: a
+            // 16-byte buffer store WITH a scalar offset register, followed at once by a vector-ALU instruction that
+            // writes its data registers, stored that instruction's result as the first of its four values now and then
+            // (the compiler pads this hazard only for stores without a scalar offset register, as here).
+            const long long at = (long long)((j * 32 + 8 * it) * ld + i * 32);
+            const __amdgpu_buffer_rsrc_t to = __builtin_amdgcn_make_buffer_rsrc(C + (long long)n0 * ldc + m0 + at, 0, tile_bytes, 0x00020000);
+            const vuint4 raw = {__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)};
+            __builtin_amdgcn_raw_buffer_store_b128(raw, to, vmir, 0, 0);
+            if (EPI == EPI_NEWTON_M) {
+              const __amdgpu_buffer_rsrc_t to2 = __builtin_amdgcn_make_buffer_rsrc(C2 + (long long)n0 * ldc + m0 + at, 0, tile_bytes, 0x00020000);
+              const vuint4 mp = {__float_as_uint(__fmul_rn(v.x, mp_scale)), __float_as_uint(__fmul_rn(v.y, mp_scale)),
+                                 __float_as_uint(__fmul_rn(v.z, mp_scale)), __float_as_uint(__fmul_rn(v.w, mp_scale))};
+              __builtin_amdgcn_raw_buffer_store_b128(mp, to2, vmir, 0, 0);
+            }
+          }
+          __builtin_amdgcn_wave_barrier();
+          asm volatile("" ::: "memory");
+        }
+      if (EPI == EPI_NEWTON_M) local = __uint_as_float(worst);
+    }
+  }
+  if (!stored) {
 #pragma unroll
   for (int i = 0; i < WB; ++i) {
 #pragma unroll
@@ -716,6 +788,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
       }
     }
   }
+  }  // !stored
   if (EPI == EPI_STORE_SQNORM) {
     local = wave_sum(local);
     if (lane == 0) red[wave] = local;
