@@ -639,6 +639,25 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
       if (EPI == EPI_NEWTON_M) local = __uint_as_float(worst);
     }
   }
+  // the same for plain products over whole tiles (the preconditioning pair, the rotations of the eigenvalue-corrected step)
+  constexpr bool FAST_PLAIN = !TRI && !LOWER && !EDGE && WB == 2 && (EPI == EPI_STORE || EPI == EPI_STORE_SQNORM);
+  if constexpr (FAST_PLAIN) {
+    stored = true;
+    const int ld = (int)ldc;
+    const __amdgpu_buffer_rsrc_t cd =
+        __builtin_amdgcn_make_buffer_rsrc(C + (long long)m0 * ldc + n0, 0, ((BM - 1) * ld + BN) * 4, 0x00020000);
+    const int vdir = ((wm * 64 + 4 * h) * ld + wn * 64 + l32) * 4;
+#pragma unroll
+    for (int i = 0; i < WB; ++i)
+#pragma unroll
+      for (int j = 0; j < WB; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const float v = acc[i][j][e];
+          __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), cd, vdir, ((i * 32 + 8 * (e >> 2) + (e & 3)) * ld + j * 32) * 4, 0);
+          if (EPI == EPI_STORE_SQNORM) local += v * v;
+        }
+  }
   if (!stored) {
 #pragma unroll
   for (int i = 0; i < WB; ++i) {
