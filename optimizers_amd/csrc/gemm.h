@@ -568,38 +568,66 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
   bool local_nan = false;
   float* __restrict__ C = P.C;
   const long long ldc = P.ldc;
-  // Tiles above the diagonal of a symmetric product (all but 16 of 136 at order 2048) have nothing to decide per element:
-  // their epilogue is written like the main loop, with the addresses on the scalar side.  Every vector-ALU instruction
-  // here is taken from the matrix pipe of the other workgroups on the SIMD, and the general epilogue below spends 750
-  // (store) to 1900 (Newton M) of them per wavefront on 64-bit addresses and per-element predicates.
+  // Symmetric products over whole tiles write their epilogue like the main loop, with the addresses on the scalar side:
+  // every vector-ALU instruction here is taken from the matrix pipe of the other workgroups on the SIMD, and the general
+  // epilogue below spends 750 (store) to 1900 (Newton M) of them per wavefront on 64-bit addresses and per-element
+  // predicates.  A block of 32 x 32 above the diagonal is stored as computed and, turned in LDS, as its mirror image; a
+  // block ON the diagonal (four per diagonal tile) keeps what lies on or above the diagonal and mirrors what lies strictly
+  // above it, the other elements' stores pointed past the buffer resource; blocks below the diagonal are dropped.
   constexpr bool FAST_SYM = TRI && !EDGE && WB == 2 && (EPI == EPI_STORE || EPI == EPI_NEWTON_M);
   bool stored = false;
   if constexpr (FAST_SYM) {
-    if (tm != tn) {
-      stored = true;
+    stored = true;
+    const bool diag_tile = tm == tn;
+    if (!diag_tile || wm <= wn) {
       const int ld = (int)ldc;
       const int tile_bytes = ((BM - 1) * ld + BN) * 4;
+      constexpr int NOWHERE = 0x7ffffff0;  // a byte offset past every resource: the store is dropped
       const __amdgpu_buffer_rsrc_t cd = __builtin_amdgcn_make_buffer_rsrc(C + (long long)m0 * ldc + n0, 0, tile_bytes, 0x00020000);
       float* const C2 = P.C2;
       const __amdgpu_buffer_rsrc_t c2d = __builtin_amdgcn_make_buffer_rsrc(C2 + (long long)m0 * ldc + n0, 0, tile_bytes, 0x00020000);
-      const float mp_scale = sc.mp_scale;
+      const float mp_scale = sc.mp_scale, mp_diag = sc.mp_diag;
+      const int order = P.d;
       // as computed: element e of block (i, j) is row 32 i + 8 (e / 4) + 4 h + e % 4, column 32 j + l32 of the wavefront's quadrant
       const int vdir = ((wm * 64 + 4 * h) * ld + wn * 64 + l32) * 4;
-      unsigned worst = 0;  // largest |M| as a bit pattern: NaN above infinity above every finite value
+      unsigned worst = 0;  // largest |M - I| as a bit pattern: NaN above infinity above every finite value
 #pragma unroll
       for (int i = 0; i < WB; ++i)
 #pragma unroll
-        for (int j = 0; j < WB; ++j)
+        for (int j = 0; j < WB; ++j) {
+          const bool on_diagonal = diag_tile && wm == wn && i == j;
+          if (diag_tile && wm == wn && i > j) continue;
+          if (!on_diagonal) {
 #pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            const int soff = ((i * 32 + 8 * (e >> 2) + (e & 3)) * ld + j * 32) * 4;
-            const float v = acc[i][j][e];
-            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), cd, vdir, soff, 0);
-            if (EPI == EPI_NEWTON_M) {
-              __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(__fmul_rn(v, mp_scale)), c2d, vdir, soff, 0);
-              worst = max(worst, __float_as_uint(v) & 0x7fffffffu);
+            for (int e = 0; e < 16; ++e) {
+              const int soff = ((i * 32 + 8 * (e >> 2) + (e & 3)) * ld + j * 32) * 4;
+              const float v = acc[i][j][e];
+              __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), cd, vdir, soff, 0);
+              if (EPI == EPI_NEWTON_M) {
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(__fmul_rn(v, mp_scale)), c2d, vdir, soff, 0);
+                worst = max(worst, __float_as_uint(v) & 0x7fffffffu);
+              }
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+              const int soff = ((i * 32 + 8 * (e >> 2) + (e & 3)) * ld + j * 32) * 4;
+              const int rb = 8 * (e >> 2) + (e & 3) + 4 * h;  // row inside the block; l32 is the column
+              const bool keep = rb <= l32, unit = rb == l32 && m0 + wm * 64 + i * 32 + rb < order;
+              const int voff = keep ? vdir : NOWHERE;
+              const float v = acc[i][j][e];
+              __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), cd, voff, soff, 0);
+              if (EPI == EPI_NEWTON_M) {
+                float mp = __fmul_rn(v, mp_scale);
+                if (unit) mp = __fadd_rn(mp, mp_diag);
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(mp), c2d, voff, soff, 0);
+                // the diagonal beyond the order is padding (zero, and not part of the error)
+                const float dv = unit ? v - 1.0f : ((rb == l32) ? 0.0f : v);
+                if (keep) worst = max(worst, __float_as_uint(dv) & 0x7fffffffu);
+              }
             }
           }
+        }
       // mirrored: each 32 x 32 block is turned in LDS (a private region per wavefront) and leaves as 16-byte stores
       constexpr int TS = 36;
       float* stage = (wave < 2) ? &As[wave & 1][0] : &Bs[wave & 1][0];
@@ -610,6 +638,8 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
       for (int i = 0; i < WB; ++i)
 #pragma unroll
         for (int j = 0; j < WB; ++j) {
+          const bool on_diagonal = diag_tile && wm == wn && i == j;
+          if (diag_tile && wm == wn && i > j) continue;
 #pragma unroll
           for (int q = 0; q < 4; ++q)
             *reinterpret_cast<float4*>(put + 8 * q) = make_float4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
@@ -624,13 +654,25 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
             // (the compiler pads this hazard only for stores without a scalar offset register, as here).
             const long long at = (long long)((j * 32 + 8 * it) * ld + i * 32);
             const __amdgpu_buffer_rsrc_t to = __builtin_amdgcn_make_buffer_rsrc(C + (long long)n0 * ldc + m0 + at, 0, tile_bytes, 0x00020000);
-            const vuint4 raw = {__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)};
-            __builtin_amdgcn_raw_buffer_store_b128(raw, to, vmir, 0, 0);
-            if (EPI == EPI_NEWTON_M) {
-              const __amdgpu_buffer_rsrc_t to2 = __builtin_amdgcn_make_buffer_rsrc(C2 + (long long)n0 * ldc + m0 + at, 0, tile_bytes, 0x00020000);
-              const vuint4 mp = {__float_as_uint(__fmul_rn(v.x, mp_scale)), __float_as_uint(__fmul_rn(v.y, mp_scale)),
-                                 __float_as_uint(__fmul_rn(v.z, mp_scale)), __float_as_uint(__fmul_rn(v.w, mp_scale))};
-              __builtin_amdgcn_raw_buffer_store_b128(mp, to2, vmir, 0, 0);
+            const __amdgpu_buffer_rsrc_t to2 = __builtin_amdgcn_make_buffer_rsrc(C2 + (long long)n0 * ldc + m0 + at, 0, tile_bytes, 0x00020000);
+            if (!on_diagonal) {
+              const vuint4 raw = {__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)};
+              __builtin_amdgcn_raw_buffer_store_b128(raw, to, vmir, 0, 0);
+              if (EPI == EPI_NEWTON_M) {
+                const vuint4 mp = {__float_as_uint(__fmul_rn(v.x, mp_scale)), __float_as_uint(__fmul_rn(v.y, mp_scale)),
+                                   __float_as_uint(__fmul_rn(v.z, mp_scale)), __float_as_uint(__fmul_rn(v.w, mp_scale))};
+                __builtin_amdgcn_raw_buffer_store_b128(mp, to2, vmir, 0, 0);
+              }
+            } else {
+              // this lane holds row c = lane / 8 + 8 it of the mirror image, columns r4 .. r4 + 3: those left of c are kept
+              const int c = (lane >> 3) + 8 * it, r4 = (lane & 7) * 4;
+              const float vv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+              for (int k = 0; k < 4; ++k) {
+                const int voff = (c > r4 + k) ? vmir + 4 * k : NOWHERE;
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(vv[k]), to, voff, 0, 0);
+                if (EPI == EPI_NEWTON_M) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(__fmul_rn(vv[k], mp_scale)), to2, voff, 0, 0);
+              }
             }
           }
           __builtin_amdgcn_wave_barrier();
