@@ -700,6 +700,28 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
           if (EPI == EPI_STORE_SQNORM) local += v * v;
         }
   }
+  // C -= product over whole tiles (the block-reflector updates of the QR refresh): k is 32 to 128 there, so the tile is
+  // mostly epilogue; a block's sixteen old values are all requested before the first difference is stored
+  constexpr bool FAST_SUB = EPI == EPI_SUB && !TRI && !EDGE;
+  if constexpr (FAST_SUB) {
+    stored = true;
+    const int ld = (int)ldc;
+    const __amdgpu_buffer_rsrc_t cd =
+        __builtin_amdgcn_make_buffer_rsrc(C + (long long)m0 * ldc + n0, 0, ((BM - 1) * ld + BN) * 4, 0x00020000);
+    const int vdir = ((wm * 32 * WB + 4 * h) * ld + wn * 32 * WB + l32) * 4;
+#pragma unroll
+    for (int i = 0; i < WB; ++i)
+#pragma unroll
+      for (int j = 0; j < WB; ++j) {
+        float old[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          old[e] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(cd, vdir, ((i * 32 + 8 * (e >> 2) + (e & 3)) * ld + j * 32) * 4, 0));
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(old[e] - acc[i][j][e]), cd, vdir, ((i * 32 + 8 * (e >> 2) + (e & 3)) * ld + j * 32) * 4, 0);
+      }
+  }
   if (!stored) {
 #pragma unroll
   for (int i = 0; i < WB; ++i) {
