@@ -76,7 +76,7 @@ WORKLOADS = {
 # runs, each scaled by what the counter reads for sa::copy_kernel's 1 GiB copy: 2.000 and 1.000); the
 # commands and per-kernel figures are in profiles/grouped_gemm_newton_llama3_8b_layer.md.  Keyed by
 # (workload, symmetric-product policy); None where no counter run was made.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {("llama3_8b_layer", 2): 10.2e9}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {("llama3_8b_layer", 2): 9.4e9}
 TRAFFIC_SOURCE = "profiles/grouped_gemm_newton_llama3_8b_layer.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, separate runs)"
 DOMINANT_PHASE = {"newton": "newton_gemm", "soap_qr": "precondition_gemm", "eigh": "jacobi"}
 # Deviations from the configs as literally stated, needed for the REFERENCE to run at all
