@@ -519,15 +519,26 @@ __global__ __launch_bounds__(256) void sym_pass_kernel(const SymFactor* __restri
   const float* __restrict__ dense_in = F.dense_in;
   if (MODE == SYM_COMMIT && F.select != nullptr && *F.select != 0) dense_in = F.dense_in_alt;
   const int d = F.d, dpad = F.dpad;
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 x 4
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;        // loads: 64 columns x 4 rows
+  const int qx = (threadIdx.x & 15) * 4, qy = threadIdx.x >> 4;  // stores: 16 groups of four columns x 16 rows
 
   float z = 1.0f, x0 = 0.f;
   if (MODE == SYM_NEWTON_INIT) {
-    if (threadIdx.x == 0) {
-      float ssum = 0.f;
-      for (int i = 0; i < F.n_norm_partial; ++i) ssum += F.norm_partial[i];
-      zsh = (float)(F.root + 1) / (2.0f * sqrtf(ssum));
+    // ||A||_F^2 from the per-chunk partial sums, added in their order by one thread; the workgroup fetches them together
+    // (a thread that loads and adds them one after the other holds its workgroup for the latency of every load)
+    __shared__ float part[256];
+    float ssum = 0.f;
+    for (int base = 0; base < F.n_norm_partial; base += 256) {
+      const int i = base + (int)threadIdx.x;
+      part[threadIdx.x] = i < F.n_norm_partial ? F.norm_partial[i] : 0.f;
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        const int m = min(256, F.n_norm_partial - base);
+        for (int k = 0; k < m; ++k) ssum += part[k];
+      }
+      __syncthreads();
     }
+    if (threadIdx.x == 0) zsh = (float)(F.root + 1) / (2.0f * sqrtf(ssum));
     __syncthreads();
     z = zsh;
     x0 = powf(z, 1.0f / (float)F.root);
@@ -557,34 +568,49 @@ __global__ __launch_bounds__(256) void sym_pass_kernel(const SymFactor* __restri
 
   float errmax = 0.f;
   bool errnan = false;
-  // upper placement (bi, bj) and, for off-diagonal tiles, the mirrored placement (bj, bi)
+  // upper placement (bi, bj) and, for off-diagonal tiles, the mirrored placement (bj, bi); four columns per thread,
+  // 16-byte stores (rows of the dense matrices start on 256-byte boundaries: dpad is a multiple of the tile)
   for (int pass = 0; pass < ((bi == bj) ? 1 : 2); ++pass) {
-    for (int rr = ty; rr < ST; rr += 4) {
+#pragma unroll
+    for (int rr = qy; rr < ST; rr += 16) {
       const int r = (pass == 0 ? bi : bj) * ST + rr;
-      const int c = (pass == 0 ? bj : bi) * ST + tx;
-      const float v = (pass == 0) ? tile[rr][tx] : tile[tx][rr];
+      const int c = (pass == 0 ? bj : bi) * ST + qx;
+      float v[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) v[k] = (pass == 0) ? tile[rr][qx + k] : tile[qx + k][rr];
       const long long o = (long long)r * dpad + c;
       if (MODE == SYM_UNPACK) {
-        F.dense_out[0][o] = v;
+        *reinterpret_cast<float4*>(F.dense_out[0] + o) = make_float4(v[0], v[1], v[2], v[3]);
       } else if (MODE == SYM_COMMIT) {
-        F.dense_out[0][o] = v;
-        if (pass == 0 && F.packed_out != nullptr && r < d && c < d && c >= r) F.packed_out[packed_off(r, c, d)] = v;
-      } else {
-        const float m = z * v;
-        float mp = __fmul_rn(m, mp_scale);
-        const bool diag = (r == c && r < d);
-        if (diag) mp = __fadd_rn(mp, mp_diag);
-        F.dense_out[0][o] = m;
-        F.dense_out[1][o] = mp;
-        F.dense_out[2][o] = diag ? x0 : 0.f;
-        // X is a multiple of the identity, so the first X M_p is x0 * M_p entry by entry: exactly what the product
-        // would give (every other term of the dot product is an exact zero)
-        if (F.dense_out[3] != nullptr) F.dense_out[3][o] = __fmul_rn(x0, mp);
-        if (r < d && c < d) {
-          const float dv = fabsf(m - (r == c ? 1.0f : 0.0f));
-          if (dv != dv) errnan = true;
-          errmax = fmaxf(errmax, dv);
+        *reinterpret_cast<float4*>(F.dense_out[0] + o) = make_float4(v[0], v[1], v[2], v[3]);
+        if (pass == 0 && F.packed_out != nullptr && r < d) {
+#pragma unroll
+          for (int k = 0; k < 4; ++k)
+            if (c + k < d && c + k >= r) F.packed_out[packed_off(r, c + k, d)] = v[k];
         }
+      } else {
+        float m[4], mp[4], xd[4], x1[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          m[k] = z * v[k];
+          mp[k] = __fmul_rn(m[k], mp_scale);
+          const bool diag = (r == c + k && r < d);
+          if (diag) mp[k] = __fadd_rn(mp[k], mp_diag);
+          xd[k] = diag ? x0 : 0.f;
+          // X is a multiple of the identity, so the first X M_p is x0 * M_p entry by entry: exactly what the product
+          // would give (every other term of the dot product is an exact zero)
+          x1[k] = __fmul_rn(x0, mp[k]);
+          if (r < d && c + k < d) {
+            const float dv = fabsf(m[k] - (r == c + k ? 1.0f : 0.0f));
+            if (dv != dv) errnan = true;
+            errmax = fmaxf(errmax, dv);
+          }
+        }
+        *reinterpret_cast<float4*>(F.dense_out[0] + o) = make_float4(m[0], m[1], m[2], m[3]);
+        *reinterpret_cast<float4*>(F.dense_out[1] + o) = make_float4(mp[0], mp[1], mp[2], mp[3]);
+        *reinterpret_cast<float4*>(F.dense_out[2] + o) = make_float4(xd[0], xd[1], xd[2], xd[3]);
+        if (F.dense_out[3] != nullptr)
+          *reinterpret_cast<float4*>(F.dense_out[3] + o) = make_float4(x1[0], x1[1], x1[2], x1[3]);
       }
     }
   }
