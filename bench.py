@@ -466,6 +466,30 @@ def gemm_standalone(lib, device, reps: int = 100) -> dict:
             tf = 2.0 * n**3 * batch / (ms * 1e-3) / 1e12
             rows.append({"batch": batch, "order": n, "A": label, "ms_per_launch": ms, "TFLOP/s": tf,
                          "frac_of_fp32_mfma_peak": tf / PEAK_FP32_MFMA_TFLOPS})
+        # the same launch with fewer problems: time against rounds of resident workgroups (1024 = 256 CUs x 4), which
+        # separates what a launch costs once (ramp, last round) from what it costs per round
+        sweep = []
+        tiles_per_problem = ((n + 127) // 128) ** 2
+        for part in (1, 2, 4, 8, 16, 32):
+            nb = max(1, round(part * 1024 / tiles_per_problem))
+            if nb > batch:
+                break
+            call = lambda: native.check(lib.sa_gemm_f32(a.data_ptr(), b.data_ptr(), c.data_ptr(), n, n, n, n, n, n, 1, 0,
+                                                        nb, n * n, n * n, n * n, st), "sa_gemm_f32")
+            call()
+            torch.cuda.synchronize()
+            k = max(20, int(400 / part))
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(k):
+                call()
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / k
+            rounds = nb * tiles_per_problem / 1024.0
+            sweep.append({"batch": nb, "rounds": rounds, "ms_per_launch": ms, "ms_per_round": ms / rounds,
+                          "frac_of_fp32_mfma_peak": 2.0 * n**3 * nb / (ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS})
+        rows.append({"order": n, "A": "A[k][m]", "rounds_sweep": sweep})
         del a, b, c
     return {"metric": "grouped_gemm_standalone", "unit": "TFLOP/s", "launches_per_row": reps, "rows": rows}
 
