@@ -434,7 +434,9 @@ int32_t sa_set_symmetric_newton(int32_t policy);
 /* No counterpart in the reference.  Launches of the coupled Newton loop, the factor update and the first
  * preconditioning product that hold fewer than `tiles` 128 x 128 output tiles run with 64 x 64 tiles instead (four times
  * the workgroups for a launch that cannot fill the chip); the results are bit-identical either way.  Default 256 (one
- * large tile per CU); 0 switches the small tiles off.  Process-wide. */
+ * large tile per CU); 0 switches the small tiles off.  The late iterations of a coupled Newton batch, in which the factors
+ * that the host expects to be still iterating (from their previous solve) hold fewer than 1.25 x `tiles` large tiles per
+ * product, take the small tiles too.  Process-wide. */
 int32_t sa_set_small_launch_tiles(int32_t tiles);
 /* The same choice for one plan (sa_set_symmetric_newton sets the default that plans created afterwards start with). */
 int32_t sa_plan_set_symmetric_newton(sa_plan* plan, int32_t policy);

@@ -98,7 +98,7 @@ __device__ __forceinline__ float gload1(const float* p) { return *(const __attri
 __host__ __device__ inline size_t live_work_offset(int n) { return ((size_t)n + 1 + NUM_XCD + 1 + 1) & ~(size_t)1; }
 __host__ __device__ inline size_t live_ints(int n) { return live_work_offset(n) + 2 * ((size_t)n + 1); }
 __global__ __launch_bounds__(256) void gemm_live_tiles_kernel(const GemmProblem* __restrict__ problems, int n, int triangular,
-                                                              int* __restrict__ live_begin, int cap) {
+                                                              int* __restrict__ live_begin, int cap, int small_tiles) {
   __shared__ int part[256];
   __shared__ long long wpart[256];
   __shared__ int carry;
@@ -114,7 +114,8 @@ __global__ __launch_bounds__(256) void gemm_live_tiles_kernel(const GemmProblem*
     if (i < n) {
       const GemmProblem& P = problems[i];
       const bool on = P.active == nullptr || *P.active != 0;
-      w = !on ? 0 : (triangular ? P.tiles_n * (P.tiles_n + 1) / 2 : P.tiles_m * P.tiles_n);
+      const int t_m = small_tiles ? P.tiles_m_s : P.tiles_m, t_n = small_tiles ? P.tiles_n_s : P.tiles_n;
+      w = !on ? 0 : (triangular ? t_n * (t_n + 1) / 2 : t_m * t_n);
       ww = (long long)w * max(P.K, 1);
     }
     part[threadIdx.x] = w;

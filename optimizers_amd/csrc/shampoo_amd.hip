@@ -194,9 +194,20 @@ int SMALL_LAUNCH_TILES = 256;  // launches below this many 128 x 128 tiles run a
 
 // launch_gemm over the problems whose `active` flag is set when the launch runs: a one-workgroup pass lays the live
 // tiles out first, so the skipped problems leave no holes in the walk (and no idle XCDs).
+// few_live: the caller expects so few of the problems to be active that their large tiles would not fill the chip; the
+// live tiles are then laid out and walked as 64 x 64 tiles (same bits; a wrong guess only costs the small tiles' lower rate)
 template <int AL, int BL, int EPI, bool EDGE, bool TRI>
-int launch_gemm_live(GemmTable& g, GemmScalars sc, hipStream_t s) {
+int launch_gemm_live(GemmTable& g, GemmScalars sc, hipStream_t s, bool few_live = false) {
   if (g.total_tiles == 0) return SA_OK;
+  if (few_live && g.total_tiles >= SMALL_LAUNCH_TILES && g.total_tiles_s > 0) {
+    SACHECK(g.need_live());
+    const int per = (g.total_tiles_s + NUM_XCD - 1) / NUM_XCD, cap = per + per / 4 + 1;
+    hipLaunchKernelGGL(gemm_live_tiles_kernel, dim3(1), dim3(256), 0, s, g.t.dev, (int)g.t.n, TRI ? 1 : 0, g.live, cap, 1);
+    hipLaunchKernelGGL((grouped_gemm_kernel<AL, BL, EPI, EDGE, TRI, false, 1>), dim3(cap * NUM_XCD), dim3(GEMM_THREADS), 0, s,
+                       g.t.dev, (int)g.t.n, g.total_tiles_s, sc, (const int*)g.live);
+    HIPCHECK(hipGetLastError());
+    return SA_OK;
+  }
   // a launch that fits the chip twice over at most is latency bound: the extra pass would cost more than idle XCDs
   if (g.total_tiles < SMALL_LAUNCH_TILES) {
     // too few large tiles to fill the chip: the same problems as 64 x 64 tiles (four times the workgroups)
@@ -210,7 +221,7 @@ int launch_gemm_live(GemmTable& g, GemmScalars sc, hipStream_t s) {
   SACHECK(g.need_live());
   // runs of equal work may differ in their numbers of tiles: a quarter more workgroups per XCD than an even split needs
   const int per = (g.total_tiles + NUM_XCD - 1) / NUM_XCD, cap = per + per / 4 + 1;
-  hipLaunchKernelGGL(gemm_live_tiles_kernel, dim3(1), dim3(256), 0, s, g.t.dev, (int)g.t.n, TRI ? 1 : 0, g.live, cap);
+  hipLaunchKernelGGL(gemm_live_tiles_kernel, dim3(1), dim3(256), 0, s, g.t.dev, (int)g.t.n, TRI ? 1 : 0, g.live, cap, 0);
   hipLaunchKernelGGL((grouped_gemm_kernel<AL, BL, EPI, EDGE, TRI>), dim3(cap * NUM_XCD), dim3(GEMM_THREADS), 0, s,
                      g.t.dev, (int)g.t.n, g.total_tiles, sc, (const int*)g.live);
   HIPCHECK(hipGetLastError());
@@ -1756,6 +1767,9 @@ struct NewtonRun {
   bool spans = true;  // record one timing span per iteration (off when two lanes overlap: their spans would add up twice)
   float alpha = 0.f, one_minus_alpha = 0.f;
   std::vector<char> ops;
+  // per product variant: (iterations of the factor's previous solve, its large tiles per product), and the tiles' sum
+  std::vector<std::pair<int, long long>> previous[2];
+  long long previous_tiles[2] = {0, 0};
 
   GemmTable (&nt_a())[2][2] { return lane ? p->nlane2.a : p->nt_a; }
   GemmTable (&nt_pow())[2][8] { return lane ? p->nlane2.pow : p->nt_pow; }
@@ -1823,10 +1837,17 @@ struct NewtonRun {
       q.active = p->d_active + (&f - p->factors.data());
       return q;
     };
+    for (int v = 0; v < 2; ++v) { previous[v].clear(); previous_tiles[v] = 0; }
+    const bool have_history = (int)p->newton_history.size() == (int)p->factors.size();
     for (int i = 0; i < n; ++i) {
       const Factor& f = p->factors[ids[i]];
       const bool sym = symmetric[i] != 0;
       const int v = sym ? 1 : 0;
+      {
+        const long long t = f.dpad / BM, tiles = sym ? t * (t + 1) / 2 : t * t;
+        previous[v].push_back({have_history ? p->newton_history[ids[i]] : 0, tiles});
+        previous_tiles[v] += tiles;
+      }
       // buffer that finally holds M_p^root (depends only on the chain length)
       const float* power = nullptr;
       for (int par = 0; par < 2; ++par) {
@@ -1920,17 +1941,34 @@ struct NewtonRun {
       std::unique_ptr<Span> span;
       if (spans) span.reset(new Span("newton_gemm", s, 0.0, nl, false));
       else if (g_profiling) g_phases["newton_gemm"].launches += nl;
+      // Towards the end only a few factors still iterate, and their large tiles no longer fill the chip (the hardware
+      // packs four workgroups on a CU before it takes the next one, so 400 tiles take as long as 1024).  Which factors
+      // those are is known on the device only; the host goes by the iterations every factor took in its previous solve
+      // (factors drift slowly), or, once the batch has outlived that guess, by the count of the last control pass.
+      bool few[2];
+      for (int v = 0; v < 2; ++v) {
+        long long live = 0, largest = 0;
+        for (const auto& e : previous[v]) {
+          if (e.first <= 0 || e.first > it) live += e.second;
+          largest = std::max(largest, e.second);
+        }
+        if (expected > 0 && it >= expected) live = std::max(live, (long long)n_active * largest);
+        // judged by the tiles of one product per factor, so the choice is the same for every stage of the iteration; the
+        // bound is a little above one large tile per CU (measured: with 400 to 800 live tiles of order 2048 the small
+        // tiles are the slower choice, below 320 they gain 1 % of the step on the GPT-2 parameter set)
+        few[v] = previous_tiles[v] > 0 && live > 0 && live < SMALL_LAUNCH_TILES + SMALL_LAUNCH_TILES / 4;
+      }
       // the two variants touch disjoint factors, so their launches of one stage are independent
       // symmetric variant: every operand is an exactly mirrored matrix, so A is read through its transpose (slabs
       // load and store as 16-byte rows instead of four scalar LDS stores per thread; same values, same results)
-      SACHECK((launch_gemm_live<A_KM, B_KN, EPI_STORE, false, true>(it == 0 ? nt_a0()[1] : nt_a()[1][parity], unit, s)));
-      SACHECK((launch_gemm_live<A_MK, B_KN, EPI_STORE, false, false>(it == 0 ? nt_a0()[0] : nt_a()[0][parity], unit, s)));
+      SACHECK((launch_gemm_live<A_KM, B_KN, EPI_STORE, false, true>(it == 0 ? nt_a0()[1] : nt_a()[1][parity], unit, s, few[1])));
+      SACHECK((launch_gemm_live<A_MK, B_KN, EPI_STORE, false, false>(it == 0 ? nt_a0()[0] : nt_a()[0][parity], unit, s, few[0])));
       for (int k = 0; k < 4; ++k) {
-        SACHECK((launch_gemm_live<A_KM, B_KN, EPI_STORE, false, true>(nt_pow()[1][parity * 4 + k], unit, s)));
-        SACHECK((launch_gemm_live<A_MK, B_KN, EPI_STORE, false, false>(nt_pow()[0][parity * 4 + k], unit, s)));
+        SACHECK((launch_gemm_live<A_KM, B_KN, EPI_STORE, false, true>(nt_pow()[1][parity * 4 + k], unit, s, few[1])));
+        SACHECK((launch_gemm_live<A_MK, B_KN, EPI_STORE, false, false>(nt_pow()[0][parity * 4 + k], unit, s, few[0])));
       }
-      SACHECK((launch_gemm_live<A_KM, B_KN, EPI_NEWTON_M, false, true>(nt_m()[1][parity], msc, s)));
-      SACHECK((launch_gemm_live<A_MK, B_KN, EPI_NEWTON_M, false, false>(nt_m()[0][parity], msc, s)));
+      SACHECK((launch_gemm_live<A_KM, B_KN, EPI_NEWTON_M, false, true>(nt_m()[1][parity], msc, s, few[1])));
+      SACHECK((launch_gemm_live<A_MK, B_KN, EPI_NEWTON_M, false, false>(nt_m()[0][parity], msc, s, few[0])));
       *launches_acc += nl;
     }
     parity ^= 1;

@@ -538,6 +538,46 @@ def test_small_launches_give_the_same_bits_with_either_tile_size(kind):
 
 
 @pytest.mark.gpu
+def test_late_newton_iterations_in_small_tiles_give_the_same_bits():
+    """A coupled Newton batch whose launches are large (here 32 factors of order 512: 512 large tiles per full product, 320
+    per symmetric one) ends with a few badly conditioned factors still iterating; from the
+    second solve on the host knows from the previous one which, and runs those late stages in 64 x 64 tiles.  Parameters
+    and inverse roots must equal, bit for bit, those of a run that keeps the large tiles throughout."""
+    import optimizers_amd as oa
+    from optimizers_amd import native
+
+    lib = native.load()
+
+    def run(tiles):
+        native.check(lib.sa_set_small_launch_tiles(tiles), "sa_set_small_launch_tiles")
+        g = torch.Generator().manual_seed(11)
+        ps = [torch.nn.Parameter((torch.randn(512, 512, generator=g) * 0.1).to(DEV)) for _ in range(16)]
+        # spectra from flat to steep: the Newton iteration counts of the factors spread over a wide range
+        decay = [10.0 ** (-0.05 * i * torch.linspace(0, 1, 512)) for i in range(16)]
+        o = oa.DistributedShampoo(ps, lr=0.01, betas=(0.9, 0.99), epsilon=1e-8, max_preconditioner_dim=512,
+                                  precondition_frequency=1, start_preconditioning_step=1,
+                                  preconditioner_config=oa.RootInvShampooPreconditionerConfig(
+                                      amortized_computation_config=oa.CoupledNewtonConfig()),
+                                  grafting_config=oa.AdamPreconditionerConfig(beta2=0.99, epsilon=1e-8))
+        out = []
+        for _ in range(4):
+            for p, w in zip(ps, decay):
+                p.grad = (torch.randn(512, 512, generator=g) * w[None, :] * w[:, None]).to(DEV)
+            o.step()
+            out.append([o.state[p]["block_0"]["shampoo"]["inv_factor_matrices"][j].clone() for p in ps for j in (0, 1)]
+                       + [p.detach().clone() for p in ps])
+        return out
+
+    try:
+        large, small = run(0), run(256)
+    finally:
+        native.check(lib.sa_set_small_launch_tiles(256), "sa_set_small_launch_tiles")
+    for a, b in zip(large, small):
+        for x, y in zip(a, b):
+            assert torch.equal(x, y)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("kind", ["newton", "higher_order", "eigh", "newton_f64", "eigh_f64", "soap_qr", "soap_eigh", "eigendecomposed"])
 def test_every_amortized_computation_gives_the_same_bits_in_waves(kind):
     """sa_plan_set_scratch_budget cuts the factors of an amortized computation into consecutive waves that share one
