@@ -440,7 +440,8 @@ def gemm_standalone(lib, device, reps: int = 100) -> dict:
     """Stand-alone launches of the grouped GEMM through the C ABI (sa_gemm_f32: full products, plain store): the Newton
     shapes of the Llama layer (108 x 2048^3) and of GPT-2 (400 x 768^3), operand layouts A as stored / A through its
     transpose, `reps` launches back to back timed with events on the launch stream (about 1.3 s per row: sustained
-    clocks, not a burst)."""
+    clocks, not a burst); then the same launch with 1, 2, 4 ... rounds of resident workgroups (`rounds_sweep`), which
+    shows what a launch costs once beside what it costs per round."""
     import torch
 
     from optimizers_amd import native
