@@ -723,6 +723,46 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
           __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(old[e] - acc[i][j][e]), cd, vdir, ((i * 32 + 8 * (e >> 2) + (e & 3)) * ld + j * 32) * 4, 0);
       }
   }
+  // The factor update over whole tiles: a read-modify-write of the packed upper triangle.  The general epilogue below
+  // handles one element at a time (its load, a wait for it and for the store before it, the store: 64 round trips to
+  // memory per wavefront, as long as the main loop of a 1024-deep product); here the sixteen old values of a block are
+  // requested together.  Element (r, c), c >= r, of the packed matrix of order n lives at r n - r (r + 1) / 2 + c; for
+  // row r0 + k that is k (n - r0) - k (k + 1) / 2 past row r0's, so an element's offset is one multiply-add.  The
+  // elements below the diagonal (blocks on the diagonal of a diagonal tile) are pointed past the resource.
+  constexpr bool FAST_SYRK = EPI == EPI_SYRK_EMA && TRI && !EDGE && WB == 2;
+  if constexpr (FAST_SYRK) {
+    if (N <= 16384) {  // byte offsets and the resource's extent stay below 2^31
+      stored = true;
+      const bool diag_tile = tm == tn;
+      if (!diag_tile || wm <= wn) {
+        constexpr int NOWHERE = 0x7ffffff0;
+        const int n = N;
+        const __amdgpu_buffer_rsrc_t cd = __builtin_amdgcn_make_buffer_rsrc(C, 0, n * (n + 1) / 2 * 4, 0x00020000);
+        const float alpha = sc.alpha, beta = sc.beta;
+#pragma unroll
+        for (int i = 0; i < WB; ++i)
+#pragma unroll
+          for (int j = 0; j < WB; ++j) {
+            const bool on_diagonal = diag_tile && wm == wn && i == j;
+            if (diag_tile && wm == wn && i > j) continue;
+            const int r0 = m0 + wm * 64 + i * 32 + 4 * h, c = n0 + wn * 64 + j * 32 + l32;
+            const int first = (r0 * n - r0 * (r0 + 1) / 2 + c) * 4, pitch = (n - r0) * 4;
+            int voff[16];
+            float old[16];
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+              const int k = 8 * (e >> 2) + (e & 3);
+              voff[e] = first + k * pitch - 2 * k * (k + 1);
+              if (on_diagonal && k + 4 * h > l32) voff[e] = NOWHERE;
+              old[e] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(cd, voff[e], 0, 0));
+            }
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+              __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(__builtin_fmaf(acc[i][j][e], alpha, old[e] * beta)), cd, voff[e], 0, 0);
+          }
+      }
+    }
+  }
   if (!stored) {
 #pragma unroll
   for (int i = 0; i < WB; ++i) {
