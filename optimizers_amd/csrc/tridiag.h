@@ -872,32 +872,50 @@ __global__ __launch_bounds__(256) void tdc_bisect_kernel(const TrdJob* __restric
   for (int it = 0; it < 64; ++it) {
     const double mid = 0.5 * (lo + hi);
     if (mid <= lo || mid >= hi) break;  // the interval is down to neighbouring numbers
-    // number of eigenvalues of the block below mid: negative pivots of the LDL^T factorisation of T - mid I
-    int cnt = 0;
-    double q = 1.0;
-    // first row: no coupling term
-    q = dd[s] - mid;
-    if (fabs(q) < TDC_PIVMIN) q = -TDC_PIVMIN;
-    cnt += (q < 0.0) ? 1 : 0;
-    for (int r0 = s + 1; r0 < t; r0 += TDC_PF) {
+    // Number of eigenvalues of the block below mid: sign changes in the sequence of leading principal minors of
+    // T - mid I, p_i = (d_i - mid) p_(i-1) - e_(i-1)^2 p_(i-2) with p_(-1) = 1.  The pivots of the LDL^T factorisation are
+    // the ratios p_i / p_(i-1); dividing at every row makes a chain of a reciprocal, its refinement and a product per
+    // row (250 cycles), the minors themselves one fused multiply-add.  A minor that is exactly zero counts as positive,
+    // and the one after it has the sign opposite to the one before it, so the pair still counts one change.  The pair is
+    // scaled back to magnitude one after every TDC_PF rows: a row multiplies it by at most 4 and, inside an unreduced
+    // block (|e| > 1.5e-8), by no less than 1.5e-8 on average, so TDC_PF rows stay far inside the range of a double.
+    double p2 = 1.0, p1 = dd[s] - mid;
+    unsigned neg = (unsigned)__double2hiint(p1) >> 31;
+    int cnt = (int)neg;
+    int r0 = s + 1;
+    for (; r0 + TDC_PF <= t; r0 += TDC_PF) {
       // the operands of a block of rows are read from LDS before the dependent chain of the block starts
       double a[TDC_PF], b[TDC_PF];
 #pragma unroll
       for (int j = 0; j < TDC_PF; ++j) {
-        const int r = min(r0 + j, t - 1);
-        a[j] = dd[r] - mid;
-        b[j] = e2[r - 1];
+        a[j] = dd[r0 + j] - mid;
+        b[j] = e2[r0 + j - 1];
       }
+      unsigned signs = neg;  // the signs of the minors, the newest in bit 0
 #pragma unroll
       for (int j = 0; j < TDC_PF; ++j) {
-        if (r0 + j < t) {
-          double qi = (double)__builtin_amdgcn_rcpf((float)q);
-          qi = qi * (2.0 - q * qi);
-          q = a[j] - b[j] * qi;
-          if (fabs(q) < TDC_PIVMIN) q = -TDC_PIVMIN;
-          cnt += (q < 0.0) ? 1 : 0;
-        }
+        const double p = fma(a[j], p1, -(b[j] * p2));
+        signs = __builtin_amdgcn_alignbit(signs, (unsigned)__double2hiint(p), 31);  // (signs << 1) | sign of p
+        p2 = p1;
+        p1 = p;
       }
+      static_assert(TDC_PF == 16, "the sign word below holds the previous minor and sixteen new ones");
+      cnt += __popc((signs ^ (signs >> 1)) & 0xffffu);
+      neg = signs & 1u;
+      const double m = fmax(fabs(p1), fabs(p2));
+      if (m > 0.0) {
+        const int ex = ilogb(m);
+        p1 = ldexp(p1, -ex);
+        p2 = ldexp(p2, -ex);
+      }
+    }
+    for (; r0 < t; ++r0) {  // fewer than TDC_PF rows are left
+      const double p = fma(dd[r0] - mid, p1, -(e2[r0 - 1] * p2));
+      const unsigned n = (unsigned)__double2hiint(p) >> 31;
+      cnt += (int)(n ^ neg);
+      neg = n;
+      p2 = p1;
+      p1 = p;
     }
     if (cnt > k) hi = mid; else lo = mid;
   }
