@@ -723,6 +723,57 @@ __global__ __launch_bounds__(GEMM_THREADS, 4) void grouped_gemm_kernel(
           __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(old[e] - acc[i][j][e]), cd, vdir, ((i * 32 + 8 * (e >> 2) + (e & 3)) * ld + j * 32) * 4, 0);
       }
   }
+  // The fused eigenvalue-correction epilogue over whole tiles: two state arrays are read and three written per element,
+  // with two IEEE divisions and a square root in between.  The general epilogue below handles one element at a time
+  // behind 64-bit addresses (a round trip to memory per element, each waiting for the stores of the one before it);
+  // here eight elements' old values are requested together, through buffer resources with scalar row offsets.
+  constexpr bool FAST_EC = EPI == EPI_EC_FUSED && !TRI && !LOWER && !EDGE && WB == 2;
+  if constexpr (FAST_EC) {
+    stored = true;
+    const int ld = (int)ldc;
+    const int tile_bytes = ((BM - 1) * ld + BN) * 4;
+    const long long at = (long long)m0 * ldc + n0;
+    const bool has_m = P.C2 != nullptr;
+    const __amdgpu_buffer_rsrc_t cd = __builtin_amdgcn_make_buffer_rsrc(C + at, 0, tile_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t c2d = __builtin_amdgcn_make_buffer_rsrc(has_m ? P.C2 + at : C + at, 0, has_m ? tile_bytes : 0, 0x00020000);
+    const __amdgpu_buffer_rsrc_t c3d = __builtin_amdgcn_make_buffer_rsrc(P.C3 + at, 0, tile_bytes, 0x00020000);
+    const int vdir = ((wm * 64 + 4 * h) * ld + wn * 64 + l32) * 4;
+    const float alpha = sc.alpha, beta = sc.beta, mom_w = sc.mom_w, mom_div = sc.mom_div, div = sc.div, pow_exp = sc.pow_exp, eps = sc.eps;
+#pragma unroll
+    for (int i = 0; i < WB; ++i)
+#pragma unroll
+      for (int j = 0; j < WB; ++j)
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          float sq_old[8], m_old[8];
+#pragma unroll
+          for (int q = 0; q < 8; ++q) {
+            const int e = 8 * half + q;
+            const int soff = ((i * 32 + 8 * (e >> 2) + (e & 3)) * ld + j * 32) * 4;
+            sq_old[q] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(cd, vdir, soff, 0));
+            m_old[q] = has_m ? __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(c2d, vdir, soff, 0)) : 0.f;
+          }
+#pragma unroll
+          for (int q = 0; q < 8; ++q) {
+            const int e = 8 * half + q;
+            const int soff = ((i * 32 + 8 * (e >> 2) + (e & 3)) * ld + j * 32) * 4;
+            const float v = acc[i][j][e];
+            const float sq = __fadd_rn(__fmul_rn(sq_old[q], beta), __fmul_rn(__fmul_rn(alpha, v), v));
+            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(sq), cd, vdir, soff, 0);
+            float num = v;
+            if (has_m) {
+              // torch.lerp(m, g, w): m + w (g - m) for w < 0.5, g - (g - m)(1 - w) otherwise
+              const float m_0 = m_old[q];
+              const float m_1 = mom_w < 0.5f ? m_0 + mom_w * (v - m_0) : v - (v - m_0) * (1.0f - mom_w);
+              __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(m_1), c2d, vdir, soff, 0);
+              num = m_1 / mom_div;
+            }
+            const float x = sq / div;
+            const float r = (pow_exp == 0.5f) ? sqrtf(x) : powf(x, pow_exp);
+            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(num / (r + eps)), c3d, vdir, soff, 0);
+          }
+        }
+  }
   // The factor update over whole tiles: a read-modify-write of the packed upper triangle.  The general epilogue below
   // handles one element at a time (its load, a wait for it and for the store before it, the store: 64 round trips to
   // memory per wavefront, as long as the main loop of a 1024-deep product); here the sixteen old values of a block are
